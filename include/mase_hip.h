@@ -1,0 +1,140 @@
+/*
+ * mase_hip.h - C ABI of libmase_hip.so: MXFP / minifloat quantisation and the MXFP GEMM for
+ * AMD MI355X (gfx950).
+ *
+ * The reference (DeepWok/mase-triton) has no FFI of its own: its seam is the Python "kernels"
+ * modules that the functional layer calls for GPU tensors.  Every entry point below replaces
+ * one of those module functions (cited per function, paths relative to the reference
+ * checkout) and takes what that function takes, flattened to plain pointers and sizes.
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers on the current HIP device.  The library never
+ *     allocates, frees or synchronises; work is enqueued on `stream` (a hipStream_t, NULL for
+ *     the default stream) and the call returns immediately.
+ *   - dtype codes:      0 = float32, 1 = float16, 2 = bfloat16   (MASE_F32/F16/BF16)
+ *   - round_mode codes: 0 = rn (nearest even), 1 = ru, 2 = rd, 3 = rz
+ *   - is_finite != 0: the all-ones exponent is an ordinary binade (the reference's "_fn"
+ *     presets); 0: it encodes inf/NaN.
+ *   - Element codes: uint16 for minifloat, uint8 (one code per byte, never bit-packed) for MXFP.
+ *     MXFP scales: one uint8 biased exponent per block of `block_size` consecutive elements.
+ *   - Return value: 0 on success; -1 invalid argument, -2 unsupported combination, -3 HIP
+ *     runtime error.  mase_hip_last_error() gives the message of the calling thread's last
+ *     failure.
+ *   - Inputs are never written.  Buffers must not overlap unless stated.
+ */
+#ifndef MASE_HIP_H
+#define MASE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MASE_F32 0
+#define MASE_F16 1
+#define MASE_BF16 2
+
+#define MASE_RN 0
+#define MASE_RU 1
+#define MASE_RD 2
+#define MASE_RZ 3
+
+#define MASE_OK 0
+#define MASE_ERR_INVALID (-1)
+#define MASE_ERR_UNSUPPORTED (-2)
+#define MASE_ERR_RUNTIME (-3)
+
+/* ABI version of the loaded library (bumped on any signature change). */
+int mase_hip_abi_version(void);
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* mase_hip_last_error(void);
+
+/*
+ * x[n] (x_dtype) -> codes[n] (uint16).
+ * Replaces extract_minifloat_component(x, minifloat_meta)
+ *   src/mase_triton/minifloat/kernels/cast.py:148-170, numerics of minifloat/fake.py:7-78.
+ * The reference's functional layer upcasts to float32 first (minifloat/functional/cast.py:27);
+ * here the 16-bit dtypes are read directly, which gives the same codes.
+ */
+int mase_hip_extract_minifloat(const void* x, int x_dtype, uint16_t* codes, int64_t n,
+                               int exp_bits, int frac_bits, int is_finite, int round_mode,
+                               void* stream);
+
+/*
+ * codes[n] (uint16) -> out[n] (out_dtype).
+ * Replaces compose_minifloat_component(elements, minifloat_meta, output_dtype)
+ *   src/mase_triton/minifloat/kernels/cast.py:263-288, numerics of minifloat/fake.py:81-125.
+ */
+int mase_hip_compose_minifloat(const uint16_t* codes, void* out, int out_dtype, int64_t n,
+                               int exp_bits, int frac_bits, int is_finite, void* stream);
+
+/*
+ * out[n] = compose(extract(x[n])) in one pass, codes never stored.  `out` may alias `x` when
+ * both dtypes have the same size.
+ * Replaces quantize_dequantize(tensor, minifloat_meta, output_dtype)
+ *   src/mase_triton/minifloat/functional/cast.py:72-90.
+ */
+int mase_hip_qdq_minifloat(const void* x, int x_dtype, void* out, int out_dtype, int64_t n,
+                           int exp_bits, int frac_bits, int is_finite, int round_mode,
+                           void* stream);
+
+/*
+ * x[n] -> scales[n / block_size] (uint8), elements[n] (uint8); blocks are consecutive runs of
+ * block_size elements of the flat array; n must be a multiple of block_size.
+ * Replaces extract_mxfp_components(x, mxfp_meta)
+ *   src/mase_triton/mxfp/kernels/cast.py:126-160, numerics of mxfp/fake.py:11-59.
+ * (exp_bits, frac_bits) must be one of (4,3) (5,2) (2,3) (3,2) (2,1)  (mxfp/meta.py:21-34);
+ * the scale has 8 exponent bits.
+ */
+int mase_hip_extract_mxfp(const void* x, int x_dtype, uint8_t* scales, uint8_t* elements,
+                          int64_t n, int block_size, int exp_bits, int frac_bits, int is_finite,
+                          int round_mode, void* stream);
+
+/*
+ * scales[n / block_size], elements[n] -> out[n] (out_dtype).
+ * Replaces compose_mxfp_tensor(scales, elements, mxfp_meta, output_dtype)
+ *   src/mase_triton/mxfp/kernels/cast.py:237-272, numerics of mxfp/fake.py:62-79.
+ */
+int mase_hip_compose_mxfp(const uint8_t* scales, const uint8_t* elements, void* out,
+                          int out_dtype, int64_t n, int block_size, int exp_bits, int frac_bits,
+                          int is_finite, void* stream);
+
+/*
+ * out[n] = compose(extract(x[n])) in one pass.  `out` may alias `x` when both dtypes have the
+ * same size.
+ * Replaces quantize_dequantize(tensor, block_dim, mxfp_meta, output_dtype) for a flat,
+ * block-contiguous tensor  src/mase_triton/mxfp/functional/cast.py:103-129 (and the activation
+ * half of mxfp_linear_XqWq, mxfp/functional/linear.py:50-53).
+ */
+int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int64_t n,
+                      int block_size, int exp_bits, int frac_bits, int is_finite, int round_mode,
+                      void* stream);
+
+/*
+ * y[M,N] (out_dtype) = A[M,K] * W[N,K]^T (+ bias[N]), fp32 accumulation on bf16 MFMA.
+ *
+ *   A: either dense (a_dense != NULL, dtype a_dtype, row-major [M,K], NOT yet quantised: it is
+ *      used as is), or MXFP components (a_dense == NULL; a_scales[M*K/block], a_elements[M*K],
+ *      blocks along K).
+ *   W: MXFP components w_scales[N*K/block], w_elements[N*K], blocks along K, as produced by
+ *      mase_hip_extract_mxfp on the row-major [N,K] weight.
+ *   bias: NULL or bias[N] of dtype bias_dtype, added in fp32 before the output rounding.
+ *
+ * K must be a multiple of block_size, block_size must be 32, M, N, K >= 1.
+ * Replaces the body of mxfp_linear_XqWq / mxfp_linear_XWq with backend="fused", which the
+ * reference leaves unimplemented (src/mase_triton/mxfp/functional/linear.py:31-32,63-64); the
+ * result equals the "separate" backend (compose, then torch.nn.functional.linear, :50-61) up
+ * to the summation order of the fp32 accumulation.
+ */
+int mase_hip_mxfp_gemm(const void* a_dense, int a_dtype, const uint8_t* a_scales,
+                       const uint8_t* a_elements, int a_exp_bits, int a_frac_bits,
+                       const uint8_t* w_scales, const uint8_t* w_elements, int w_exp_bits,
+                       int w_frac_bits, const void* bias, int bias_dtype, void* y, int out_dtype,
+                       int64_t M, int64_t N, int64_t K, int block_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MASE_HIP_H */

@@ -1,0 +1,528 @@
+// Bandwidth-bound cast kernels for gfx950: minifloat extract / compose / fused QDQ and MXFP
+// extract / compose / fused QDQ, plus their C-ABI entry points.
+//
+// Data layout: every tensor is a flat array in HBM.  A lane moves EPT consecutive elements per
+// step with 128-bit accesses; consecutive lanes take consecutive EPT-runs, so a wavefront reads
+// and writes whole contiguous segments.  An MXFP block of B elements is owned by B/EPT adjacent
+// lanes, which agree on the block maximum with xor-shuffles; one of them stores the scale byte.
+#include "../../include/mase_hip.h"
+#include "mase_host.h"
+
+namespace mase {
+
+constexpr int kThreads = 256;
+
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+
+// ------------------------------------------------------------------------------ vector I/O
+// EPT elements starting at element index `off` of a flat array, as fp32 bit patterns.
+template <int DT, int EPT>
+__device__ inline void load_bits(const void* base, int64_t off, uint32_t (&u)[EPT]) {
+    if (DT == F32) {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint32_t*>(base) + off);
+#pragma unroll
+        for (int v = 0; v < EPT / 4; ++v) {
+            const uint4 r = p[v];
+            u[4 * v + 0] = r.x; u[4 * v + 1] = r.y; u[4 * v + 2] = r.z; u[4 * v + 3] = r.w;
+        }
+    } else {
+        const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + off);
+#pragma unroll
+        for (int v = 0; v < EPT / 8; ++v) {
+            const uint4 r = p[v];
+            const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (DT == BF16) {
+                    u[8 * v + 2 * j] = w[j] << 16;
+                    u[8 * v + 2 * j + 1] = w[j] & 0xFFFF0000u;
+                } else {
+                    u[8 * v + 2 * j] = half_bits_to_f32_bits(w[j] & 0xFFFFu);
+                    u[8 * v + 2 * j + 1] = half_bits_to_f32_bits(w[j] >> 16);
+                }
+            }
+        }
+    }
+}
+
+template <int DT>
+__device__ inline uint32_t load_bits_scalar(const void* base, int64_t i) {
+    if (DT == F32) return static_cast<const uint32_t*>(base)[i];
+    const uint32_t h = static_cast<const uint16_t*>(base)[i];
+    return DT == BF16 ? h << 16 : half_bits_to_f32_bits(h);
+}
+
+__device__ inline uint32_t pack_bf16(float a, float b) {
+    const bf16x2 r = __builtin_convertvector(floatx2{a, b}, bf16x2);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ inline uint32_t pack_f16(float a, float b) {
+    return f32_bits_to_half_bits(f32_bits(a)) | (f32_bits_to_half_bits(f32_bits(b)) << 16);
+}
+
+template <int DT, int EPT>
+__device__ inline void store_vals(void* base, int64_t off, const float (&y)[EPT]) {
+    if (DT == F32) {
+        uint4* p = reinterpret_cast<uint4*>(static_cast<float*>(base) + off);
+#pragma unroll
+        for (int v = 0; v < EPT / 4; ++v)
+            p[v] = make_uint4(f32_bits(y[4 * v]), f32_bits(y[4 * v + 1]), f32_bits(y[4 * v + 2]), f32_bits(y[4 * v + 3]));
+    } else {
+        uint4* p = reinterpret_cast<uint4*>(static_cast<uint16_t*>(base) + off);
+#pragma unroll
+        for (int v = 0; v < EPT / 8; ++v) {
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                w[j] = DT == BF16 ? pack_bf16(y[8 * v + 2 * j], y[8 * v + 2 * j + 1])
+                                  : pack_f16(y[8 * v + 2 * j], y[8 * v + 2 * j + 1]);
+            p[v] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+}
+
+template <int DT>
+__device__ inline void store_val_scalar(void* base, int64_t i, float y) {
+    if (DT == F32) static_cast<float*>(base)[i] = y;
+    else if (DT == BF16) static_cast<uint16_t*>(base)[i] = (uint16_t)(pack_bf16(y, 0.0f) & 0xFFFFu);
+    else static_cast<uint16_t*>(base)[i] = (uint16_t)f32_bits_to_half_bits(f32_bits(y));
+}
+
+// ------------------------------------------------------------------------------ minifloat
+template <int DT_IN, class F, int UNROLL>
+__global__ __launch_bounds__(kThreads) void extract_minifloat_kernel(const void* __restrict__ x,
+                                                                      uint16_t* __restrict__ codes, int64_t n, F f) {
+    constexpr int EPT = 8;
+    const int64_t n_chunks = n / EPT;
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint32_t u[UNROLL][EPT];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) load_bits<DT_IN, EPT>(x, c * EPT, u[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) {
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                w[j] = encode_f32_bits(u[r][2 * j], f) | (encode_f32_bits(u[r][2 * j + 1], f) << 16);
+            *reinterpret_cast<uint4*>(codes + c * EPT) = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n % EPT)) {
+        const int64_t i = n_chunks * EPT + threadIdx.x;
+        codes[i] = (uint16_t)encode_f32_bits(load_bits_scalar<DT_IN>(x, i), f);
+    }
+}
+
+template <int DT_OUT, class F, int UNROLL>
+__global__ __launch_bounds__(kThreads) void compose_minifloat_kernel(const uint16_t* __restrict__ codes,
+                                                                      void* __restrict__ out, int64_t n, F f) {
+    constexpr int EPT = 8;
+    const int64_t n_chunks = n / EPT;
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint4 raw[UNROLL];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) raw[r] = *reinterpret_cast<const uint4*>(codes + c * EPT);
+    }
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) {
+            const uint32_t w[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
+            float y[EPT];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                y[2 * j] = decode_f32(w[j] & 0xFFFFu, f);
+                y[2 * j + 1] = decode_f32(w[j] >> 16, f);
+            }
+            store_vals<DT_OUT, EPT>(out, c * EPT, y);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n % EPT)) {
+        const int64_t i = n_chunks * EPT + threadIdx.x;
+        store_val_scalar<DT_OUT>(out, i, decode_f32(codes[i], f));
+    }
+}
+
+template <int DT_IN, int DT_OUT, class F, int UNROLL>
+__global__ __launch_bounds__(kThreads) void qdq_minifloat_kernel(const void* x, void* out, int64_t n, F f) {
+    constexpr int EPT = 8;
+    const int64_t n_chunks = n / EPT;
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint32_t u[UNROLL][EPT];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) load_bits<DT_IN, EPT>(x, c * EPT, u[r]);
+    }
+    // the scalar tail reads before anything is written, so that `out` may alias `x`
+    uint32_t tail_bits = 0;
+    const bool has_tail = blockIdx.x == 0 && threadIdx.x < (n % EPT);
+    if (has_tail) tail_bits = load_bits_scalar<DT_IN>(x, n_chunks * EPT + threadIdx.x);
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) {
+            float y[EPT];
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) y[j] = decode_f32(encode_f32_bits(u[r][j], f), f);
+            store_vals<DT_OUT, EPT>(out, c * EPT, y);
+        }
+    }
+    if (has_tail) store_val_scalar<DT_OUT>(out, n_chunks * EPT + threadIdx.x, decode_f32(encode_f32_bits(tail_bits, f), f));
+}
+
+// ------------------------------------------------------------------------------ MXFP
+// Largest |x| bit pattern over the `lpb` adjacent lanes that share a block.
+__device__ inline uint32_t block_max(uint32_t amax, int lpb) {
+    for (int off = 1; off < lpb; off <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)amax, off);
+        amax = o > amax ? o : amax;
+    }
+    return amax;
+}
+
+template <int DT_IN, class F, int EPT>
+__device__ inline void mxfp_encode_run(const uint32_t (&u)[EPT], int lpb, const F& f, uint32_t (&code)[EPT],
+                                       uint32_t& scale) {
+    uint32_t amax = 0;
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+        const uint32_t a = u[j] & 0x7FFFFFFFu;
+        amax = a > amax ? a : amax;
+    }
+    amax = block_max(amax, lpb);
+    const int se = shared_exponent<F, DT_IN != F32>(amax, f);
+    scale = amax < 0x00800000u ? 0u : (uint32_t)(se + 127);  // all elements flushed -> 0
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) code[j] = encode_mxfp_element(u[j], se, f);
+}
+
+// Vector path: B % EPT == 0, B / EPT a power of two <= 64.  lpb = lanes per block.
+template <int DT_IN, class F, int EPT, int UNROLL>
+__global__ __launch_bounds__(kThreads) void extract_mxfp_kernel(const void* __restrict__ x, uint8_t* __restrict__ scales,
+                                                                 uint8_t* __restrict__ elements, int64_t n, int lpb,
+                                                                 int lpb_shift, F f) {
+    const int64_t n_chunks = n / EPT;
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint32_t u[UNROLL][EPT];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) load_bits<DT_IN, EPT>(x, c * EPT, u[r]);
+        else {
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) u[r][j] = 0u;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        uint32_t code[EPT], scale;
+        mxfp_encode_run<DT_IN, F, EPT>(u[r], lpb, f, code, scale);  // all lanes take part in the shuffles
+        if (c < n_chunks) {
+            uint32_t w[EPT / 4];
+#pragma unroll
+            for (int j = 0; j < EPT / 4; ++j)
+                w[j] = code[4 * j] | (code[4 * j + 1] << 8) | (code[4 * j + 2] << 16) | (code[4 * j + 3] << 24);
+            if constexpr (EPT == 16) *reinterpret_cast<uint4*>(elements + c * EPT) = make_uint4(w[0], w[1], w[2], w[3]);
+            else *reinterpret_cast<uint2*>(elements + c * EPT) = make_uint2(w[0], w[1]);
+            if ((c & (lpb - 1)) == 0) scales[c >> lpb_shift] = (uint8_t)scale;
+        }
+    }
+}
+
+// Fallback for any block size / alignment: one lane owns one block.
+template <int DT_IN, class F>
+__global__ __launch_bounds__(kThreads) void extract_mxfp_block_kernel(const void* __restrict__ x, uint8_t* __restrict__ scales,
+                                                                       uint8_t* __restrict__ elements, int64_t n_blocks, int B,
+                                                                       F f) {
+    const int64_t b = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (b >= n_blocks) return;
+    uint32_t amax = 0;
+    for (int j = 0; j < B; ++j) {
+        const uint32_t a = load_bits_scalar<DT_IN>(x, b * B + j) & 0x7FFFFFFFu;
+        amax = a > amax ? a : amax;
+    }
+    const int se = shared_exponent<F, DT_IN != F32>(amax, f);
+    scales[b] = amax < 0x00800000u ? (uint8_t)0 : (uint8_t)(se + 127);
+    for (int j = 0; j < B; ++j) elements[b * B + j] = (uint8_t)encode_mxfp_element(load_bits_scalar<DT_IN>(x, b * B + j), se, f);
+}
+
+template <class F>
+__device__ inline float mxfp_value(uint32_t code, float scale, const F& f) {
+    return decode_f32(code, f) * scale;
+}
+
+// Vector path: B % EPT == 0 (a lane's run lies inside one block).
+template <int DT_OUT, class F, int EPT, int UNROLL>
+__global__ __launch_bounds__(kThreads) void compose_mxfp_kernel(const uint8_t* __restrict__ scales,
+                                                                 const uint8_t* __restrict__ elements, void* __restrict__ out,
+                                                                 int64_t n, int chunks_per_block, F f) {
+    const int64_t n_chunks = n / EPT;
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint32_t w[UNROLL][EPT / 4];
+    uint32_t sc[UNROLL];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) {
+            if constexpr (EPT == 16) {
+                const uint4 v = *reinterpret_cast<const uint4*>(elements + c * EPT);
+                w[r][0] = v.x; w[r][1] = v.y; w[r][2] = v.z; w[r][3] = v.w;
+            } else {
+                const uint2 v = *reinterpret_cast<const uint2*>(elements + c * EPT);
+                w[r][0] = v.x; w[r][1] = v.y;
+            }
+            sc[r] = scales[c / chunks_per_block];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) {
+            const float s = scale_f32(sc[r]);
+            float y[EPT];
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) y[j] = mxfp_value((w[r][j / 4] >> (8 * (j % 4))) & 0xFFu, s, f);
+            store_vals<DT_OUT, EPT>(out, c * EPT, y);
+        }
+    }
+}
+
+template <int DT_OUT, class F>
+__global__ __launch_bounds__(kThreads) void compose_mxfp_scalar_kernel(const uint8_t* __restrict__ scales,
+                                                                        const uint8_t* __restrict__ elements,
+                                                                        void* __restrict__ out, int64_t n, int B, F f) {
+    const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= n) return;
+    store_val_scalar<DT_OUT>(out, i, mxfp_value(elements[i], scale_f32(scales[i / B]), f));
+}
+
+template <int DT_IN, int DT_OUT, class F, int EPT, int UNROLL>
+__global__ __launch_bounds__(kThreads) void qdq_mxfp_kernel(const void* x, void* out, int64_t n, int lpb, F f) {
+    const int64_t n_chunks = n / EPT;
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint32_t u[UNROLL][EPT];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        if (c < n_chunks) load_bits<DT_IN, EPT>(x, c * EPT, u[r]);
+        else {
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) u[r][j] = 0u;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        uint32_t code[EPT], scale;
+        mxfp_encode_run<DT_IN, F, EPT>(u[r], lpb, f, code, scale);
+        if (c < n_chunks) {
+            const float s = scale_f32(scale);
+            float y[EPT];
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) y[j] = mxfp_value(code[j], s, f);
+            store_vals<DT_OUT, EPT>(out, c * EPT, y);
+        }
+    }
+}
+
+template <int DT_IN, int DT_OUT, class F>
+__global__ __launch_bounds__(kThreads) void qdq_mxfp_block_kernel(const void* x, void* out, int64_t n_blocks, int B, F f) {
+    const int64_t b = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (b >= n_blocks) return;
+    uint32_t amax = 0;
+    for (int j = 0; j < B; ++j) {
+        const uint32_t a = load_bits_scalar<DT_IN>(x, b * B + j) & 0x7FFFFFFFu;
+        amax = a > amax ? a : amax;
+    }
+    const int se = shared_exponent<F, DT_IN != F32>(amax, f);
+    const float s = scale_f32(amax < 0x00800000u ? 0u : (uint32_t)(se + 127));
+    // a lane reads and writes only its own block, element by element, so in-place use is safe
+    for (int j = 0; j < B; ++j) {
+        const uint32_t code = encode_mxfp_element(load_bits_scalar<DT_IN>(x, b * B + j), se, f);
+        store_val_scalar<DT_OUT>(out, b * B + j, mxfp_value(code, s, f));
+    }
+}
+
+// ------------------------------------------------------------------------------ launch helpers
+inline unsigned grid_for(int64_t items, int per_block) {
+    return (unsigned)((items + per_block - 1) / per_block);
+}
+
+inline bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+inline int ilog2(int v) { int s = 0; while ((1 << s) < v) ++s; return s; }
+
+}  // namespace mase
+
+using namespace mase;
+
+namespace mase {
+std::string& last_error() {
+    static thread_local std::string msg;
+    return msg;
+}
+}  // namespace mase
+
+extern "C" {
+
+int mase_hip_abi_version(void) { return 1; }
+
+const char* mase_hip_last_error(void) { return last_error().c_str(); }
+
+int mase_hip_extract_minifloat(const void* x, int x_dtype, uint16_t* codes, int64_t n, int exp_bits, int frac_bits,
+                               int is_finite, int round_mode, void* stream) {
+    if (int rc = check_minifloat_fmt(exp_bits, frac_bits, round_mode)) return rc;
+    if (int rc = check_dtype(x_dtype, "input")) return rc;
+    if (n < 0) return fail(ERR_INVALID, "n must be non-negative");
+    if (n == 0) return OK;
+    if (!x || !codes) return fail(ERR_INVALID, "null pointer");
+    if (!aligned(x, 16) || !aligned(codes, 16)) return fail(ERR_INVALID, "x and codes must be 16-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    constexpr int UNROLL = 2;
+    const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        return dispatch_dtype(x_dtype, [&](auto dt) {
+            hipLaunchKernelGGL((extract_minifloat_kernel<decltype(dt)::value, decltype(f), UNROLL>), dim3(grid), dim3(kThreads), 0, s, x,
+                               codes, n, f);
+            return check_launch("extract_minifloat");
+        });
+    });
+}
+
+int mase_hip_compose_minifloat(const uint16_t* codes, void* out, int out_dtype, int64_t n, int exp_bits, int frac_bits,
+                               int is_finite, void* stream) {
+    if (int rc = check_minifloat_fmt(exp_bits, frac_bits, RN)) return rc;
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (n < 0) return fail(ERR_INVALID, "n must be non-negative");
+    if (n == 0) return OK;
+    if (!codes || !out) return fail(ERR_INVALID, "null pointer");
+    if (!aligned(codes, 16) || !aligned(out, 16)) return fail(ERR_INVALID, "codes and out must be 16-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    constexpr int UNROLL = 2;
+    const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, RN, [&](auto f) {
+        return dispatch_dtype(out_dtype, [&](auto dt) {
+            hipLaunchKernelGGL((compose_minifloat_kernel<decltype(dt)::value, decltype(f), UNROLL>), dim3(grid), dim3(kThreads), 0, s,
+                               codes, out, n, f);
+            return check_launch("compose_minifloat");
+        });
+    });
+}
+
+int mase_hip_qdq_minifloat(const void* x, int x_dtype, void* out, int out_dtype, int64_t n, int exp_bits, int frac_bits,
+                           int is_finite, int round_mode, void* stream) {
+    if (int rc = check_minifloat_fmt(exp_bits, frac_bits, round_mode)) return rc;
+    if (int rc = check_dtype(x_dtype, "input")) return rc;
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (n < 0) return fail(ERR_INVALID, "n must be non-negative");
+    if (n == 0) return OK;
+    if (!x || !out) return fail(ERR_INVALID, "null pointer");
+    if (!aligned(x, 16) || !aligned(out, 16)) return fail(ERR_INVALID, "x and out must be 16-byte aligned");
+    if (x == out && dtype_size(x_dtype) != dtype_size(out_dtype)) return fail(ERR_INVALID, "in-place use needs equal element sizes");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    constexpr int UNROLL = 2;
+    const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        return dispatch_dtype(x_dtype, [&](auto di) {
+            return dispatch_dtype(out_dtype, [&](auto dout) {
+                hipLaunchKernelGGL((qdq_minifloat_kernel<decltype(di)::value, decltype(dout)::value, decltype(f), UNROLL>), dim3(grid),
+                                   dim3(kThreads), 0, s, x, out, n, f);
+                return check_launch("qdq_minifloat");
+            });
+        });
+    });
+}
+
+int mase_hip_extract_mxfp(const void* x, int x_dtype, uint8_t* scales, uint8_t* elements, int64_t n, int block_size,
+                          int exp_bits, int frac_bits, int is_finite, int round_mode, void* stream) {
+    if (int rc = check_mxfp_fmt(exp_bits, frac_bits, round_mode, n, block_size)) return rc;
+    if (int rc = check_dtype(x_dtype, "input")) return rc;
+    if (n == 0) return OK;
+    if (!x || !scales || !elements) return fail(ERR_INVALID, "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    constexpr int EPT = 8, UNROLL = 4;
+    const int B = block_size;
+    const bool vec = B % EPT == 0 && pow2(B / EPT) && B / EPT <= 64 && aligned(x, 16) && aligned(elements, 8);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        return dispatch_dtype(x_dtype, [&](auto dt) {
+            if (vec) {
+                const int lpb = B / EPT;
+                hipLaunchKernelGGL((extract_mxfp_kernel<decltype(dt)::value, decltype(f), EPT, UNROLL>),
+                                   dim3(grid_for(n / EPT, UNROLL * kThreads)), dim3(kThreads), 0, s, x, scales, elements, n, lpb,
+                                   ilog2(lpb), f);
+            } else {
+                hipLaunchKernelGGL((extract_mxfp_block_kernel<decltype(dt)::value, decltype(f)>), dim3(grid_for(n / B, kThreads)),
+                                   dim3(kThreads), 0, s, x, scales, elements, n / B, B, f);
+            }
+            return check_launch("extract_mxfp");
+        });
+    });
+}
+
+int mase_hip_compose_mxfp(const uint8_t* scales, const uint8_t* elements, void* out, int out_dtype, int64_t n,
+                          int block_size, int exp_bits, int frac_bits, int is_finite, void* stream) {
+    if (int rc = check_mxfp_fmt(exp_bits, frac_bits, RN, n, block_size)) return rc;
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (n == 0) return OK;
+    if (!scales || !elements || !out) return fail(ERR_INVALID, "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    constexpr int UNROLL = 2;
+    const int B = block_size;
+    const bool al = aligned(elements, 16) && aligned(out, 16);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, RN, [&](auto f) {
+        return dispatch_dtype(out_dtype, [&](auto dt) {
+            if (al && B % 16 == 0) {
+                hipLaunchKernelGGL((compose_mxfp_kernel<decltype(dt)::value, decltype(f), 16, UNROLL>),
+                                   dim3(grid_for(n / 16, UNROLL * kThreads)), dim3(kThreads), 0, s, scales, elements, out, n, B / 16,
+                                   f);
+            } else if (al && B % 8 == 0) {
+                hipLaunchKernelGGL((compose_mxfp_kernel<decltype(dt)::value, decltype(f), 8, UNROLL>),
+                                   dim3(grid_for(n / 8, UNROLL * kThreads)), dim3(kThreads), 0, s, scales, elements, out, n, B / 8, f);
+            } else {
+                hipLaunchKernelGGL((compose_mxfp_scalar_kernel<decltype(dt)::value, decltype(f)>), dim3(grid_for(n, kThreads)),
+                                   dim3(kThreads), 0, s, scales, elements, out, n, B, f);
+            }
+            return check_launch("compose_mxfp");
+        });
+    });
+}
+
+int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int64_t n, int block_size, int exp_bits,
+                      int frac_bits, int is_finite, int round_mode, void* stream) {
+    if (int rc = check_mxfp_fmt(exp_bits, frac_bits, round_mode, n, block_size)) return rc;
+    if (int rc = check_dtype(x_dtype, "input")) return rc;
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (n == 0) return OK;
+    if (!x || !out) return fail(ERR_INVALID, "null pointer");
+    if (x == out && dtype_size(x_dtype) != dtype_size(out_dtype)) return fail(ERR_INVALID, "in-place use needs equal element sizes");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    constexpr int EPT = 8, UNROLL = 4;
+    const int B = block_size;
+    const bool vec = B % EPT == 0 && pow2(B / EPT) && B / EPT <= 64 && aligned(x, 16) && aligned(out, 16);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        return dispatch_dtype(x_dtype, [&](auto di) {
+            return dispatch_dtype(out_dtype, [&](auto dout) {
+                if (vec) {
+                    hipLaunchKernelGGL((qdq_mxfp_kernel<decltype(di)::value, decltype(dout)::value, decltype(f), EPT, UNROLL>),
+                                       dim3(grid_for(n / EPT, UNROLL * kThreads)), dim3(kThreads), 0, s, x, out, n, B / EPT, f);
+                } else {
+                    hipLaunchKernelGGL((qdq_mxfp_block_kernel<decltype(di)::value, decltype(dout)::value, decltype(f)>),
+                                       dim3(grid_for(n / B, kThreads)), dim3(kThreads), 0, s, x, out, n / B, B, f);
+                }
+                return check_launch("qdq_mxfp");
+            });
+        });
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,101 @@
+"""ctypes binding of lib/libmase_hip.so (declarations: include/mase_hip.h at the repo root)."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+from .dtype import ROUND_MODE_TO_CODE, TORCH_DTYPE_TO_CODE
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libmase_hip.so")
+_lib = None
+
+_i32, _i64, _vp = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p
+
+SIGNATURES = {
+    "mase_hip_abi_version": (_i32, []),
+    "mase_hip_last_error": (ctypes.c_char_p, []),
+    "mase_hip_extract_minifloat": (_i32, [_vp, _i32, _vp, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "mase_hip_compose_minifloat": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp]),
+    "mase_hip_qdq_minifloat": (_i32, [_vp, _i32, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "mase_hip_extract_mxfp": (_i32, [_vp, _i32, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "mase_hip_compose_mxfp": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "mase_hip_qdq_mxfp": (_i32, [_vp, _i32, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "mase_hip_mxfp_gemm": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
+                                  _vp, _i32, _i64, _i64, _i64, _i32, _vp]),
+}
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library; raises if it has not been built (there is no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build it with `python mase-triton_amd/build.py` "
+                "(mase_hip has no other implementation to fall back to)")
+        lib = ctypes.CDLL(_LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+class MaseHipError(RuntimeError):
+    pass
+
+
+def check(rc: int) -> None:
+    if rc == 0:
+        return
+    msg = load().mase_hip_last_error().decode()
+    if rc == -1:
+        raise ValueError(f"mase_hip: invalid argument: {msg}")
+    if rc == -2:
+        raise NotImplementedError(f"mase_hip: unsupported: {msg}")
+    raise MaseHipError(f"mase_hip: HIP error: {msg}")
+
+
+def require_gpu(t: torch.Tensor, what: str) -> None:
+    if t.device.type != "cuda":
+        raise RuntimeError(
+            f"mase_hip: {what} is on {t.device}; this package only runs HIP kernels on a GPU "
+            "and has no CPU implementation")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return TORCH_DTYPE_TO_CODE[dtype]
+    except KeyError:
+        raise TypeError(f"mase_hip: unsupported dtype {dtype}; use float32, float16 or bfloat16") from None
+
+
+def round_code(mode: str) -> int:
+    try:
+        return ROUND_MODE_TO_CODE[mode]
+    except KeyError:
+        raise ValueError(f"Unknown rounding mode: {mode}") from None
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def dense(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned (what the vector kernels assume)."""
+    t = t.contiguous()
+    if t.data_ptr() % 16:
+        t = t.clone()
+    return t
+
+
+def as_float_input(t: torch.Tensor) -> torch.Tensor:
+    """Kernels read float32 / float16 / bfloat16; anything else is widened to float32 first,
+    as the reference's fake path does with ``.float()``."""
+    return t if t.dtype in TORCH_DTYPE_TO_CODE else t.to(torch.float32)

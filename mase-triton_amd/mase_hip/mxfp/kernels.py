@@ -1,0 +1,119 @@
+"""GPU MXFP casts and the MXFP GEMM: tensor-level wrappers over the C ABI.
+
+``extract_mxfp_components`` / ``compose_mxfp_tensor`` have the names and signatures of the
+reference's Triton wrappers (src/mase_triton/mxfp/kernels/cast.py:126-160, 237-272); results are
+bit-identical to the reference's PyTorch "fake" implementation (src/mase_triton/mxfp/fake.py).
+``quantize_dequantize`` and ``mxfp_gemm`` have no counterpart there (fused paths).
+"""
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from .. import _lib
+from .meta import MXFPMeta
+
+
+def _fmt(meta: MXFPMeta):
+    assert meta.scale_exp_bits == 8
+    return meta.element_exp_bits, meta.element_frac_bits, int(meta.element_is_finite)
+
+
+def extract_mxfp_components(x: Tensor, mxfp_meta: MXFPMeta) -> tuple[Tensor, Tensor]:
+    """1-D float tensor -> (scales uint8 [n/B, 1], elements uint8 [n/B, B])."""
+    assert x.ndim == 1
+    _lib.require_gpu(x, "input tensor")
+    x = _lib.dense(_lib.as_float_input(x))
+    n, B = x.numel(), mxfp_meta.block_size
+    assert n % B == 0
+    scales = torch.empty((n // B, 1), dtype=torch.uint8, device=x.device)
+    elements = torch.empty((n // B, B), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().mase_hip_extract_mxfp(
+            x.data_ptr(), _lib.dtype_code(x.dtype), scales.data_ptr(), elements.data_ptr(), n, B,
+            *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
+    return scales, elements
+
+
+def compose_mxfp_tensor(scales: Tensor, elements: Tensor, mxfp_meta: MXFPMeta, output_dtype: torch.dtype) -> Tensor:
+    """(scales, elements) -> flat tensor [n] of ``output_dtype``."""
+    assert scales.dtype == torch.uint8
+    assert elements.dtype == torch.uint8
+    _lib.require_gpu(elements, "elements")
+    _lib.require_gpu(scales, "scales")
+    scales, elements = _lib.dense(scales), _lib.dense(elements)
+    n, B = elements.numel(), mxfp_meta.block_size
+    assert n % B == 0 and scales.numel() == n // B
+    out = torch.empty((n,), dtype=output_dtype, device=elements.device)
+    with torch.cuda.device(elements.device):
+        _lib.check(_lib.load().mase_hip_compose_mxfp(
+            scales.data_ptr(), elements.data_ptr(), out.data_ptr(), _lib.dtype_code(output_dtype), n, B,
+            *_fmt(mxfp_meta), _lib.stream_ptr(elements.device)))
+    return out
+
+
+def quantize_dequantize(x: Tensor, mxfp_meta: MXFPMeta, output_dtype: torch.dtype) -> Tensor:
+    """compose(extract(x)) for a flat tensor in a single pass; nothing is materialised."""
+    assert x.ndim == 1
+    _lib.require_gpu(x, "input tensor")
+    x = _lib.dense(_lib.as_float_input(x))
+    n, B = x.numel(), mxfp_meta.block_size
+    assert n % B == 0
+    out = torch.empty((n,), dtype=output_dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().mase_hip_qdq_mxfp(
+            x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(output_dtype), n, B,
+            *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
+    return out
+
+
+def mxfp_gemm(
+    a: Tensor | None,
+    a_scales: Tensor | None,
+    a_elements: Tensor | None,
+    a_meta: MXFPMeta | None,
+    w_scales: Tensor,
+    w_elements: Tensor,
+    w_meta: MXFPMeta,
+    bias: Tensor | None,
+    M: int,
+    N: int,
+    K: int,
+    output_dtype: torch.dtype,
+) -> Tensor:
+    """y[M,N] = A[M,K] @ W[N,K]^T (+ bias) on bf16 MFMA with fp32 accumulation.
+
+    A is either a dense [M,K] tensor (``a``; used as is) or MXFP components blocked along K.
+    W is MXFP components of the row-major [N,K] weight, blocked along K.
+    """
+    dev = w_elements.device
+    _lib.require_gpu(w_elements, "w_elements")
+    assert w_scales.dtype == torch.uint8 and w_elements.dtype == torch.uint8
+    assert w_meta.block_size == 32 and K % 32 == 0
+    assert w_elements.numel() == N * K and w_scales.numel() == N * K // 32
+    w_scales, w_elements = _lib.dense(w_scales), _lib.dense(w_elements)
+    a_ptr = a_sc_ptr = a_el_ptr = None
+    a_dt, a_e, a_m = 0, 0, 0
+    if a is not None:
+        _lib.require_gpu(a, "activations")
+        a = _lib.dense(a)
+        assert a.numel() == M * K
+        a_ptr, a_dt = a.data_ptr(), _lib.dtype_code(a.dtype)
+    else:
+        assert a_meta is not None and a_meta.block_size == 32
+        a_scales, a_elements = _lib.dense(a_scales), _lib.dense(a_elements)
+        assert a_elements.numel() == M * K and a_scales.numel() == M * K // 32
+        a_sc_ptr, a_el_ptr = a_scales.data_ptr(), a_elements.data_ptr()
+        a_e, a_m = a_meta.element_exp_bits, a_meta.element_frac_bits
+    b_ptr, b_dt = None, 0
+    if bias is not None:
+        bias = _lib.dense(bias)
+        assert bias.numel() == N
+        b_ptr, b_dt = bias.data_ptr(), _lib.dtype_code(bias.dtype)
+    y = torch.empty((M, N), dtype=output_dtype, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.load().mase_hip_mxfp_gemm(
+            a_ptr, a_dt, a_sc_ptr, a_el_ptr, a_e, a_m, w_scales.data_ptr(), w_elements.data_ptr(),
+            w_meta.element_exp_bits, w_meta.element_frac_bits, b_ptr, b_dt, y.data_ptr(),
+            _lib.dtype_code(output_dtype), M, N, K, 32, _lib.stream_ptr(dev)))
+    return y

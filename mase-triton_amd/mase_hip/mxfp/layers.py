@@ -1,0 +1,142 @@
+"""Post-training-quantised linear layer with MXFP operands
+(API of src/mase_triton/mxfp/layers.py:11-211)."""
+from __future__ import annotations
+
+from typing import Literal
+
+import torch
+from torch import Tensor, nn
+
+from ..utils.qlayer import ChangeDtypeError
+from . import functional as MXFP_F
+from .meta import MXFPMeta, MXFPTensorMeta
+
+LayerType = Literal["XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq"]
+
+
+class MXFPLinearPTQ(nn.Module):
+    """``y = x W^T + b`` with any of x / W / b held or rounded in an MXFP format.
+
+    A quantised weight is stored as two frozen uint8 parameters, ``w_scales`` [N*K/B, 1] and
+    ``w_elements`` [N*K/B, B], blocked along in_features; likewise ``b_scales``/``b_elements``.
+    Their dtype may never change (``.to(dtype=...)`` raises ``ChangeDtypeError``); moving the
+    module between devices refreshes the device recorded in the tensor metas.  Unlike the
+    reference, ``backend="fused"`` (the default) works: it runs the dequant-fused MFMA GEMM.
+    """
+
+    in_features: int
+    out_features: int
+    _CODE_PARAMS = ("w_scales", "w_elements", "b_scales", "b_elements")
+
+    def __init__(
+        self,
+        weight: Tensor | None,
+        bias: Tensor | None,
+        x_mxfp_meta: MXFPMeta | None,
+        w_mxfp_meta: MXFPMeta | None,
+        b_mxfp_meta: MXFPMeta | None,
+        layer_type: LayerType,
+        backend: Literal["separate", "fused"] = "fused",
+        dtype: torch.dtype | None = None,
+        device: torch.device | None = None,
+        w_scales: Tensor | None = None,
+        w_elements: Tensor | None = None,
+        w_tensor_meta: MXFPTensorMeta | None = None,
+        b_scales: Tensor | None = None,
+        b_elements: Tensor | None = None,
+        b_tensor_meta: MXFPTensorMeta | None = None,
+    ):
+        super().__init__()
+        assert weight is None or weight.ndim == 2
+        assert bias is None or bias.ndim == 1
+        have_w_parts = w_scales is not None and w_elements is not None and w_tensor_meta is not None
+        have_b_parts = b_scales is not None and b_elements is not None and b_tensor_meta is not None
+        assert (weight is not None) ^ have_w_parts
+        if bias is not None and have_b_parts:
+            raise ValueError("Either bias or b_scales, b_elements, b_tensor_meta must be None, not both.")
+        if weight is None:
+            out_features, in_features = w_tensor_meta.shape
+        else:
+            out_features, in_features = weight.shape
+        assert bias is None or bias.shape[0] == out_features
+
+        self.in_features, self.out_features = in_features, out_features
+        self.x_mxfp_meta, self.w_mxfp_meta, self.b_mxfp_meta = x_mxfp_meta, w_mxfp_meta, b_mxfp_meta
+        self.layer_type = layer_type
+        self.backend = backend
+        self.dtype, self.device = dtype, device
+
+        self.weight = self.bias = None
+        self.w_scales = self.w_elements = self.w_tensor_meta = None
+        self.b_scales = self.b_elements = self.b_tensor_meta = None
+
+        if "Wq" in layer_type:
+            if w_scales is None:
+                w_scales, w_elements, w_tensor_meta = MXFP_F.extract_mxfp_components(
+                    weight, block_dim=1, mxfp_meta=w_mxfp_meta)
+            self.w_scales = nn.Parameter(w_scales, requires_grad=False)
+            self.w_elements = nn.Parameter(w_elements, requires_grad=False)
+            self.w_tensor_meta = w_tensor_meta
+        else:
+            assert weight is not None
+            self.weight = nn.Parameter(weight.to(dtype=dtype, device=device), requires_grad=False)
+
+        if "Bq" in layer_type:
+            if bias is not None or b_scales is not None:
+                if b_scales is None:
+                    b_scales, b_elements, b_tensor_meta = MXFP_F.extract_mxfp_components(
+                        bias, block_dim=0, mxfp_meta=b_mxfp_meta)
+                self.b_scales = nn.Parameter(b_scales, requires_grad=False)
+                self.b_elements = nn.Parameter(b_elements, requires_grad=False)
+                self.b_tensor_meta = b_tensor_meta
+        elif bias is not None:
+            self.bias = nn.Parameter(bias.to(dtype=dtype, device=device), requires_grad=False)
+
+    def _apply(self, fn, recurse=True):
+        before = {n: getattr(self, n).dtype for n in self._CODE_PARAMS if getattr(self, n) is not None}
+        result = super()._apply(fn, recurse)
+        for name, dt in before.items():
+            now = getattr(self, name).dtype
+            if now != dt:
+                raise ChangeDtypeError(f"Changing dtype of {name} from {dt} to {now} is not allowed.")
+        if self.w_tensor_meta is not None and self.w_scales is not None:
+            self.w_tensor_meta = self.w_tensor_meta.create(device=self.w_scales.device)
+        if self.b_tensor_meta is not None and self.b_scales is not None:
+            self.b_tensor_meta = self.b_tensor_meta.create(device=self.b_scales.device)
+        return result
+
+    @torch.no_grad()
+    def forward(self, input: Tensor) -> Tensor:
+        return MXFP_F.mxfp_linear(
+            x=input, x_meta=self.x_mxfp_meta, w=self.weight, w_scales=self.w_scales, w_elements=self.w_elements,
+            w_tensor_meta=self.w_tensor_meta, b=self.bias, b_scales=self.b_scales, b_elements=self.b_elements,
+            b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend)
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
+                f"layer_type={self.layer_type}, w_mxfp_meta={self.w_mxfp_meta}, x_mxfp_meta={self.x_mxfp_meta}, "
+                f"b_mxfp_meta={self.b_mxfp_meta}")
+
+    @classmethod
+    def from_linear(cls, layer: nn.Linear, x_mxfp_meta: MXFPMeta | None, w_mxfp_meta: MXFPMeta | None,
+                    b_mxfp_meta: MXFPMeta | None, layer_type: LayerType, backend: Literal["separate", "fused"]):
+        """Quantise a trained ``nn.Linear``."""
+        assert isinstance(layer, nn.Linear), "layer must be an instance of nn.Linear"
+        with torch.no_grad():
+            return cls(weight=layer.weight.clone(), bias=None if layer.bias is None else layer.bias.clone(),
+                       x_mxfp_meta=x_mxfp_meta, w_mxfp_meta=w_mxfp_meta, b_mxfp_meta=b_mxfp_meta,
+                       layer_type=layer_type, backend=backend)
+
+    @classmethod
+    def from_quantized(cls, w_scales: Tensor | None, w_elements: Tensor | None, w_tensor_meta: MXFPTensorMeta | None,
+                       bias: Tensor | None, b_scales: Tensor | None, b_elements: Tensor | None,
+                       b_tensor_meta: MXFPTensorMeta | None, x_mxfp_meta: MXFPMeta | None,
+                       layer_type: Literal["XWqB", "XWqBq", "XqWqB", "XqWqBq"],
+                       backend: Literal["separate", "fused"]):
+        """Re-hydrate from stored components (tensor metas are not part of ``state_dict``)."""
+        assert w_scales is not None and w_elements is not None and w_tensor_meta is not None
+        return cls(weight=None, bias=bias, x_mxfp_meta=x_mxfp_meta, w_mxfp_meta=None, b_mxfp_meta=None,
+                   layer_type=layer_type, backend=backend, dtype=getattr(torch, w_tensor_meta.dtype),
+                   device=torch.device(w_tensor_meta.device), w_scales=w_scales, w_elements=w_elements,
+                   w_tensor_meta=w_tensor_meta, b_scales=b_scales, b_elements=b_elements,
+                   b_tensor_meta=b_tensor_meta)

@@ -1,0 +1,215 @@
+"""GPU parity tests for the dequant-fused MXFP GEMM, mxfp_linear / mxfp_matmul and the PTQ
+layers.  Tolerance: relative Frobenius error <= 1e-3 against dequantize-then-matmul with fp32
+(or wider) accumulation, as stated for this path; fp32 outputs are held to 1e-5."""
+import pytest
+import torch
+
+import oracle
+from helpers import PRESETS
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+REL_FRO_TOL = 1e-3
+
+
+def rel_fro(y, y_ref):
+    y, y_ref = y.double().cpu(), y_ref.double().cpu()
+    return ((y - y_ref).norm() / y_ref.norm()).item()
+
+
+@pytest.fixture(scope="module")
+def mh():
+    import mase_hip.mxfp.functional as F
+    import mase_hip.mxfp.kernels as mxk
+    from mase_hip import _lib
+    from mase_hip.mxfp import meta
+    from mase_hip.mxfp.layers import MXFPLinearPTQ
+
+    _lib.load()
+
+    class NS:
+        pass
+
+    ns = NS()
+    ns.F, ns.mxk, ns.meta, ns.MXFPLinearPTQ = F, mxk, meta, MXFPLinearPTQ
+    return ns
+
+
+def preset(mh, tag):
+    return getattr(mh.meta, tag)
+
+
+def make_operands(M, N, K, x_tag, w_tag, seed=0):
+    """bf16 x, w on the CPU plus their checker-side quantisation."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    xe, xm = PRESETS[x_tag]
+    we, wm = PRESETS[w_tag]
+    x_dq = oracle.qdq_mxfp(x, 32, xe, xm)
+    w_sc, w_el = oracle.extract_mxfp(w, 32, we, wm)
+    w_dq = oracle.compose_mxfp(w_sc, w_el, 32, we, wm, True, torch.bfloat16).view(N, K)
+    return x, w, x_dq, w_sc, w_el, w_dq
+
+
+@pytest.mark.parametrize("MNK", [(64, 64, 64), (128, 128, 32), (200, 136, 96), (1, 1, 32), (257, 129, 160), (384, 512, 1024)])
+@pytest.mark.parametrize("x_tag,w_tag", [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP6_E3M2"),
+                                         ("MXFP8_E5M2_fn", "OCP_MXFP4_E2M1"), ("OCP_MXFP6_E2M3", "MXFP8_E5M2_fn")])
+def test_gemm_vs_checker(mh, MNK, x_tag, w_tag):
+    M, N, K = MNK
+    x, w, x_dq, w_sc, w_el, w_dq = make_operands(M, N, K, x_tag, w_tag, seed=M + N + K)
+    y_ref = oracle.matmul_nt(x_dq, w_dq)  # float64 accumulation of the exact dequantised operands
+    w_meta = preset(mh, w_tag)
+    # dense (already quantised) A
+    y32 = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), w_meta, None, M, N, K, torch.float32)
+    assert y32.shape == (M, N)
+    assert rel_fro(y32, y_ref) <= 1e-5
+    y16 = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), w_meta, None, M, N, K, torch.bfloat16)
+    assert rel_fro(y16, y_ref.to(torch.bfloat16)) <= REL_FRO_TOL
+    # MXFP A: same bf16 operands, same summation order -> identical bits
+    xe, xm = PRESETS[x_tag]
+    x_sc, x_el = oracle.extract_mxfp(x, 32, xe, xm)
+    y32b = mh.mxk.mxfp_gemm(None, x_sc.to(DEV), x_el.to(DEV), preset(mh, x_tag), w_sc.to(DEV), w_el.to(DEV), w_meta, None,
+                            M, N, K, torch.float32)
+    assert torch.equal(y32b, y32)
+
+
+def test_gemm_bias_and_dtypes(mh):
+    M, N, K = 96, 160, 128
+    x, w, x_dq, w_sc, w_el, w_dq = make_operands(M, N, K, "MXFP8_E4M3_fn", "MXFP8_E4M3_fn", seed=3)
+    w_meta = preset(mh, "MXFP8_E4M3_fn")
+    for bdt in (torch.float32, torch.bfloat16, torch.float16):
+        b = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(bdt)
+        y_ref = oracle.matmul_nt(x_dq, w_dq) + b.float()
+        for odt, tol in ((torch.float32, 1e-5), (torch.bfloat16, REL_FRO_TOL), (torch.float16, REL_FRO_TOL)):
+            y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), w_meta, b.to(DEV), M, N, K, odt)
+            assert y.dtype == odt
+            assert rel_fro(y, y_ref.to(odt)) <= tol
+
+
+def test_gemm_special_values_propagate(mh):
+    """A weight block that held an inf composes to NaN/inf (scale 255) and must poison exactly
+    the outputs of that row, as dequantize-then-matmul does."""
+    M, N, K = 64, 64, 64
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    w[5, 40] = float("inf")
+    w_sc, w_el = oracle.extract_mxfp(w, 32, 4, 3)
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), None,
+                         M, N, K, torch.float32).cpu()
+    assert y[:, 5].isnan().all()
+    keep = torch.ones(N, dtype=torch.bool)
+    keep[5] = False
+    assert y[:, keep].isfinite().all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("layer_type", ["XqWqB", "XWqB", "XqWB", "XWB", "XqWqBq"])
+@pytest.mark.parametrize("bias", [True, False])
+def test_mxfp_linear_fused_matches_separate(mh, dtype, layer_type, bias):
+    """backend="fused" against backend="separate" (compose, then the vendor GEMM), both on the GPU."""
+    M, N, K = 192, 256, 512
+    g = torch.Generator().manual_seed(7)
+    x = (torch.randn(3, M // 3, K, generator=g) * 3).to(dtype).to(DEV)
+    lin = torch.nn.Linear(K, N, bias=bias, dtype=dtype, device=DEV)
+    x_meta = preset(mh, "MXFP8_E4M3_fn") if layer_type.startswith("Xq") else None
+    w_meta = preset(mh, "OCP_MXFP6_E3M2") if "Wq" in layer_type else None
+    b_meta = preset(mh, "MXFP8_E4M3_fn") if layer_type.endswith("Bq") and bias else None
+    fused = mh.MXFPLinearPTQ.from_linear(lin, x_meta, w_meta, b_meta, layer_type, "fused")
+    separate = mh.MXFPLinearPTQ.from_linear(lin, x_meta, w_meta, b_meta, layer_type, "separate")
+    y_f, y_s = fused(x), separate(x)
+    assert y_f.shape == (3, M // 3, N) and y_f.dtype == dtype
+    assert rel_fro(y_f, y_s) <= (REL_FRO_TOL if dtype == torch.bfloat16 else 1e-5)
+
+
+def test_mxfp_linear_vs_cpu_reference_path(mh):
+    """mxfp_linear(XqWqB, fused) against the tensor-op restatement of the reference's CPU path."""
+    from oracle import torch_fake
+
+    M, N, K = 256, 384, 512
+    x, w, *_ = make_operands(M, N, K, "MXFP8_E4M3_fn", "MXFP8_E4M3_fn", seed=11)
+    w_sc, w_el, w_tm = mh.F.extract_mxfp_components(w.to(DEV), block_dim=1, mxfp_meta=preset(mh, "MXFP8_E4M3_fn"))
+    y = mh.F.mxfp_linear(x=x.to(DEV), x_meta=preset(mh, "MXFP8_E4M3_fn"), w=None, w_scales=w_sc, w_elements=w_el,
+                         w_tensor_meta=w_tm, b=None, b_scales=None, b_elements=None, b_tensor_meta=None,
+                         layer_type="XqWqB", backend="fused")
+    y_ref = torch_fake.mxfp_linear_xq_wq(x, w_sc.cpu(), w_el.cpu(), (N, K), torch.bfloat16, (4, 3), (4, 3))
+    assert y.dtype == torch.bfloat16
+    assert rel_fro(y, y_ref) <= REL_FRO_TOL
+
+
+def test_config_c4_full_size(mh):
+    """x [16384,4096] . W [14336,4096]^T, both MXFP8 E4M3.  The whole output is compared with
+    the GPU dequantize-then-matmul (fp32 accumulate, bf16 out); a sample of rows and columns
+    with float64 accumulation on the CPU."""
+    from workloads import make_c4
+
+    x, w = make_c4()
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    xd, wd = x.to(DEV), w.to(DEV)
+    w_sc, w_el, w_tm = mh.F.extract_mxfp_components(wd, block_dim=1, mxfp_meta=fmt)
+    args = dict(x=xd, x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
+                b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
+    y = mh.F.mxfp_linear(**args, backend="fused")
+    y_sep = mh.F.mxfp_linear(**args, backend="separate")
+    assert y.shape == (16384, 14336) and y.dtype == torch.bfloat16
+    num = (y.float() - y_sep.float()).square().sum().double().sqrt().item()
+    den = y_sep.float().square().sum().double().sqrt().item()
+    assert num / den <= REL_FRO_TOL
+    rows = torch.arange(0, 16384, 257)
+    cols = torch.arange(0, 14336, 113)
+    x_dq = oracle.qdq_mxfp(x[rows], 32, 4, 3)
+    w_dq = oracle.qdq_mxfp(w[cols], 32, 4, 3)
+    y_ref = oracle.matmul_nt(x_dq, w_dq).to(torch.bfloat16)
+    assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref) <= REL_FRO_TOL
+
+
+def test_config_c5_swiglu_chain(mh):
+    """down(silu(gate(x)) * up(x)) with MXFP6 E3M2 weights and MXFP8 E4M3 activations."""
+    from workloads import make_c5
+
+    x, wg, wu, wd = make_c5()
+    xfmt, wfmt = preset(mh, "MXFP8_E4M3_fn"), preset(mh, "OCP_MXFP6_E3M2")
+
+    def layers(backend):
+        out = []
+        for w in (wg, wu, wd):
+            lin = torch.nn.Linear(w.shape[1], w.shape[0], bias=False, dtype=torch.bfloat16, device=DEV)
+            lin.weight.data.copy_(w)
+            out.append(mh.MXFPLinearPTQ.from_linear(lin, xfmt, wfmt, None, "XqWqB", backend))
+        return out
+
+    def mlp(ls, inp):
+        g, u, d = ls
+        return d(torch.nn.functional.silu(g(inp)) * u(inp))
+
+    xd = x.to(DEV)
+    y = mlp(layers("fused"), xd)
+    y_sep = mlp(layers("separate"), xd)
+    assert y.shape == (4, 2048, 4096)
+    assert rel_fro(y, y_sep) <= 3 * REL_FRO_TOL  # three chained GEMMs, each within 1e-3
+
+
+@pytest.mark.parametrize("func_type", ["XW", "XqW", "XWq", "XqWq"])
+@pytest.mark.parametrize("backend", ["separate", "fused"])
+def test_mxfp_matmul(mh, func_type, backend):
+    g = torch.Generator().manual_seed(0)
+    a = (torch.randn(2, 4, 128, 1024, generator=g) * 5).to(torch.bfloat16).to(DEV)
+    b = (torch.randn(2, 4, 1024, 512, generator=g) * 3).to(torch.bfloat16).to(DEV)
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    y = mh.F.mxfp_matmul(a, b, fmt if "Xq" in func_type else None, fmt if "Wq" in func_type else None, func_type, backend)
+    y_ref = torch.matmul(a, b)
+    assert y.shape == y_ref.shape
+    ratio = ((y - y_ref).abs().mean() / y_ref.abs().mean()).item()
+    assert ratio == 0 if func_type == "XW" else ratio < 0.2  # reference test/test_mxfp_functional.py:248-252
+    # and against the checker's quantisation of the same operands
+    a_q = oracle.qdq_mxfp(a.cpu(), 32, 4, 3) if "Xq" in func_type else a.cpu()
+    if "Wq" in func_type:
+        bt = b.cpu().transpose(-1, -2).contiguous()
+        b_q = oracle.qdq_mxfp(bt, 32, 4, 3).transpose(-1, -2)
+    else:
+        b_q = b.cpu()
+    y_chk = torch.matmul(a_q.float(), b_q.float()).to(torch.bfloat16)
+    assert rel_fro(y, y_chk) <= REL_FRO_TOL
