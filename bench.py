@@ -1,0 +1,279 @@
+#!/usr/bin/env python3
+"""Benchmark of the MXFP hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--skip-hbm]
+
+One step = one mxfp_linear call on the headline shape: x [16384, 4096] bf16 ~N(0,1), W [14336, 4096]
+bf16 ~N(0,0.02) held as MXFP8 E4M3 components (block 32 along K), activations quantised to MXFP8
+E4M3 on the fly, bf16 output, fp32 accumulation: the fused QDQ kernel over x followed by the
+dequant-fused MFMA GEMM.  Inputs are resident in HBM before the timed region.  The same run also
+measures the bandwidth-bound cast kernels on their own configurations (extra "hbm_kernels" list)
+and times the reference's CPU path (tensor-op restatement under oracle/) on a bounded sample.
+
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "mase-triton_amd"), os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--skip-hbm", action="store_true", help="skip the cast-kernel bandwidth section")
+    ap.add_argument("--only-gemm-kernel", action="store_true",
+                    help="profiling aid: launch only the GEMM kernel in the timed loop")
+    return ap.parse_args()
+
+
+def event_ms(pairs):
+    return [a.elapsed_time(b) for a, b in pairs]
+
+
+def bench_linear(args, torch, MXFP_F, kernels, fmt):
+    dev = "cuda:0"
+    M, K, N = 16384, 4096, 14336
+    gen = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
+    w_sc, w_el, w_tm = MXFP_F.extract_mxfp_components(w, block_dim=1, mxfp_meta=fmt)
+    del w
+    call = dict(x=x, x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
+                b_elements=None, b_tensor_meta=None, layer_type="XqWqB", backend="fused")
+
+    def step(ev=None):
+        # same two kernels as MXFP_F.mxfp_linear(**call), split so that events can bracket the GEMM
+        a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
+        if ev is not None:
+            ev[0].record()
+        y = kernels.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt, None, M, N, K, torch.bfloat16)
+        if ev is not None:
+            ev[1].record()
+        return y
+
+    y_api = MXFP_F.mxfp_linear(**call)
+    assert torch.equal(step().view(torch.int16), y_api.view(torch.int16)), "bench step differs from mxfp_linear"
+    del y_api
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    if args.only_gemm_kernel:
+        a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            pairs[i][0].record()
+            kernels.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt, None, M, N, K, torch.bfloat16)
+            pairs[i][1].record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    else:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(pairs[i])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    gemm_ms = sum(event_ms(pairs)) / args.steps
+    flop = 2.0 * M * N * K
+    return {
+        "ms_per_step": ms_per_step,
+        "tflops_step": flop / (ms_per_step * 1e-3) / 1e12,
+        "gemm_ms": gemm_ms,
+        "tflops_gemm": flop / (gemm_ms * 1e-3) / 1e12,
+        "shape": (M, N, K),
+    }
+
+
+def time_kernel(torch, launch, n_variants, iters=50, warmup=10):
+    """Average launch duration with HIP events on the launch stream, rotating through
+    n_variants independent buffer sets so that consecutive launches do not hit the same lines."""
+    for i in range(warmup):
+        launch(i % n_variants)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for i in range(iters):
+        ev[i][0].record()
+        launch(i % n_variants)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    ms = sorted(event_ms(ev))
+    return sum(ms) / len(ms), ms[len(ms) // 2]
+
+
+def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
+    """Cast kernels on their own configurations.  Algorithmic bytes per element: MXFP extract from
+    bf16 2 + 1 + 1/32, compose to bf16 1 + 1/32 + 2, fused minifloat QDQ fp32->fp32 4 + 4."""
+    dev = "cuda:0"
+    out = []
+
+    def roof(name, workload, bytes_per_launch, avg_ms, med_ms, cached_ms):
+        gbs = bytes_per_launch / (avg_ms * 1e-3) / 1e9
+        out.append({
+            "kernel": name, "workload": workload, "bytes_per_launch": bytes_per_launch,
+            "avg_ms": round(avg_ms, 5), "median_ms": round(med_ms, 5),
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+            "cache_resident_GBps": round(bytes_per_launch / (cached_ms * 1e-3) / 1e9, 1),
+        })
+
+    def mxfp_case(tag, rows, cols, e, m, copies):
+        meta = mx_meta(e, m)
+        n = rows * cols
+        gen = torch.Generator(device=dev).manual_seed(0)
+        xs = [(torch.randn(n, generator=gen, device=dev)).to(torch.bfloat16) for _ in range(copies)]
+        comps = [mxk.extract_mxfp_components(x, meta) for x in xs]
+        ext_bytes = n * (2 + 1 + 1 / 32)
+        cmp_bytes = n * (1 + 1 / 32 + 2)
+        # pre-allocated outputs so that the timed region holds only the kernel
+        from mase_hip import _lib
+        lib = _lib.load()
+        sp = _lib.stream_ptr(torch.device(dev))
+        sc_o = [torch.empty_like(c[0]) for c in comps]
+        el_o = [torch.empty_like(c[1]) for c in comps]
+        y_o = [torch.empty_like(x) for x in xs]
+
+        def ext(i):
+            _lib.check(lib.mase_hip_extract_mxfp(xs[i].data_ptr(), 2, sc_o[i].data_ptr(), el_o[i].data_ptr(), n, 32, e, m, 1, 0, sp))
+
+        def cmp(i):
+            _lib.check(lib.mase_hip_compose_mxfp(comps[i][0].data_ptr(), comps[i][1].data_ptr(), y_o[i].data_ptr(), 2, n, 32, e, m, 1, sp))
+
+        def both(i):
+            ext(i)
+            cmp(i)
+
+        def qdq(i):
+            _lib.check(lib.mase_hip_qdq_mxfp(xs[i].data_ptr(), 2, y_o[i].data_ptr(), 2, n, 32, e, m, 1, 0, sp))
+
+        wl = f"{tag}: {rows}x{cols} bf16, E{e}M{m}, block 32"
+        for name, fn, nbytes in (("extract_mxfp", ext, ext_bytes), ("compose_mxfp", cmp, cmp_bytes),
+                                 ("extract+compose_mxfp", both, ext_bytes + cmp_bytes), ("qdq_mxfp_fused", qdq, n * 4.0)):
+            avg, med = time_kernel(torch, fn, copies)
+            cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
+            roof(name, wl, nbytes, avg, med, cavg)
+        assert torch.equal(sc_o[0], comps[0][0]) and torch.equal(el_o[0], comps[0][1])
+
+    mxfp_case("C1", 4096, 4096, 4, 3, copies=12)   # 12 x (32 + 16.5) MiB in flight > 256 MiB cache
+    mxfp_case("C3", 14336, 4096, 2, 1, copies=4)
+
+    # C2: fused minifloat QDQ on 2^24 fp32
+    n = 1 << 24
+    from mase_hip import _lib
+    lib = _lib.load()
+    sp = _lib.stream_ptr(torch.device(dev))
+    gen = torch.Generator(device=dev).manual_seed(1)
+    xs = [torch.randn(n, generator=gen, device=dev) for _ in range(6)]
+    ys = [torch.empty_like(x) for x in xs]
+    cs = [torch.empty(n, dtype=torch.uint16, device=dev) for _ in xs]
+    for e, m in ((4, 3), (5, 2)):
+        def qdq(i):
+            _lib.check(lib.mase_hip_qdq_minifloat(xs[i].data_ptr(), 0, ys[i].data_ptr(), 0, n, e, m, 1, 0, sp))
+
+        def ext(i):
+            _lib.check(lib.mase_hip_extract_minifloat(xs[i].data_ptr(), 0, cs[i].data_ptr(), n, e, m, 1, 0, sp))
+
+        def cmp(i):
+            _lib.check(lib.mase_hip_compose_minifloat(cs[i].data_ptr(), ys[i].data_ptr(), 0, n, e, m, 1, sp))
+
+        wl = f"C2: 2^24 fp32, FP8 E{e}M{m}"
+        for name, fn, nbytes in (("qdq_minifloat_fused", qdq, n * 8.0), ("extract_minifloat", ext, n * 6.0),
+                                 ("compose_minifloat", cmp, n * 6.0)):
+            avg, med = time_kernel(torch, fn, len(xs))
+            cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
+            roof(name, wl, nbytes, avg, med, cavg)
+    return out
+
+
+def cpu_baseline(torch):
+    """The reference's CPU path (dequantize everything with tensor ops, then F.linear) on a bounded
+    sample of the headline workload: 256 of the 16384 activation rows against the full weight."""
+    from oracle import torch_fake
+
+    rows, K, N = 256, 4096, 14336
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    w_sc, w_el = torch_fake.mxfp_split(w, 32, 4, 3)
+    threads = torch.get_num_threads()
+    t0 = time.perf_counter()
+    y = torch_fake.mxfp_linear_xq_wq(x, w_sc, w_el, (N, K), torch.bfloat16, (4, 3), (4, 3))
+    t1 = time.perf_counter()
+    assert y.shape == (rows, N)
+    flop = 2.0 * rows * N * K
+    return {"value": round(flop / (t1 - t0) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{rows} of 16384 activation rows x full W [14336,4096]: tensor-op restatement of the reference's "
+                      f"CPU path (quantise x, dequantise x and W, F.linear), {t1 - t0:.1f} s"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this pool has a single MI355X and the path has no "
+              "cross-GPU step; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the product has no CPU path)", file=sys.stderr)
+        sys.exit(2)
+    import mase_hip.minifloat.kernels as mfk
+    import mase_hip.mxfp.functional as MXFP_F
+    import mase_hip.mxfp.kernels as mxk
+    from mase_hip.minifloat.meta import MinifloatMeta
+    from mase_hip.mxfp.meta import MXFP8_E4M3_fn, MXFPMeta
+
+    torch.cuda.set_device(0)
+    lin = bench_linear(args, torch, MXFP_F, mxk, MXFP8_E4M3_fn)
+    M, N, K = lin["shape"]
+    result = {
+        "metric": "mxfp_linear TFLOP/s at 16384x4096x14336 (MXFP8 E4M3 x MXFP8 E4M3, block 32)",
+        "value": round(lin["tflops_step"], 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(lin["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "C4 mxfp_linear: x[16384,4096] bf16 ~N(0,1) quantised on the fly to MXFP8 E4M3, "
+                               "W[14336,4096] ~N(0,0.02) stored as MXFP8 E4M3, block 32 along K, no bias, bf16 out, "
+                               "fp32 accumulate; step = fused QDQ kernel + dequant-fused GEMM kernel",
+                   "M": M, "N": N, "K": K},
+        "roofline": {"bound": "mfma", "achieved": round(lin["tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "mxfp_gemm_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4)},
+    }
+    if not args.skip_hbm:
+        result["hbm_kernels"] = bench_hbm(
+            torch, mxk, mfk,
+            lambda e, m: MXFPMeta(32, 8, e, m, True, "rn"), lambda e, m: MinifloatMeta(e, m, True, "rn"))
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
