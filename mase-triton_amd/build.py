@@ -57,7 +57,7 @@ def build_library(force: bool = False, save_temps: bool = False, verbose: bool =
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True, cwd=OBJ)
 
-    with ThreadPoolExecutor(max_workers=min(4, len(srcs))) as ex:
+    with ThreadPoolExecutor(max_workers=min(7, len(srcs))) as ex:
         list(ex.map(compile_one, zip(srcs, objs)))
     if force or _stale(LIB, objs):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB]

@@ -1,0 +1,35 @@
+// C-ABI entry point of the MXFP GEMM; the kernels are in gemm_impl.h, instantiated per weight
+// format in gemm_w_*.hip.
+#include "gemm_impl.h"
+
+using namespace mase;
+
+extern "C" int mase_hip_mxfp_gemm(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements,
+                                  int a_exp_bits, int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements,
+                                  int w_exp_bits, int w_frac_bits, const void* bias, int bias_dtype, void* y, int out_dtype,
+                                  int64_t M, int64_t N, int64_t K, int block_size, void* stream) {
+    if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
+    if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(ERR_INVALID, "M, N, K must fit in 31 bits");
+    if (block_size != 32) return fail(ERR_UNSUPPORTED, "the GEMM supports block_size 32 only");
+    if (K % 32 != 0) return fail(ERR_INVALID, "K must be a multiple of the block size");
+    if (!w_scales || !w_elements || !y) return fail(ERR_INVALID, "null pointer");
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (bias) if (int rc = check_dtype(bias_dtype, "bias")) return rc;
+    const bool a_is_dense = a_dense != nullptr;
+    if (a_is_dense) {
+        if (a_dtype != BF16) return fail(ERR_UNSUPPORTED, "a dense A operand must be bfloat16");
+        if (!aligned(a_dense, 16)) return fail(ERR_INVALID, "A must be 16-byte aligned");
+    } else {
+        if (!a_scales || !a_elements) return fail(ERR_INVALID, "A needs either a dense pointer or scales and elements");
+        if (!aligned(a_elements, 16)) return fail(ERR_INVALID, "a_elements must be 16-byte aligned");
+    }
+    if (!aligned(w_elements, 16)) return fail(ERR_INVALID, "w_elements must be 16-byte aligned");
+    const GemmArgs g{a_dense, a_scales, a_elements, a_is_dense ? 0 : a_exp_bits, a_frac_bits, w_scales, w_elements, bias, bias_dtype,
+                     y, out_dtype, (int)M, (int)N, (int)K, static_cast<hipStream_t>(stream)};
+    if (w_exp_bits == 4 && w_frac_bits == 3) return gemm_w_e4m3(g);
+    if (w_exp_bits == 5 && w_frac_bits == 2) return gemm_w_e5m2(g);
+    if (w_exp_bits == 2 && w_frac_bits == 3) return gemm_w_e2m3(g);
+    if (w_exp_bits == 3 && w_frac_bits == 2) return gemm_w_e3m2(g);
+    if (w_exp_bits == 2 && w_frac_bits == 1) return gemm_w_e2m1(g);
+    return fail(ERR_INVALID, "MXFP element (exp_bits, frac_bits) must be one of (4,3) (5,2) (2,3) (3,2) (2,1)");
+}

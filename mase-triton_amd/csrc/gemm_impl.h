@@ -1,0 +1,519 @@
+// Dequant-fused MXFP GEMM for gfx950:  y[M,N] = A[M,K] * W[N,K]^T (+ bias), fp32 accumulation
+// on v_mfma_f32_32x32x16_bf16.
+//
+// W (and optionally A) arrive as MXFP components: one uint8 code per element, one uint8 scale
+// per 32 elements along K.  A workgroup owns a TM x TN tile of y.  Per K-step it stages a
+// TM x TK slab of A and a TN x TK slab of W in LDS as bf16; MXFP operands are composed to bf16
+// in registers on the way (code -> fp16 by field placement, -> fp32, times 2^(scale - bias'),
+// -> bf16; exact, every MXFP value has at most 4 significant bits).  LDS is double buffered:
+// while the MFMAs consume slab k, slab k+1 (already in registers) is composed and written to the
+// other buffer and the global loads of slab k+2 are in flight; one barrier per K-step.
+//
+// MFMA operand layout (wave64): lane l supplies row l%32 of the first operand / column l%32 of
+// the second and the 8 consecutive k values starting at 8*(l/32); accumulator register v of
+// lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32].  W is fed as the FIRST operand, so a lane ends
+// up with runs of 4 consecutive n for one m and can store 8 contiguous bytes of bf16 output.
+#pragma once
+#include "../../include/mase_hip.h"
+#include "mase_host.h"
+
+namespace mase {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 halfx2_t __attribute__((ext_vector_type(2)));
+
+__device__ inline uint32_t cvt_pk_bf16(float a, float b) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2_t{a, b}, bf16x2_t));
+}
+
+// ---------------------------------------------------------------------------------------------
+// In-register compose of MXFP codes to bf16.
+//
+// A code's magnitude bits, placed so that its exponent field sits in the low bits of an fp16
+// exponent field, read as fp16 give value * 2^(bias - 15) for normal AND subnormal codes (an fp16
+// subnormal has the same meaning as a minifloat subnormal) and 0 for the zero code.  The hardware
+// fp16 -> fp32 convert is exact; one fp32 multiply by 2^(15 - bias + scale - 127) finishes the
+// job with the single rounding the reference has (only when the product leaves the fp32 normal
+// range), and the fp32 -> bf16 convert is round-to-nearest-even like the reference's cast.
+// ---------------------------------------------------------------------------------------------
+template <class F>
+struct Composer {
+    float c1, c2;     // value = (fp16-read * c1) * c2 ; c2 == 1 unless the scale is extreme
+    bool two_step;
+    __device__ inline explicit Composer(uint32_t scale) {
+        const F f{};
+        const int field = (int)scale + 15 - fmt_bias(f);  // exponent field of 2^(15 - bias + scale - 127)
+        two_step = field < 1 || field > 254;
+        if (f.E() >= 5) { two_step = false; c1 = 1.0f; c2 = scale_f32(scale); }
+        else if (!two_step) { c1 = bits_f32((uint32_t)field << 23); c2 = 1.0f; }
+        else { c1 = bits_f32((uint32_t)(142 - fmt_bias(f)) << 23); c2 = scale_f32(scale); }
+    }
+    // codes in bytes (2p, 2p+1) of w -> packed fp16 pair
+    template <int P>
+    __device__ static inline uint32_t half_pair(uint32_t w) {
+        const F f{};
+        constexpr uint32_t sel = P == 0 ? 0x010C000Cu : 0x030C020Cu;
+        const uint32_t x = __builtin_amdgcn_perm(0u, w, sel);  // each 16-bit half = code << 8
+        const int E = f.E(), M = f.M();
+        const uint32_t mag_mask = (((1u << (E + M)) - 1u) << 8) * 0x00010001u;
+        uint32_t mag = x & mag_mask;
+        if (M > 2) mag >>= (M - 2);
+        if (M < 2) mag <<= (2 - M);
+        const uint32_t sgn = (x << (7 - E - M)) & 0x80008000u;
+        return mag | sgn;
+    }
+    __device__ inline uint32_t bf16_pair(uint32_t halves) const {
+        const halfx2_t h = __builtin_bit_cast(halfx2_t, halves);
+        float a = (float)h[0] * c1, b = (float)h[1] * c1;
+        if (two_step) { a *= c2; b *= c2; }
+        return cvt_pk_bf16(a, b);
+    }
+    // E = 5 fills the whole fp16 exponent field (field 31 would read as inf/NaN): decode those
+    // codes with the generic integer path instead
+    __device__ inline uint32_t bf16_pair_wide(uint32_t w, int p) const {
+        const F f{};
+        const float a = decode_f32((w >> (16 * p)) & 0xFFu, f) * c2, b = decode_f32((w >> (16 * p + 8)) & 0xFFu, f) * c2;
+        return cvt_pk_bf16(a, b);
+    }
+    // 16 codes (one 128-bit word) of one block -> 16 bf16 (two 128-bit words)
+    __device__ inline void run16(const uint4& codes, uint4& lo, uint4& hi) const {
+        const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
+        uint32_t o[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (F{}.E() >= 5) {
+                o[2 * j] = bf16_pair_wide(w[j], 0);
+                o[2 * j + 1] = bf16_pair_wide(w[j], 1);
+            } else {
+                o[2 * j] = bf16_pair(half_pair<0>(w[j]));
+                o[2 * j + 1] = bf16_pair(half_pair<1>(w[j]));
+            }
+        }
+        lo = make_uint4(o[0], o[1], o[2], o[3]);
+        hi = make_uint4(o[4], o[5], o[6], o[7]);
+    }
+};
+
+__device__ inline float load_bias(const void* bias, int bias_dtype, int col) {
+    if (bias_dtype == F32) return static_cast<const float*>(bias)[col];
+    const uint32_t h = static_cast<const uint16_t*>(bias)[col];
+    return bits_f32(bias_dtype == BF16 ? h << 16 : half_bits_to_f32_bits(h));
+}
+
+template <int DT_OUT>
+__device__ inline void store_out(void* y, int64_t o, float r) {
+    if (DT_OUT == F32) static_cast<float*>(y)[o] = r;
+    else if (DT_OUT == BF16) static_cast<uint16_t*>(y)[o] = (uint16_t)(cvt_pk_bf16(r, 0.0f) & 0xFFFFu);
+    else static_cast<uint16_t*>(y)[o] = (uint16_t)f32_bits_to_half_bits(f32_bits(r));
+}
+
+// 4 consecutive outputs of one row, starting at a column that is a multiple of 4
+template <int DT_OUT>
+__device__ inline void store_out4(void* y, int64_t o, const float (&r)[4], bool vec_ok, int valid) {
+    if (vec_ok && valid == 4) {
+        if (DT_OUT == F32) *reinterpret_cast<float4*>(static_cast<float*>(y) + o) = make_float4(r[0], r[1], r[2], r[3]);
+        else if (DT_OUT == BF16)
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + o) = make_uint2(cvt_pk_bf16(r[0], r[1]), cvt_pk_bf16(r[2], r[3]));
+        else
+            *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + o) =
+                make_uint2(f32_bits_to_half_bits(f32_bits(r[0])) | (f32_bits_to_half_bits(f32_bits(r[1])) << 16),
+                           f32_bits_to_half_bits(f32_bits(r[2])) | (f32_bits_to_half_bits(f32_bits(r[3])) << 16));
+    } else {
+        for (int t = 0; t < valid; ++t) store_out<DT_OUT>(y, o + t, r[t]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Main kernel: 256 x 256 x 64 tiles, 4 waves (2 x 2), each wave 128 x 128 = 4 x 4 MFMA tiles.
+// ---------------------------------------------------------------------------------------------
+constexpr int TM = 256, TN = 256, TK = 64;
+constexpr int kGemmThreads = 256;
+constexpr int ROW_BYTES = TK * 2 + 16;  // 144: rows 16 B apart modulo 256 -> conflict-free 128-bit reads
+constexpr int SLAB_BYTES = TM * ROW_BYTES;  // one operand, one buffer (TM == TN)
+
+// A_MODE: 0 = dense bf16 A, 1 = MXFP A (format FA).  W is always MXFP (format FW).
+template <int A_MODE, class FA, class FW, int DT_OUT, bool GUARD_K>
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_kernel(
+    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ a_elements,
+    const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements, const void* __restrict__ bias,
+    int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t* const lds_a = lds;                    // [2][TM][ROW_BYTES]
+    uint8_t* const lds_w = lds + 2 * SLAB_BYTES;   // [2][TN][ROW_BYTES]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+
+    // Tile order: workgroup ids go round-robin over the 8 XCDs (each with its own L2), so XCD x
+    // takes the contiguous band of tile rows [x * band, (x+1) * band); inside the band ids walk
+    // the N direction fastest in groups of 8 columns so that concurrent tiles share A and W slabs.
+    int tile_m, tile_n;
+    {
+        const int id = blockIdx.x, n_tiles = tiles_m * tiles_n;
+        const int xcd = id & 7, local = id >> 3;
+        const int per_xcd = (n_tiles + 7) >> 3;
+        int linear = xcd * per_xcd + local;
+        if (per_xcd * 8 != n_tiles) linear = id;  // irregular tile counts: plain order
+        tile_m = linear / tiles_n;
+        tile_n = linear - tile_m * tiles_n;
+        if (tile_m >= tiles_m) return;
+    }
+    const int m0 = tile_m * TM, n0 = tile_n * TN;
+    const int kblocks = K / 32;
+    const int ksteps = (K + TK - 1) / TK;  // K % 32 == 0; a last half step is zero-filled
+
+    // ---- global -> register staging assignment, in 4 parts (one per MFMA phase of a K-step)
+    // dense A: 8 lanes cover one 128-byte row slab; load j (0..7) takes row j*32 + tid/8; part p owns j = 2p, 2p+1
+    // MXFP operands: 4 lanes cover one 64-code row slab; load j (0..3) takes row j*64 + tid/4; part p owns j = p
+    const int a_chunk = tid & 7, a_row0 = tid >> 3;
+    const int c_chunk = tid & 3, c_row0 = tid >> 2;
+    const int last_step = ksteps - 1;
+
+    uint4 ra[A_MODE == 0 ? 8 : 4];
+    uint4 rw[4];
+    uint32_t sa[4], sw[4];
+
+    // Rows past the matrix edge are clamped to the last row: they only feed outputs that are never
+    // stored.  Offsets are 32-bit (the host checks the operand sizes) and constant over the K loop;
+    // the slab's k0 is folded into a uniform base pointer.
+    uint32_t a_off[A_MODE == 0 ? 8 : 4], as_off[4], w_off[4], ws_off[4];
+#pragma unroll
+    for (int j = 0; j < (A_MODE == 0 ? 8 : 4); ++j) {
+        if (A_MODE == 0) {
+            const int row = min(m0 + j * 32 + a_row0, M - 1);
+            a_off[j] = ((uint32_t)row * (uint32_t)K + a_chunk * 8) * 2u;
+        } else {
+            const int row = min(m0 + j * 64 + c_row0, M - 1);
+            a_off[j] = (uint32_t)row * (uint32_t)K + c_chunk * 16;
+            as_off[j] = (uint32_t)row * (uint32_t)kblocks + (c_chunk >> 1);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = min(n0 + j * 64 + c_row0, N - 1);
+        w_off[j] = (uint32_t)row * (uint32_t)K + c_chunk * 16;
+        ws_off[j] = (uint32_t)row * (uint32_t)kblocks + (c_chunk >> 1);
+    }
+    const uint8_t* const a_bytes = A_MODE == 0 ? reinterpret_cast<const uint8_t*>(a_dense) : a_elements;
+
+    auto fetch_part = [&](int p, int kt) {
+        const int ktc = kt < last_step ? kt : last_step;  // past the end: reload the last slab (never used)
+        const bool k_ok = !GUARD_K || ktc * TK + c_chunk * 16 < K;  // only a trailing half slab can fail
+        if (A_MODE == 0) {
+            const uint8_t* const base = a_bytes + (size_t)ktc * (TK * 2);
+            const bool ak_ok = !GUARD_K || ktc * TK + a_chunk * 8 < K;
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int j = 2 * p + jj;
+                // a chunk past K is never dereferenced: its address could lie beyond the last row
+                ra[j] = ak_ok ? *reinterpret_cast<const uint4*>(base + a_off[j]) : make_uint4(0, 0, 0, 0);
+            }
+        } else {
+            ra[p] = k_ok ? *reinterpret_cast<const uint4*>(a_bytes + (size_t)ktc * TK + a_off[p]) : make_uint4(0, 0, 0, 0);
+            sa[p] = k_ok ? (a_scales + (size_t)ktc * (TK / 32))[as_off[p]] : 0u;
+        }
+        rw[p] = k_ok ? *reinterpret_cast<const uint4*>(w_elements + (size_t)ktc * TK + w_off[p]) : make_uint4(0, 0, 0, 0);
+        sw[p] = k_ok ? (w_scales + (size_t)ktc * (TK / 32))[ws_off[p]] : 0u;
+    };
+
+    auto stage_part = [&](int p, int buf) {
+        uint8_t* const pa = lds_a + buf * SLAB_BYTES;
+        uint8_t* const pw = lds_w + buf * SLAB_BYTES;
+        if (A_MODE == 0) {
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int j = 2 * p + jj;
+                *reinterpret_cast<uint4*>(pa + (j * 32 + a_row0) * ROW_BYTES + a_chunk * 16) = ra[j];
+            }
+        } else {
+            uint4 lo, hi;
+            Composer<FA>(sa[p]).run16(ra[p], lo, hi);
+            uint4* q = reinterpret_cast<uint4*>(pa + (p * 64 + c_row0) * ROW_BYTES + c_chunk * 32);
+            q[0] = lo; q[1] = hi;
+        }
+        {
+            uint4 lo, hi;
+            Composer<FW>(sw[p]).run16(rw[p], lo, hi);
+            uint4* q = reinterpret_cast<uint4*>(pw + (p * 64 + c_row0) * ROW_BYTES + c_chunk * 32);
+            q[0] = lo; q[1] = hi;
+        }
+    };
+
+    floatx16 acc[4][4];  // [n-tile j][m-tile i]
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.0f;
+
+    const int frag_off = (lane & 31) * ROW_BYTES + (lane >> 5) * 16;  // the lane's row and its 8 k values
+    const uint8_t* const frag_a = lds_a + wave_m * 128 * ROW_BYTES + frag_off;
+    const uint8_t* const frag_w = lds_w + wave_n * 128 * ROW_BYTES + frag_off;
+    auto load_frags = [&](int buf, int ks, bf16x8 (&af)[4], bf16x8 (&wf)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(frag_a + buf * SLAB_BYTES + i * 32 * ROW_BYTES + ks * 32);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(frag_w + buf * SLAB_BYTES + j * 32 * ROW_BYTES + ks * 32);
+    };
+    auto mfma16 = [&](const bf16x8 (&af)[4], const bf16x8 (&wf)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], af[i], acc[j][i], 0, 0, 0);
+    };
+    // one MFMA, then a slice of the phase's other work: keeps the matrix pipe fed while the
+    // vector ALU composes, the LDS is read and written and the next global loads are issued
+    auto interleave = [&]() {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+            if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);   // VALU
+            if (i >= 8 && i < 12) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
+            if (i >= 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
+        }
+    };
+
+    // ---- prologue: slab 0 complete in LDS[0], part 0 of slab 1 in LDS[1]; registers hold parts
+    //      1..3 of slab 1 and part 0 of slab 2
+#pragma unroll
+    for (int p = 0; p < 4; ++p) fetch_part(p, 0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) stage_part(p, 0);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) fetch_part(p, 1);
+    stage_part(0, 1);
+    fetch_part(0, 2);
+    __syncthreads();
+
+    bf16x8 fa0[4], fw0[4], fa1[4], fw1[4];
+    load_frags(0, 0, fa0, fw0);
+
+    // ---- main loop.  Step kt multiplies slab kt (LDS[cur]).  Its phases 0..2 finish staging slab
+    //      kt+1 into LDS[nxt]; after the barrier LDS[cur] is free and phase 3 starts staging slab kt+2.
+    //      Each register part is refilled from global memory right after it has been staged, one
+    //      whole K-step before it is needed again.
+    for (int kt = 0; kt < ksteps; ++kt) {
+        const int cur = kt & 1, nxt = cur ^ 1;
+        load_frags(cur, 1, fa1, fw1);
+        mfma16(fa0, fw0);
+        stage_part(1, nxt);
+        fetch_part(1, kt + 2);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+
+        load_frags(cur, 2, fa0, fw0);
+        mfma16(fa1, fw1);
+        stage_part(2, nxt);
+        fetch_part(2, kt + 2);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+
+        load_frags(cur, 3, fa1, fw1);
+        mfma16(fa0, fw0);
+        stage_part(3, nxt);
+        fetch_part(3, kt + 2);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+
+        __syncthreads();
+
+        load_frags(nxt, 0, fa0, fw0);
+        mfma16(fa1, fw1);
+        stage_part(0, cur);
+        fetch_part(0, kt + 3);
+        interleave();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- epilogue: lane holds, for tile (j, i) and g = 0..3, y[m][n .. n+3] with
+    //      m = m0 + wave_m*128 + i*32 + lane%32,  n = n0 + wave_n*128 + j*32 + 8*g + 4*(lane/32)
+    const bool vec_ok = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int n = n0 + wave_n * 128 + j * 32 + 8 * g + 4 * (lane >> 5);
+            const int valid = N - n >= 4 ? 4 : (N - n > 0 ? N - n : 0);
+            float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (bias)
+                for (int t = 0; t < valid; ++t) b[t] = load_bias(bias, bias_dtype, n + t);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int m = m0 + wave_m * 128 + i * 32 + (lane & 31);
+                if (m >= M || valid == 0) continue;
+                const float r[4] = {acc[j][i][4 * g] + b[0], acc[j][i][4 * g + 1] + b[1], acc[j][i][4 * g + 2] + b[2],
+                                    acc[j][i][4 * g + 3] + b[3]};
+                store_out4<DT_OUT>(y, (int64_t)m * N + n, r, vec_ok, valid);
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Small-shape kernel: 128 x 128 x 32 tiles, single LDS buffer.  Used when the problem cannot
+// fill the chip with 256 x 256 tiles.
+// ---------------------------------------------------------------------------------------------
+constexpr int SBM = 128, SBN = 128, SBK = 32;
+constexpr int S_STRIDE = SBK + 8;  // bf16 elements per tile row: 80 bytes
+
+template <int A_MODE, class FA, class FW, int DT_OUT>
+__global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
+    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ a_elements,
+    const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements, const void* __restrict__ bias,
+    int bias_dtype, void* __restrict__ y, int M, int N, int K) {
+    __shared__ __attribute__((aligned(16))) uint16_t lds_a[SBM * S_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_w[SBN * S_STRIDE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave >> 1, wave_n = wave & 1;  // 2 x 2 waves, 64 x 64 each
+    const int m0 = blockIdx.y * SBM, n0 = blockIdx.x * SBN;
+    const int kblocks = K / 32;
+
+    const int srow = tid >> 1, shalf = tid & 1;  // thread stages tile row tid/2, 16 k values
+    const bool a_row_ok = m0 + srow < M, w_row_ok = n0 + srow < N;
+    const int64_t a_row = (int64_t)(m0 + srow), w_row = (int64_t)(n0 + srow);
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    uint4 ra0 = make_uint4(0, 0, 0, 0), ra1 = ra0, rw = ra0;
+    uint32_t sa = 0, sw = 0;
+    auto fetch = [&](int kt) {
+        const int64_t k = (int64_t)kt * SBK + shalf * 16;
+        if (a_row_ok) {
+            if (A_MODE == 0) {
+                const uint4* p = reinterpret_cast<const uint4*>(a_dense + a_row * K + k);
+                ra0 = p[0];
+                ra1 = p[1];
+            } else {
+                ra0 = *reinterpret_cast<const uint4*>(a_elements + a_row * K + k);
+                sa = a_scales[a_row * kblocks + kt];
+            }
+        }
+        if (w_row_ok) {
+            rw = *reinterpret_cast<const uint4*>(w_elements + w_row * K + k);
+            sw = w_scales[w_row * kblocks + kt];
+        }
+    };
+
+    const int ktiles = K / SBK;
+    fetch(0);
+    for (int kt = 0; kt < ktiles; ++kt) {
+        __syncthreads();  // everyone finished reading the previous slab
+        {
+            uint4 lo, hi;
+            if (A_MODE == 0) { lo = ra0; hi = ra1; }
+            else Composer<FA>(sa).run16(ra0, lo, hi);
+            uint4* pa = reinterpret_cast<uint4*>(&lds_a[srow * S_STRIDE + shalf * 16]);
+            pa[0] = lo; pa[1] = hi;
+            Composer<FW>(sw).run16(rw, lo, hi);
+            uint4* pw = reinterpret_cast<uint4*>(&lds_w[srow * S_STRIDE + shalf * 16]);
+            pw[0] = lo; pw[1] = hi;
+        }
+        __syncthreads();
+        if (kt + 1 < ktiles) fetch(kt + 1);
+#pragma unroll
+        for (int ks = 0; ks < SBK / 16; ++ks) {
+            bf16x8 af[2], wf[2];
+            const int kofs = ks * 16 + (lane >> 5) * 8;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                af[i] = *reinterpret_cast<const bf16x8*>(&lds_a[(wave_m * 64 + i * 32 + (lane & 31)) * S_STRIDE + kofs]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                wf[j] = *reinterpret_cast<const bf16x8*>(&lds_w[(wave_n * 64 + j * 32 + (lane & 31)) * S_STRIDE + kofs]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wave_n * 64 + j * 32 + (lane & 31);
+            if (col >= N) continue;
+            const float b = bias ? load_bias(bias, bias_dtype, col) : 0.0f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = m0 + wave_m * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < M) store_out<DT_OUT>(y, (int64_t)row * N + col, acc[i][j][v] + b);
+            }
+        }
+}
+
+template <int A_MODE, class FA, class FW, int DT_OUT>
+int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_elements, const uint8_t* w_scales,
+                const uint8_t* w_elements, const void* bias, int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
+    const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
+    const int64_t big_tiles = (int64_t)tiles_m * tiles_n;
+    // 256 x 256 tiles need enough of them to occupy the 256 CUs; smaller problems use 128 x 128
+    const bool fits32 = (int64_t)M * K * 2 < ((int64_t)1 << 32) && (int64_t)N * K < ((int64_t)1 << 32);  // 32-bit operand offsets
+    const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
+    if (use_big) {
+        const bool guard_k = K % TK != 0;
+        auto kern = guard_k ? mxfp_gemm_kernel<A_MODE, FA, FW, DT_OUT, true> : mxfp_gemm_kernel<A_MODE, FA, FW, DT_OUT, false>;
+        constexpr int lds_bytes = 4 * SLAB_BYTES;
+        static bool attr_set[2] = {false, false};
+        if (!attr_set[guard_k]) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
+            attr_set[guard_k] = true;
+        }
+        const unsigned grid = (unsigned)(((big_tiles + 7) / 8) * 8);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), a_scales,
+                           a_elements, w_scales, w_elements, bias, bias_dtype, y, M, N, K, tiles_m, tiles_n);
+    } else {
+        const dim3 grid((unsigned)((N + SBN - 1) / SBN), (unsigned)((M + SBM - 1) / SBM));
+        if (grid.y > 65535u) return fail(ERR_UNSUPPORTED, "M too large for the launch grid");
+        hipLaunchKernelGGL((mxfp_gemm_small_kernel<A_MODE, FA, FW, DT_OUT>), grid, dim3(kGemmThreads), 0, s,
+                           static_cast<const uint16_t*>(a_dense), a_scales, a_elements, w_scales, w_elements, bias, bias_dtype, y, M,
+                           N, K);
+    }
+    return check_launch("mxfp_gemm");
+}
+
+
+// One entry per weight format; each lives in its own translation unit (gemm_w_*.hip) so that the
+// formats compile in parallel.  a_exp_bits == 0 selects the dense-A kernel.
+struct GemmArgs {
+    const void* a_dense; const uint8_t* a_scales; const uint8_t* a_elements; int a_exp_bits, a_frac_bits;
+    const uint8_t* w_scales; const uint8_t* w_elements; const void* bias; int bias_dtype; void* y; int out_dtype;
+    int M, N, K; hipStream_t stream;
+};
+int gemm_w_e4m3(const GemmArgs& g);
+int gemm_w_e5m2(const GemmArgs& g);
+int gemm_w_e2m3(const GemmArgs& g);
+int gemm_w_e3m2(const GemmArgs& g);
+int gemm_w_e2m1(const GemmArgs& g);
+
+template <class FW>
+int gemm_for_weight_format(const GemmArgs& g) {
+    return dispatch_dtype(g.out_dtype, [&](auto dout) {
+        constexpr int DO = decltype(dout)::value;
+        if (g.a_dense)
+            return launch_gemm<0, SFmt<4, 3>, FW, DO>(g.a_dense, nullptr, nullptr, g.w_scales, g.w_elements, g.bias, g.bias_dtype, g.y,
+                                                      g.M, g.N, g.K, g.stream);
+        const int E = g.a_exp_bits, M = g.a_frac_bits;
+#define MASE_A_FMT(e, m)                                                                                                       \
+        if (E == e && M == m)                                                                                                  \
+            return launch_gemm<1, SFmt<e, m>, FW, DO>(nullptr, g.a_scales, g.a_elements, g.w_scales, g.w_elements, g.bias,     \
+                                                      g.bias_dtype, g.y, g.M, g.N, g.K, g.stream);
+        MASE_A_FMT(4, 3) MASE_A_FMT(5, 2) MASE_A_FMT(2, 3) MASE_A_FMT(3, 2) MASE_A_FMT(2, 1)
+#undef MASE_A_FMT
+        return fail(ERR_INVALID, "MXFP element (exp_bits, frac_bits) must be one of (4,3) (5,2) (2,3) (3,2) (2,1)");
+    });
+}
+
+}  // namespace mase

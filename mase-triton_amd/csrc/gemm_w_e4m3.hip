@@ -1,0 +1,6 @@
+// MXFP GEMM kernels for weights in E4M3; see gemm_impl.h.
+#include "gemm_impl.h"
+
+namespace mase {
+int gemm_w_e4m3(const GemmArgs& g) { return gemm_for_weight_format<SFmt<4, 3>>(g); }
+}  // namespace mase
