@@ -35,67 +35,135 @@ __device__ inline uint32_t cvt_pk_bf16(float a, float b) {
 // A code's magnitude bits, placed so that its exponent field sits in the low bits of an fp16
 // exponent field, read as fp16 give value * 2^(bias - 15) for normal AND subnormal codes (an fp16
 // subnormal has the same meaning as a minifloat subnormal) and 0 for the zero code.  The hardware
-// fp16 -> fp32 convert is exact; one fp32 multiply by 2^(15 - bias + scale - 127) finishes the
-// job with the single rounding the reference has (only when the product leaves the fp32 normal
-// range), and the fp32 -> bf16 convert is round-to-nearest-even like the reference's cast.
+// fp16 -> fp32 convert is exact; v_ldexp_f32 by (15 - bias + scale - 127) finishes the job with
+// the single rounding the reference's fp32 multiply has (only when the product leaves the fp32
+// normal range), and the fp32 -> bf16 convert is round-to-nearest-even like the reference's cast.
+// Scale 255 means "times +inf" in the reference (0 -> NaN, anything else -> +-inf): that case is
+// patched afterwards by fix255().  E = 5 would fill the fp16 exponent field (field 31 reads as
+// inf/NaN), so E5M2 codes take the generic integer decode instead.
 // ---------------------------------------------------------------------------------------------
 template <class F>
 struct Composer {
-    float c1, c2;     // value = (fp16-read * c1) * c2 ; c2 == 1 unless the scale is extreme
-    bool two_step;
+    static constexpr int E = F{}.E(), M = F{}.M();
+    static constexpr int PRE = 7 - E - M;      // left shift that moves the sign bit to bit 7 of each byte
+    static constexpr int ASHR = 5 - E;         // then: exponent field from bits 14.. down to bits ..10 of each half
+    static constexpr uint32_t KEEP = (0x8000u | (0x7FFFu >> ASHR)) * 0x00010001u;
+
+    int n;          // ldexp exponent: 15 - bias + scale - 127
+    float s_wide;   // 2^(scale - 127), for the generic path
     __device__ inline explicit Composer(uint32_t scale) {
-        const F f{};
-        const int field = (int)scale + 15 - fmt_bias(f);  // exponent field of 2^(15 - bias + scale - 127)
-        two_step = field < 1 || field > 254;
-        if (f.E() >= 5) { two_step = false; c1 = 1.0f; c2 = scale_f32(scale); }
-        else if (!two_step) { c1 = bits_f32((uint32_t)field << 23); c2 = 1.0f; }
-        else { c1 = bits_f32((uint32_t)(142 - fmt_bias(f)) << 23); c2 = scale_f32(scale); }
+        n = (int)scale - 112 - fmt_bias(F{});
+        s_wide = scale_f32(scale);
     }
-    // codes in bytes (2p, 2p+1) of w -> packed fp16 pair
-    template <int P>
-    __device__ static inline uint32_t half_pair(uint32_t w) {
-        const F f{};
-        constexpr uint32_t sel = P == 0 ? 0x010C000Cu : 0x030C020Cu;
-        const uint32_t x = __builtin_amdgcn_perm(0u, w, sel);  // each 16-bit half = code << 8
-        const int E = f.E(), M = f.M();
-        const uint32_t mag_mask = (((1u << (E + M)) - 1u) << 8) * 0x00010001u;
-        uint32_t mag = x & mag_mask;
-        if (M > 2) mag >>= (M - 2);
-        if (M < 2) mag <<= (2 - M);
-        const uint32_t sgn = (x << (7 - E - M)) & 0x80008000u;
-        return mag | sgn;
+    __device__ inline uint32_t bf16_pair(uint32_t x) const {  // x: each 16-bit half = (code << PRE) << 8
+        typedef short shortx2 __attribute__((ext_vector_type(2)));
+        const shortx2 sh = __builtin_bit_cast(shortx2, x) >> (short)ASHR;   // v_pk_ashrrev_i16
+        const halfx2_t h = __builtin_bit_cast(halfx2_t, __builtin_bit_cast(uint32_t, sh) & KEEP);
+        return cvt_pk_bf16(ldexpf((float)h[0], n), ldexpf((float)h[1], n));
     }
-    __device__ inline uint32_t bf16_pair(uint32_t halves) const {
-        const halfx2_t h = __builtin_bit_cast(halfx2_t, halves);
-        float a = (float)h[0] * c1, b = (float)h[1] * c1;
-        if (two_step) { a *= c2; b *= c2; }
-        return cvt_pk_bf16(a, b);
-    }
-    // E = 5 fills the whole fp16 exponent field (field 31 would read as inf/NaN): decode those
-    // codes with the generic integer path instead
     __device__ inline uint32_t bf16_pair_wide(uint32_t w, int p) const {
         const F f{};
-        const float a = decode_f32((w >> (16 * p)) & 0xFFu, f) * c2, b = decode_f32((w >> (16 * p + 8)) & 0xFFu, f) * c2;
+        const float a = decode_f32((w >> (16 * p)) & 0xFFu, f) * s_wide, b = decode_f32((w >> (16 * p + 8)) & 0xFFu, f) * s_wide;
         return cvt_pk_bf16(a, b);
     }
-    // 16 codes (one 128-bit word) of one block -> 16 bf16 (two 128-bit words)
+    // ---- integer placement (E >= 4 only): for a NORMAL code the bf16 pattern is just the code's
+    // fields moved into place plus (scale - bias) added to the exponent field:
+    //     bf16 = sign << 15 | (xe + scale - bias) << 7 | xf << (7 - M)
+    // valid while 1 <= xe + scale - bias <= 254.  Codes with exponent field 0 (zero, subnormal),
+    // scale 255 and out-of-range exponents are not covered: callers test covers16() and fall back.
+    static constexpr bool kHasIntPath = E >= 4;
+    static constexpr int ISHR = 8 - (7 - M);   // half = code << 8  ->  arithmetic shift right so that xf lands at bit 7 - M
+    static constexpr uint32_t IKEEP = (0x8000u | (((1u << (E + M)) - 1u) << (7 - M))) * 0x00010001u;
+    static constexpr uint32_t EXP_BYTES = (((1u << E) - 1u) << M) * 0x01010101u;       // exponent field of every byte
+    static constexpr uint32_t EXP_LSB_COMPL = (0x80u - (1u << M)) * 0x01010101u;         // + this: bit 7 set iff field != 0
+    // true iff every one of the 16 codes is a normal code and the block scale keeps all of them
+    // inside the bf16 normal range
+    __device__ static inline bool covers16(const uint4& codes, uint32_t scale) {
+        const int lo = (int)scale - fmt_bias(F{}) + 1, hi = (int)scale - fmt_bias(F{}) + (1 << E) - 1;
+        const uint32_t a = ((codes.x & EXP_BYTES) + EXP_LSB_COMPL) & ((codes.y & EXP_BYTES) + EXP_LSB_COMPL) &
+                           ((codes.z & EXP_BYTES) + EXP_LSB_COMPL) & ((codes.w & EXP_BYTES) + EXP_LSB_COMPL);
+        return (a & 0x80808080u) == 0x80808080u && lo >= 1 && hi <= 254;
+    }
+    __device__ inline void run16_int(const uint4& codes, uint32_t scale, uint4& lo, uint4& hi) const {
+        typedef short shortx2 __attribute__((ext_vector_type(2)));
+        typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
+        const uint32_t ss = (uint32_t)((int)scale - fmt_bias(F{})) << 7;
+        const ushortx2 add = {(unsigned short)ss, (unsigned short)ss};
+        const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
+        uint32_t o[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t x = __builtin_amdgcn_perm(0u, w[j], h == 0 ? 0x010C000Cu : 0x030C020Cu);  // halves = code << 8
+                const shortx2 sh = __builtin_bit_cast(shortx2, x) >> (short)ISHR;                           // v_pk_ashrrev_i16
+                const ushortx2 t = __builtin_bit_cast(ushortx2, __builtin_bit_cast(uint32_t, sh) & IKEEP);
+                o[2 * j + h] = __builtin_bit_cast(uint32_t, (ushortx2)(t + add));                           // v_pk_add_u16
+            }
+        lo = make_uint4(o[0], o[1], o[2], o[3]);
+        hi = make_uint4(o[4], o[5], o[6], o[7]);
+    }
+    // 16 codes (one 128-bit word) of one block -> 16 bf16 (two 128-bit words), any code, any scale < 255
     __device__ inline void run16(const uint4& codes, uint4& lo, uint4& hi) const {
         const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
         uint32_t o[8];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            if (F{}.E() >= 5) {
+            if (E >= 5) {
                 o[2 * j] = bf16_pair_wide(w[j], 0);
                 o[2 * j + 1] = bf16_pair_wide(w[j], 1);
             } else {
-                o[2 * j] = bf16_pair(half_pair<0>(w[j]));
-                o[2 * j + 1] = bf16_pair(half_pair<1>(w[j]));
+                const uint32_t ws = w[j] << PRE;  // top bits of every byte are zero: no spill between bytes
+                o[2 * j] = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x010C000Cu));
+                o[2 * j + 1] = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x030C020Cu));
             }
         }
         lo = make_uint4(o[0], o[1], o[2], o[3]);
         hi = make_uint4(o[4], o[5], o[6], o[7]);
     }
+    // Complete compose of one 16-code run.  Formats with a wide exponent field almost never hold
+    // zero-exponent codes (they are > 2^14 times smaller than the block maximum), so those take
+    // the cheap integer placement and only a wave that actually meets such a code, or an extreme
+    // scale, re-does its run through the general path.
+    __device__ static inline void compose16(const uint4& codes, uint32_t scale, uint4& lo, uint4& hi) {
+        const Composer c(scale);
+        if (kHasIntPath) {
+            c.run16_int(codes, scale, lo, hi);
+            if (__builtin_amdgcn_ballot_w64(!covers16(codes, scale)) == 0) return;
+            if (covers16(codes, scale)) return;
+        }
+        c.run16(codes, lo, hi);
+        fix255(scale, codes, lo, hi);
+    }
+    // scale 255: the ldexp path gave 0 for zero codes where the reference has 0 * inf = NaN
+    // (non-zero codes already overflowed to +-inf).  Rare: one wave-uniform branch per call.
+    __device__ static inline void fix255(uint32_t scale, const uint4& codes, uint4& lo, uint4& hi) {
+        if (E >= 5) return;  // the generic path multiplies by +inf itself
+        if (__builtin_amdgcn_ballot_w64(scale == 255u) == 0) return;
+        if (scale != 255u) return;
+        const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
+        uint32_t o[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        const uint32_t mag = (1u << (E + M)) - 1u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (((w[j] >> (8 * b)) & mag) == 0u) {
+                    uint32_t& d = o[2 * j + (b >> 1)];
+                    d = (b & 1) ? ((d & 0x0000FFFFu) | 0x7FC00000u) : ((d & 0xFFFF0000u) | 0x00007FC0u);
+                }
+        lo = make_uint4(o[0], o[1], o[2], o[3]);
+        hi = make_uint4(o[4], o[5], o[6], o[7]);
+    }
 };
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which
+// would make every wave wait for its outstanding output stores; here those are meant to drain in
+// the background while the next tile starts.
+__device__ inline void lds_barrier() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads and writes are done
+    __builtin_amdgcn_s_barrier();
+}
 
 __device__ inline float load_bias(const void* bias, int bias_dtype, int col) {
     if (bias_dtype == F32) return static_cast<const float*>(bias)[col];
@@ -147,19 +215,27 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_m = wave >> 1, wave_n = wave & 1;
 
-    // Tile order: workgroup ids go round-robin over the 8 XCDs (each with its own L2), so XCD x
-    // takes the contiguous band of tile rows [x * band, (x+1) * band); inside the band ids walk
-    // the N direction fastest in groups of 8 columns so that concurrent tiles share A and W slabs.
+    // Persistent workgroups: the grid is one workgroup per CU (a multiple of 8) and each walks a list
+    // of tiles, so a tile's output stores drain while the next tile is already loading.
+    // Tile order.  Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2, so XCD x
+    // owns the contiguous range of positions [x * per_xcd, (x+1) * per_xcd) and its workgroups take
+    // them in turn; positions walk the tile grid in groups of 4 tile-rows, rows fastest, so the tiles
+    // an XCD runs at once form a 4 x 8 patch that shares 4 A slabs and 8 W slabs through that L2.
+    const int n_tiles = tiles_m * tiles_n;
+    const int per_xcd = (n_tiles + 7) >> 3;
+    const int slots = gridDim.x >> 3;
+    for (int local = blockIdx.x >> 3; local < per_xcd; local += slots) {
+    const int pos = (blockIdx.x & 7) * per_xcd + local;
+    if (pos >= n_tiles) break;
     int tile_m, tile_n;
     {
-        const int id = blockIdx.x, n_tiles = tiles_m * tiles_n;
-        const int xcd = id & 7, local = id >> 3;
-        const int per_xcd = (n_tiles + 7) >> 3;
-        int linear = xcd * per_xcd + local;
-        if (per_xcd * 8 != n_tiles) linear = id;  // irregular tile counts: plain order
-        tile_m = linear / tiles_n;
-        tile_n = linear - tile_m * tiles_n;
-        if (tile_m >= tiles_m) return;
+        constexpr int GROUP = 4;
+        const int in_group = GROUP * tiles_n;
+        const int first_m = (pos / in_group) * GROUP;
+        const int rows = min(tiles_m - first_m, GROUP);
+        const int r = pos % in_group;
+        tile_m = first_m + r % rows;
+        tile_n = r / rows;
     }
     const int m0 = tile_m * TM, n0 = tile_n * TN;
     const int kblocks = K / 32;
@@ -230,13 +306,13 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
             }
         } else {
             uint4 lo, hi;
-            Composer<FA>(sa[p]).run16(ra[p], lo, hi);
+            Composer<FA>::compose16(ra[p], sa[p], lo, hi);
             uint4* q = reinterpret_cast<uint4*>(pa + (p * 64 + c_row0) * ROW_BYTES + c_chunk * 32);
             q[0] = lo; q[1] = hi;
         }
         {
             uint4 lo, hi;
-            Composer<FW>(sw[p]).run16(rw[p], lo, hi);
+            Composer<FW>::compose16(rw[p], sw[p], lo, hi);
             uint4* q = reinterpret_cast<uint4*>(pw + (p * 64 + c_row0) * ROW_BYTES + c_chunk * 32);
             q[0] = lo; q[1] = hi;
         }
@@ -288,7 +364,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     for (int p = 0; p < 4; ++p) fetch_part(p, 1);
     stage_part(0, 1);
     fetch_part(0, 2);
-    __syncthreads();
+    lds_barrier();
 
     bf16x8 fa0[4], fw0[4], fa1[4], fw1[4];
     load_frags(0, 0, fa0, fw0);
@@ -320,7 +396,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         interleave();
         __builtin_amdgcn_sched_barrier(0);
 
-        __syncthreads();
+        lds_barrier();
 
         load_frags(nxt, 0, fa0, fw0);
         mfma16(fa1, fw1);
@@ -351,6 +427,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
                 store_out4<DT_OUT>(y, (int64_t)m * N + n, r, vec_ok, valid);
             }
         }
+    lds_barrier();  // nobody may still be reading this tile's last slabs when the next tile stages
+    }  // tile loop
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -412,10 +490,10 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
         {
             uint4 lo, hi;
             if (A_MODE == 0) { lo = ra0; hi = ra1; }
-            else Composer<FA>(sa).run16(ra0, lo, hi);
+            else Composer<FA>::compose16(ra0, sa, lo, hi);
             uint4* pa = reinterpret_cast<uint4*>(&lds_a[srow * S_STRIDE + shalf * 16]);
             pa[0] = lo; pa[1] = hi;
-            Composer<FW>(sw).run16(rw, lo, hi);
+            Composer<FW>::compose16(rw, sw, lo, hi);
             uint4* pw = reinterpret_cast<uint4*>(&lds_w[srow * S_STRIDE + shalf * 16]);
             pw[0] = lo; pw[1] = hi;
         }
@@ -471,7 +549,17 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
             attr_set[guard_k] = true;
         }
-        const unsigned grid = (unsigned)(((big_tiles + 7) / 8) * 8);
+        static int n_cus = 0;
+        if (n_cus == 0) {
+            int dev = 0;
+            hipDeviceProp_t prop;
+            if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+                return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
+            n_cus = prop.multiProcessorCount > 8 ? prop.multiProcessorCount : 8;
+        }
+        // one persistent workgroup per CU (rounded down to a multiple of 8 XCD slots), never more than tiles
+        const int64_t want = big_tiles < n_cus ? ((big_tiles + 7) / 8) * 8 : (n_cus / 8) * 8;
+        const unsigned grid = (unsigned)want;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), a_scales,
                            a_elements, w_scales, w_elements, bias, bias_dtype, y, M, N, K, tiles_m, tiles_n);
     } else {
