@@ -240,6 +240,136 @@ __global__ __launch_bounds__(kThreads) void extract_mxfp_kernel(const void* __re
     }
 }
 
+template <class F>
+__device__ inline float mxfp_value(uint32_t code, float scale, const F& f) {
+    return decode_f32(code, f) * scale;
+}
+
+// ------------------------------------------------------------------------------ bf16 fast path
+// bfloat16 input, block size 32, compile-time format.  A lane owns 8 consecutive elements (one
+// 128-bit load), four adjacent lanes own a block.  Two elements are processed per 32-bit
+// register with packed 16-bit integer instructions; there is no per-element branch.
+//
+// With h the bf16 bits, a = h & 0x7FFF and scale the block's biased shared exponent, the value
+//     t = a - ((scale - bias) << 7)        (signed, clamped at 0)
+// is  (ye << 7) | f7 : the element's exponent field in the target format above its 7 mantissa
+// bits.  Rounding to M bits, the reference's "(ye << M) | yf" with its lost carry, the one
+// reachable subnormal binade (ye == 0) and underflow (t < 0) are all functions of t alone.
+// Not covered, and sent to the exact per-element routine by a wave-uniform test: blocks holding
+// inf/NaN, and scales >= 151 (only there can a quotient underflow to exactly zero).
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+
+__device__ inline uint32_t as_u32(u16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ inline uint32_t as_u32(i16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ inline u16x2 as_u16x2(uint32_t v) { return __builtin_bit_cast(u16x2, v); }
+__device__ inline i16x2 as_i16x2(uint32_t v) { return __builtin_bit_cast(i16x2, v); }
+
+template <class F>
+struct PackedBf16 {
+    static constexpr int E = F{}.E(), M = F{}.M(), SH = 7 - M;
+    static constexpr uint32_t LSB = 0x00010001u;
+    // code magnitudes (exponent and mantissa fields, no sign) of two elements, one per 16-bit half,
+    // plus, through `t_q`, the quantised magnitude back in the t domain for the fused QDQ
+    __device__ static inline uint32_t magnitude(uint32_t a, uint32_t ssb2, uint32_t& t_q) {
+        i16x2 t = as_i16x2(a) - as_i16x2(ssb2);
+        t = __builtin_elementwise_max(t, (i16x2){0, 0});                    // underflow -> 0
+        const uint32_t tu = as_u32(t);
+        const uint32_t u = as_u32(as_u16x2(tu) >> (unsigned short)SH);    // (ye << M) | truncated mantissa
+        const uint32_t r = tu + (((1u << (SH - 1)) - 1u) * LSB) + (u & LSB);  // round half to even
+        const uint32_t v = as_u32(as_u16x2(r) >> (unsigned short)SH);     // (ye << M) + rounded mantissa
+        // a carry out of the mantissa into an odd exponent field is lost by the reference's OR
+        const uint32_t code_n = v - (((v ^ u) >> 1) & ((1u << M) * LSB));
+        // ye == 0: the mantissa (with its carry) is shifted down under an explicit leading one
+        const uint32_t w = as_u32(as_u16x2(v | ((1u << M) * LSB)) >> (unsigned short)1);
+        const uint32_t code_s = as_u32(as_u16x2(w) * __builtin_elementwise_min(as_u16x2(v), (u16x2){1, 1}));
+        const uint32_t is_norm = as_u32(((i16x2){127, 127} - t) >> (short)15);  // all ones where ye >= 1
+        // t-domain value of the code: normal codes keep their fields; subnormal code xf' (>= 2^(M-1))
+        // is 2^-bias * xf' / 2^(M-1), i.e. exponent field 0 and mantissa (xf' << (8 - M)) & 0x7F
+        const uint32_t tq_n = code_n << SH;
+        const uint32_t tq_s = (code_s << (8 - M)) & (0x7Fu * LSB);
+        t_q = (is_norm & tq_n) | (~is_norm & tq_s);
+        return (is_norm & code_n) | (~is_norm & code_s);
+    }
+    // all ones in the halves whose input has a non-zero exponent field (everything else is flushed
+    // to +0.0 by the reference before encoding and gets code 0, sign included)
+    __device__ static inline uint32_t live_mask(uint32_t a) { return as_u32(as_i16x2(a + 0x7F807F80u) >> (short)15); }
+    __device__ static inline uint32_t codes(uint32_t h, uint32_t ssb2) {
+        const uint32_t a = h & 0x7FFF7FFFu;
+        uint32_t t_q;
+        const uint32_t mag = magnitude(a, ssb2, t_q);
+        const uint32_t sgn = (h >> (15 - (E + M))) & ((1u << (E + M)) * LSB);
+        return (mag | sgn) & live_mask(a);
+    }
+    // quantise-dequantise of two bf16 values; valid when every non-zero code lands in the bf16
+    // normal range, i.e. scale > bias (smaller scales give subnormal results: slow path)
+    __device__ static inline uint32_t qdq(uint32_t h, uint32_t ssb2) {
+        const uint32_t a = h & 0x7FFF7FFFu;
+        uint32_t t_q;
+        const uint32_t mag = magnitude(a, ssb2, t_q);
+        const uint32_t nonzero = as_u32((i16x2){0, 0} - as_i16x2(as_u32(__builtin_elementwise_min(as_u16x2(mag), (u16x2){1, 1}))));
+        const uint32_t body = (t_q + ssb2) & nonzero;                      // code 0 -> +-0.0
+        return (body | (h & 0x80008000u)) & live_mask(a);
+    }
+};
+
+// MODE 0: extract (scales + elements); MODE 1: fused quantise-dequantise to bf16
+template <class F, int UNROLL, int MODE>
+__global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __restrict__ x, uint8_t* __restrict__ scales,
+                                                                  uint2* __restrict__ elements, uint4* __restrict__ out,
+                                                                  int64_t n_chunks, F f) {
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint4 raw[UNROLL];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        raw[r] = c < n_chunks ? x[c] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        const uint32_t h[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
+        // block maximum of |x| bits: packed max over the lane's four registers, then the two halves,
+        // then the four lanes of the block (DPP quad permutes)
+        u16x2 m2 = __builtin_elementwise_max(__builtin_elementwise_max(as_u16x2(h[0] & 0x7FFF7FFFu), as_u16x2(h[1] & 0x7FFF7FFFu)),
+                                             __builtin_elementwise_max(as_u16x2(h[2] & 0x7FFF7FFFu), as_u16x2(h[3] & 0x7FFF7FFFu)));
+        uint32_t amax = max((uint32_t)m2[0], (uint32_t)m2[1]);
+        amax = max(amax, (uint32_t)__builtin_amdgcn_mov_dpp((int)amax, 0xB1, 0xF, 0xF, true));  // lane ^ 1
+        amax = max(amax, (uint32_t)__builtin_amdgcn_mov_dpp((int)amax, 0x4E, 0xF, 0xF, true));  // lane ^ 2
+        const int ef_max = (int)(amax >> 7);
+        const int scale_n = max(ef_max - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
+        const bool hard = amax >= 0x7F80u || scale_n >= 151 || (MODE == 1 && amax != 0u && scale_n <= fmt_bias(f));
+        uint32_t o[4];
+        uint32_t scale = (uint32_t)scale_n;
+        if (__builtin_amdgcn_ballot_w64(hard) == 0) {
+            const uint32_t ssb = (uint32_t)((scale_n - fmt_bias(f)) << 7) & 0xFFFFu;
+            const uint32_t ssb2 = ssb | (ssb << 16);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = MODE == 0 ? PackedBf16<F>::codes(h[j], ssb2) : PackedBf16<F>::qdq(h[j], ssb2);
+        } else {
+            // exact per-element routine (the block's lanes agree on amax, so they agree on the result)
+            const uint32_t amax32 = amax << 16;
+            const int se = shared_exponent<F, true>(amax32, f);
+            scale = amax32 < 0x00800000u ? 0u : (uint32_t)(se + 127);
+            const float sc = scale_f32(scale);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t c0 = encode_mxfp_element(h[j] << 16, se, f), c1 = encode_mxfp_element(h[j] & 0xFFFF0000u, se, f);
+                o[j] = MODE == 0 ? (c0 | (c1 << 16)) : pack_bf16(mxfp_value(c0, sc, f), mxfp_value(c1, sc, f));
+            }
+        }
+        if (c < n_chunks) {
+            if (MODE == 0) {
+                // o[j] holds two codes in the low bytes of its halves: gather the 8 code bytes
+                elements[c] = make_uint2(__builtin_amdgcn_perm(o[1], o[0], 0x06040200u), __builtin_amdgcn_perm(o[3], o[2], 0x06040200u));
+                if ((c & 3) == 0) scales[c >> 2] = (uint8_t)scale;
+            } else {
+                out[c] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+        }
+    }
+}
+
 // Fallback for any block size / alignment: one lane owns one block.
 template <int DT_IN, class F>
 __global__ __launch_bounds__(kThreads) void extract_mxfp_block_kernel(const void* __restrict__ x, uint8_t* __restrict__ scales,
@@ -255,11 +385,6 @@ __global__ __launch_bounds__(kThreads) void extract_mxfp_block_kernel(const void
     const int se = shared_exponent<F, DT_IN != F32>(amax, f);
     scales[b] = amax < 0x00800000u ? (uint8_t)0 : (uint8_t)(se + 127);
     for (int j = 0; j < B; ++j) elements[b * B + j] = (uint8_t)encode_mxfp_element(load_bits_scalar<DT_IN>(x, b * B + j), se, f);
-}
-
-template <class F>
-__device__ inline float mxfp_value(uint32_t code, float scale, const F& f) {
-    return decode_f32(code, f) * scale;
 }
 
 // Vector path: B % EPT == 0 (a lane's run lies inside one block).
@@ -454,6 +579,14 @@ int mase_hip_extract_mxfp(const void* x, int x_dtype, uint8_t* scales, uint8_t* 
     const int B = block_size;
     const bool vec = B % EPT == 0 && pow2(B / EPT) && B / EPT <= 64 && aligned(x, 16) && aligned(elements, 8);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        if constexpr (decltype(f)::kStatic) {
+            if (x_dtype == BF16 && B == 32 && vec) {
+                constexpr int U = 4;
+                hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 0>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
+                                   static_cast<const uint4*>(x), scales, reinterpret_cast<uint2*>(elements), nullptr, n / 8, f);
+                return check_launch("extract_mxfp");
+            }
+        }
         return dispatch_dtype(x_dtype, [&](auto dt) {
             if (vec) {
                 const int lpb = B / EPT;
@@ -510,6 +643,14 @@ int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int6
     const int B = block_size;
     const bool vec = B % EPT == 0 && pow2(B / EPT) && B / EPT <= 64 && aligned(x, 16) && aligned(out, 16);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        if constexpr (decltype(f)::kStatic) {
+            if (x_dtype == BF16 && out_dtype == BF16 && B == 32 && vec) {
+                constexpr int U = 4;
+                hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 1>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
+                                   static_cast<const uint4*>(x), nullptr, nullptr, static_cast<uint4*>(out), n / 8, f);
+                return check_launch("qdq_mxfp");
+            }
+        }
         return dispatch_dtype(x_dtype, [&](auto di) {
             return dispatch_dtype(out_dtype, [&](auto dout) {
                 if (vec) {

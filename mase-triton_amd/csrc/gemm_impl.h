@@ -66,43 +66,6 @@ struct Composer {
         const float a = decode_f32((w >> (16 * p)) & 0xFFu, f) * s_wide, b = decode_f32((w >> (16 * p + 8)) & 0xFFu, f) * s_wide;
         return cvt_pk_bf16(a, b);
     }
-    // ---- integer placement (E >= 4 only): for a NORMAL code the bf16 pattern is just the code's
-    // fields moved into place plus (scale - bias) added to the exponent field:
-    //     bf16 = sign << 15 | (xe + scale - bias) << 7 | xf << (7 - M)
-    // valid while 1 <= xe + scale - bias <= 254.  Codes with exponent field 0 (zero, subnormal),
-    // scale 255 and out-of-range exponents are not covered: callers test covers16() and fall back.
-    static constexpr bool kHasIntPath = E >= 4;
-    static constexpr int ISHR = 8 - (7 - M);   // half = code << 8  ->  arithmetic shift right so that xf lands at bit 7 - M
-    static constexpr uint32_t IKEEP = (0x8000u | (((1u << (E + M)) - 1u) << (7 - M))) * 0x00010001u;
-    static constexpr uint32_t EXP_BYTES = (((1u << E) - 1u) << M) * 0x01010101u;       // exponent field of every byte
-    static constexpr uint32_t EXP_LSB_COMPL = (0x80u - (1u << M)) * 0x01010101u;         // + this: bit 7 set iff field != 0
-    // true iff every one of the 16 codes is a normal code and the block scale keeps all of them
-    // inside the bf16 normal range
-    __device__ static inline bool covers16(const uint4& codes, uint32_t scale) {
-        const int lo = (int)scale - fmt_bias(F{}) + 1, hi = (int)scale - fmt_bias(F{}) + (1 << E) - 1;
-        const uint32_t a = ((codes.x & EXP_BYTES) + EXP_LSB_COMPL) & ((codes.y & EXP_BYTES) + EXP_LSB_COMPL) &
-                           ((codes.z & EXP_BYTES) + EXP_LSB_COMPL) & ((codes.w & EXP_BYTES) + EXP_LSB_COMPL);
-        return (a & 0x80808080u) == 0x80808080u && lo >= 1 && hi <= 254;
-    }
-    __device__ inline void run16_int(const uint4& codes, uint32_t scale, uint4& lo, uint4& hi) const {
-        typedef short shortx2 __attribute__((ext_vector_type(2)));
-        typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
-        const uint32_t ss = (uint32_t)((int)scale - fmt_bias(F{})) << 7;
-        const ushortx2 add = {(unsigned short)ss, (unsigned short)ss};
-        const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
-        uint32_t o[8];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint32_t x = __builtin_amdgcn_perm(0u, w[j], h == 0 ? 0x010C000Cu : 0x030C020Cu);  // halves = code << 8
-                const shortx2 sh = __builtin_bit_cast(shortx2, x) >> (short)ISHR;                           // v_pk_ashrrev_i16
-                const ushortx2 t = __builtin_bit_cast(ushortx2, __builtin_bit_cast(uint32_t, sh) & IKEEP);
-                o[2 * j + h] = __builtin_bit_cast(uint32_t, (ushortx2)(t + add));                           // v_pk_add_u16
-            }
-        lo = make_uint4(o[0], o[1], o[2], o[3]);
-        hi = make_uint4(o[4], o[5], o[6], o[7]);
-    }
     // 16 codes (one 128-bit word) of one block -> 16 bf16 (two 128-bit words), any code, any scale < 255
     __device__ inline void run16(const uint4& codes, uint4& lo, uint4& hi) const {
         const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
@@ -121,19 +84,11 @@ struct Composer {
         lo = make_uint4(o[0], o[1], o[2], o[3]);
         hi = make_uint4(o[4], o[5], o[6], o[7]);
     }
-    // Complete compose of one 16-code run.  Formats with a wide exponent field almost never hold
-    // zero-exponent codes (they are > 2^14 times smaller than the block maximum), so those take
-    // the cheap integer placement and only a wave that actually meets such a code, or an extreme
-    // scale, re-does its run through the general path.
+    // SAFE = false is for callers that know no scale in reach is 255 (checked once per tile)
+    template <bool SAFE>
     __device__ static inline void compose16(const uint4& codes, uint32_t scale, uint4& lo, uint4& hi) {
-        const Composer c(scale);
-        if (kHasIntPath) {
-            c.run16_int(codes, scale, lo, hi);
-            if (__builtin_amdgcn_ballot_w64(!covers16(codes, scale)) == 0) return;
-            if (covers16(codes, scale)) return;
-        }
-        c.run16(codes, lo, hi);
-        fix255(scale, codes, lo, hi);
+        Composer(scale).run16(codes, lo, hi);
+        if (SAFE) fix255(scale, codes, lo, hi);
     }
     // scale 255: the ldexp path gave 0 for zero codes where the reference has 0 * inf = NaN
     // (non-zero codes already overflowed to +-inf).  Rare: one wave-uniform branch per call.
@@ -295,7 +250,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         sw[p] = k_ok ? (w_scales + (size_t)ktc * (TK / 32))[ws_off[p]] : 0u;
     };
 
-    auto stage_part = [&](int p, int buf) {
+    auto stage_part = [&](auto safe, int p, int buf) {
+        constexpr bool SAFE = decltype(safe)::value;
         uint8_t* const pa = lds_a + buf * SLAB_BYTES;
         uint8_t* const pw = lds_w + buf * SLAB_BYTES;
         if (A_MODE == 0) {
@@ -306,13 +262,13 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
             }
         } else {
             uint4 lo, hi;
-            Composer<FA>::compose16(ra[p], sa[p], lo, hi);
+            Composer<FA>::template compose16<SAFE>(ra[p], sa[p], lo, hi);
             uint4* q = reinterpret_cast<uint4*>(pa + (p * 64 + c_row0) * ROW_BYTES + c_chunk * 32);
             q[0] = lo; q[1] = hi;
         }
         {
             uint4 lo, hi;
-            Composer<FW>::compose16(rw[p], sw[p], lo, hi);
+            Composer<FW>::template compose16<SAFE>(rw[p], sw[p], lo, hi);
             uint4* q = reinterpret_cast<uint4*>(pw + (p * 64 + c_row0) * ROW_BYTES + c_chunk * 32);
             q[0] = lo; q[1] = hi;
         }
@@ -354,15 +310,30 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         }
     };
 
+    // ---- does any scale this tile will read equal 255 (a block that held inf/NaN)?  Decided once per
+    //      tile so that the K loop itself carries no test: thread t scans the scale row of W row
+    //      n0 + t (and of A row m0 + t when A is MXFP).
+    bool saw255 = false;
+    {
+        const uint8_t* const wr = w_scales + (size_t)min(n0 + tid, N - 1) * kblocks;
+        for (int b = 0; b < kblocks; ++b) saw255 |= wr[b] == 255;
+        if (A_MODE == 1) {
+            const uint8_t* const ar = a_scales + (size_t)min(m0 + tid, M - 1) * kblocks;
+            for (int b = 0; b < kblocks; ++b) saw255 |= ar[b] == 255;
+        }
+    }
+    const bool tile_has_255 = __syncthreads_or(saw255) != 0;
+
+    auto run_tile = [&](auto safe) {
     // ---- prologue: slab 0 complete in LDS[0], part 0 of slab 1 in LDS[1]; registers hold parts
     //      1..3 of slab 1 and part 0 of slab 2
 #pragma unroll
     for (int p = 0; p < 4; ++p) fetch_part(p, 0);
 #pragma unroll
-    for (int p = 0; p < 4; ++p) stage_part(p, 0);
+    for (int p = 0; p < 4; ++p) stage_part(safe, p, 0);
 #pragma unroll
     for (int p = 0; p < 4; ++p) fetch_part(p, 1);
-    stage_part(0, 1);
+    stage_part(safe, 0, 1);
     fetch_part(0, 2);
     lds_barrier();
 
@@ -377,21 +348,21 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         const int cur = kt & 1, nxt = cur ^ 1;
         load_frags(cur, 1, fa1, fw1);
         mfma16(fa0, fw0);
-        stage_part(1, nxt);
+        stage_part(safe, 1, nxt);
         fetch_part(1, kt + 2);
         interleave();
         __builtin_amdgcn_sched_barrier(0);
 
         load_frags(cur, 2, fa0, fw0);
         mfma16(fa1, fw1);
-        stage_part(2, nxt);
+        stage_part(safe, 2, nxt);
         fetch_part(2, kt + 2);
         interleave();
         __builtin_amdgcn_sched_barrier(0);
 
         load_frags(cur, 3, fa1, fw1);
         mfma16(fa0, fw0);
-        stage_part(3, nxt);
+        stage_part(safe, 3, nxt);
         fetch_part(3, kt + 2);
         interleave();
         __builtin_amdgcn_sched_barrier(0);
@@ -400,11 +371,15 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 
         load_frags(nxt, 0, fa0, fw0);
         mfma16(fa1, fw1);
-        stage_part(0, cur);
+        stage_part(safe, 0, cur);
         fetch_part(0, kt + 3);
         interleave();
         __builtin_amdgcn_sched_barrier(0);
     }
+
+    };
+    if (tile_has_255) run_tile(IntC<1>{});
+    else run_tile(IntC<0>{});
 
     // ---- epilogue: lane holds, for tile (j, i) and g = 0..3, y[m][n .. n+3] with
     //      m = m0 + wave_m*128 + i*32 + lane%32,  n = n0 + wave_n*128 + j*32 + 8*g + 4*(lane/32)
@@ -490,10 +465,10 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
         {
             uint4 lo, hi;
             if (A_MODE == 0) { lo = ra0; hi = ra1; }
-            else Composer<FA>::compose16(ra0, sa, lo, hi);
+            else Composer<FA>::template compose16<true>(ra0, sa, lo, hi);
             uint4* pa = reinterpret_cast<uint4*>(&lds_a[srow * S_STRIDE + shalf * 16]);
             pa[0] = lo; pa[1] = hi;
-            Composer<FW>::compose16(rw, sw, lo, hi);
+            Composer<FW>::template compose16<true>(rw, sw, lo, hi);
             uint4* pw = reinterpret_cast<uint4*>(&lds_w[srow * S_STRIDE + shalf * 16]);
             pw[0] = lo; pw[1] = hi;
         }
