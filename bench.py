@@ -27,6 +27,10 @@ for p in (ROOT, os.path.join(ROOT, "mase-triton_amd"), os.path.join(ROOT, "tests
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+# HBM-side bytes per launch of the C4 GEMM kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch
+# 955385.2 and 1004869.6), scaled by what the same counters read for a plain 256 MiB copy (x2.000 and x1.000);
+# the summary with the commands is profiles/hbm_counters_gemm_c4_cast_c3.md.  Algorithmic bytes are 0.665e9.
+GEMM_C4_TRAFFIC_BYTES = int((955385.2 * 2.0 + 1004869.6 * 1.0) * 1024)
 
 
 def parse_args():
@@ -38,6 +42,9 @@ def parse_args():
     ap.add_argument("--skip-hbm", action="store_true", help="skip the cast-kernel bandwidth section")
     ap.add_argument("--only-gemm-kernel", action="store_true",
                     help="profiling aid: launch only the GEMM kernel in the timed loop")
+    ap.add_argument("--counter-probe", action="store_true",
+                    help="profiling aid for rocprofv3 --pmc: a plain 256 MiB device copy (calibration), then 3 launches "
+                         "each of the GEMM and of the C3 extract / compose kernels; prints nothing to time")
     return ap.parse_args()
 
 
@@ -102,20 +109,33 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
     }
 
 
-def time_kernel(torch, launch, n_variants, iters=50, warmup=10):
-    """Average launch duration with HIP events on the launch stream, rotating through
-    n_variants independent buffer sets so that consecutive launches do not hit the same lines."""
+def time_kernel(torch, launch, n_variants, iters=48, warmup=8, reps=5):
+    """Average duration of one launch: `iters` back-to-back launches, rotating through n_variants
+    independent buffer sets so that consecutive launches do not hit the same lines, are captured in
+    a HIP graph (removes the host's launch cost from the GPU timeline) and the replay is bracketed
+    by HIP events on the launch stream.  Returns (mean over replays, best replay) per launch in ms."""
     for i in range(warmup):
         launch(i % n_variants)
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    for i in range(iters):
-        ev[i][0].record()
-        launch(i % n_variants)
-        ev[i][1].record()
-    torch.cuda.synchronize()
-    ms = sorted(event_ms(ev))
-    return sum(ms) / len(ms), ms[len(ms) // 2]
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        launch(0)
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(iters):
+                launch(i % n_variants)
+        times = []
+        for _ in range(reps + 1):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            graph.replay()
+            e1.record(stream)
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1) / iters)
+    stream.synchronize()
+    times = times[1:]
+    return sum(times) / len(times), min(times)
 
 
 def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
@@ -128,7 +148,7 @@ def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
         gbs = bytes_per_launch / (avg_ms * 1e-3) / 1e9
         out.append({
             "kernel": name, "workload": workload, "bytes_per_launch": bytes_per_launch,
-            "avg_ms": round(avg_ms, 5), "median_ms": round(med_ms, 5),
+            "avg_ms": round(avg_ms, 5), "best_ms": round(med_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
             "cache_resident_GBps": round(bytes_per_launch / (cached_ms * 1e-3) / 1e9, 1),
@@ -145,23 +165,23 @@ def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
         # pre-allocated outputs so that the timed region holds only the kernel
         from mase_hip import _lib
         lib = _lib.load()
-        sp = _lib.stream_ptr(torch.device(dev))
+        sp_of = lambda: _lib.stream_ptr(torch.device(dev))
         sc_o = [torch.empty_like(c[0]) for c in comps]
         el_o = [torch.empty_like(c[1]) for c in comps]
         y_o = [torch.empty_like(x) for x in xs]
 
         def ext(i):
-            _lib.check(lib.mase_hip_extract_mxfp(xs[i].data_ptr(), 2, sc_o[i].data_ptr(), el_o[i].data_ptr(), n, 32, e, m, 1, 0, sp))
+            _lib.check(lib.mase_hip_extract_mxfp(xs[i].data_ptr(), 2, sc_o[i].data_ptr(), el_o[i].data_ptr(), n, 32, e, m, 1, 0, sp_of()))
 
         def cmp(i):
-            _lib.check(lib.mase_hip_compose_mxfp(comps[i][0].data_ptr(), comps[i][1].data_ptr(), y_o[i].data_ptr(), 2, n, 32, e, m, 1, sp))
+            _lib.check(lib.mase_hip_compose_mxfp(comps[i][0].data_ptr(), comps[i][1].data_ptr(), y_o[i].data_ptr(), 2, n, 32, e, m, 1, sp_of()))
 
         def both(i):
             ext(i)
             cmp(i)
 
         def qdq(i):
-            _lib.check(lib.mase_hip_qdq_mxfp(xs[i].data_ptr(), 2, y_o[i].data_ptr(), 2, n, 32, e, m, 1, 0, sp))
+            _lib.check(lib.mase_hip_qdq_mxfp(xs[i].data_ptr(), 2, y_o[i].data_ptr(), 2, n, 32, e, m, 1, 0, sp_of()))
 
         wl = f"{tag}: {rows}x{cols} bf16, E{e}M{m}, block 32"
         for name, fn, nbytes in (("extract_mxfp", ext, ext_bytes), ("compose_mxfp", cmp, cmp_bytes),
@@ -178,20 +198,20 @@ def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
     n = 1 << 24
     from mase_hip import _lib
     lib = _lib.load()
-    sp = _lib.stream_ptr(torch.device(dev))
+    sp_of = lambda: _lib.stream_ptr(torch.device(dev))
     gen = torch.Generator(device=dev).manual_seed(1)
     xs = [torch.randn(n, generator=gen, device=dev) for _ in range(6)]
     ys = [torch.empty_like(x) for x in xs]
     cs = [torch.empty(n, dtype=torch.uint16, device=dev) for _ in xs]
     for e, m in ((4, 3), (5, 2)):
         def qdq(i):
-            _lib.check(lib.mase_hip_qdq_minifloat(xs[i].data_ptr(), 0, ys[i].data_ptr(), 0, n, e, m, 1, 0, sp))
+            _lib.check(lib.mase_hip_qdq_minifloat(xs[i].data_ptr(), 0, ys[i].data_ptr(), 0, n, e, m, 1, 0, sp_of()))
 
         def ext(i):
-            _lib.check(lib.mase_hip_extract_minifloat(xs[i].data_ptr(), 0, cs[i].data_ptr(), n, e, m, 1, 0, sp))
+            _lib.check(lib.mase_hip_extract_minifloat(xs[i].data_ptr(), 0, cs[i].data_ptr(), n, e, m, 1, 0, sp_of()))
 
         def cmp(i):
-            _lib.check(lib.mase_hip_compose_minifloat(cs[i].data_ptr(), ys[i].data_ptr(), 0, n, e, m, 1, sp))
+            _lib.check(lib.mase_hip_compose_minifloat(cs[i].data_ptr(), ys[i].data_ptr(), 0, n, e, m, 1, sp_of()))
 
         wl = f"C2: 2^24 fp32, FP8 E{e}M{m}"
         for name, fn, nbytes in (("qdq_minifloat_fused", qdq, n * 8.0), ("extract_minifloat", ext, n * 6.0),
@@ -203,24 +223,55 @@ def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
 
 
 def cpu_baseline(torch):
-    """The reference's CPU path (dequantize everything with tensor ops, then F.linear) on a bounded
-    sample of the headline workload: 256 of the 16384 activation rows against the full weight."""
+    """The reference's CPU path (quantise x, dequantise x and W with tensor ops, then F.linear) on a
+    bounded sample of the headline workload: the first `rows` of the 16384 activation rows against
+    the full weight.  A probe with 512 rows sizes the sample to roughly 12 s of CPU work."""
     from oracle import torch_fake
 
-    rows, K, N = 256, 4096, 14336
+    K, N, M = 4096, 14336, 16384
     g = torch.Generator().manual_seed(3)
-    x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
     w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
     w_sc, w_el = torch_fake.mxfp_split(w, 32, 4, 3)
+    del w
     threads = torch.get_num_threads()
-    t0 = time.perf_counter()
-    y = torch_fake.mxfp_linear_xq_wq(x, w_sc, w_el, (N, K), torch.bfloat16, (4, 3), (4, 3))
-    t1 = time.perf_counter()
-    assert y.shape == (rows, N)
+
+    def run(rows):
+        x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
+        t0 = time.perf_counter()
+        y = torch_fake.mxfp_linear_xq_wq(x, w_sc, w_el, (N, K), torch.bfloat16, (4, 3), (4, 3))
+        dt = time.perf_counter() - t0
+        assert y.shape == (rows, N)
+        return dt
+
+    t_probe = run(512)
+    rows = int(min(M, max(512, 512 * (12.0 / max(t_probe, 1e-3)))) // 256 * 256)
+    dt = run(rows)
     flop = 2.0 * rows * N * K
-    return {"value": round(flop / (t1 - t0) / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"{rows} of 16384 activation rows x full W [14336,4096]: tensor-op restatement of the reference's "
-                      f"CPU path (quantise x, dequantise x and W, F.linear), {t1 - t0:.1f} s"}
+    return {"value": round(flop / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{rows} of {M} activation rows x full W [{N},{K}]: tensor-op restatement of the reference's CPU "
+                      f"path (quantise x, dequantise x and W, F.linear), {dt:.1f} s"}
+
+
+def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
+    """Few launches of each kernel next to a copy of known size, for hardware-counter runs."""
+    dev = "cuda:0"
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)                                   # reads 256 MiB, writes 256 MiB
+    M, K, N = 16384, 4096, 14336
+    gen = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
+    w_sc, w_el, _ = MXFP_F.extract_mxfp_components(w, block_dim=1, mxfp_meta=fmt8)
+    a = mxk.quantize_dequantize(x.view(-1), fmt8, torch.bfloat16).view(M, K)
+    for _ in range(3):
+        mxk.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt8, None, M, N, K, torch.bfloat16)
+    w1 = w.view(-1)
+    for _ in range(3):
+        sc, el = mxk.extract_mxfp_components(w1, fmt4)
+        mxk.compose_mxfp_tensor(sc, el, fmt4, torch.bfloat16)
+    torch.cuda.synchronize()
 
 
 def main():
@@ -241,6 +292,9 @@ def main():
     from mase_hip.mxfp.meta import MXFP8_E4M3_fn, MXFPMeta
 
     torch.cuda.set_device(0)
+    if args.counter_probe:
+        counter_probe(torch, MXFP_F, mxk, MXFP8_E4M3_fn, MXFPMeta(32, 8, 2, 1, True, "rn"))
+        return
     lin = bench_linear(args, torch, MXFP_F, mxk, MXFP8_E4M3_fn)
     M, N, K = lin["shape"]
     result = {
@@ -261,7 +315,7 @@ def main():
                                "fp32 accumulate; step = fused QDQ kernel + dequant-fused GEMM kernel",
                    "M": M, "N": N, "K": K},
         "roofline": {"bound": "mfma", "achieved": round(lin["tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": GEMM_C4_TRAFFIC_BYTES,
                      "kernel": "mxfp_gemm_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4)},
     }
     if not args.skip_hbm:
