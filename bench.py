@@ -28,8 +28,8 @@ for p in (ROOT, os.path.join(ROOT, "mase-triton_amd"), os.path.join(ROOT, "tests
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # HBM-side bytes per launch of the C4 GEMM kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch
-# 955385.2 and 1004869.6), scaled by what the same counters read for a plain 256 MiB copy (x2.000 and x1.000);
-# the summary with the commands is profiles/hbm_counters_gemm_c4_cast_c3.md.  Algorithmic bytes are 0.665e9.
+# 955385.2 and 1004869.6), scaled by what the same counters read for a plain 256 MiB copy (x2.000 and x1.000),
+# collected with `--counter-probe`.  Algorithmic bytes are 0.665e9.
 GEMM_C4_TRAFFIC_BYTES = int((955385.2 * 2.0 + 1004869.6 * 1.0) * 1024)
 
 
