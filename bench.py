@@ -316,7 +316,7 @@ def main():
                    "M": M, "N": N, "K": K},
         "roofline": {"bound": "mfma", "achieved": round(lin["tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": GEMM_C4_TRAFFIC_BYTES,
-                     "kernel": "mxfp_gemm_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4)},
+                     "kernel": "mxfp_gemm_tall_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4)},
     }
     if not args.skip_hbm:
         result["hbm_kernels"] = bench_hbm(

@@ -66,21 +66,23 @@ struct Composer {
         const float a = decode_f32((w >> (16 * p)) & 0xFFu, f) * s_wide, b = decode_f32((w >> (16 * p + 8)) & 0xFFu, f) * s_wide;
         return cvt_pk_bf16(a, b);
     }
+    // 4 codes (one dword) -> 4 bf16 (two dwords), any code, any scale < 255
+    __device__ inline void pair2(uint32_t w, uint32_t& o0, uint32_t& o1) const {
+        if (E >= 5) {
+            o0 = bf16_pair_wide(w, 0);
+            o1 = bf16_pair_wide(w, 1);
+        } else {
+            const uint32_t ws = w << PRE;  // top bits of every byte are zero: no spill between bytes
+            o0 = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x010C000Cu));
+            o1 = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x030C020Cu));
+        }
+    }
     // 16 codes (one 128-bit word) of one block -> 16 bf16 (two 128-bit words), any code, any scale < 255
     __device__ inline void run16(const uint4& codes, uint4& lo, uint4& hi) const {
         const uint32_t w[4] = {codes.x, codes.y, codes.z, codes.w};
         uint32_t o[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (E >= 5) {
-                o[2 * j] = bf16_pair_wide(w[j], 0);
-                o[2 * j + 1] = bf16_pair_wide(w[j], 1);
-            } else {
-                const uint32_t ws = w[j] << PRE;  // top bits of every byte are zero: no spill between bytes
-                o[2 * j] = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x010C000Cu));
-                o[2 * j + 1] = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x030C020Cu));
-            }
-        }
+        for (int j = 0; j < 4; ++j) pair2(w[j], o[2 * j], o[2 * j + 1]);
         lo = make_uint4(o[0], o[1], o[2], o[3]);
         hi = make_uint4(o[4], o[5], o[6], o[7]);
     }
@@ -406,6 +408,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     }  // tile loop
 }
 
+#include "gemm_tall.h"
+
 // ---------------------------------------------------------------------------------------------
 // Small-shape kernel: 128 x 128 x 32 tiles, single LDS buffer.  Used when the problem cannot
 // fill the chip with 256 x 256 tiles.
@@ -506,6 +510,20 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
         }
 }
 
+#ifndef TALL_MIN_TILES
+#define TALL_MIN_TILES 128
+#endif
+inline int device_cu_count() {
+    static int n_cus = 0;
+    if (n_cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
+        n_cus = prop.multiProcessorCount > 8 ? prop.multiProcessorCount : 8;
+    }
+    return n_cus;
+}
+
 template <int A_MODE, class FA, class FW, int DT_OUT>
 int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_elements, const uint8_t* w_scales,
                 const uint8_t* w_elements, const void* bias, int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
@@ -514,6 +532,27 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     // 256 x 256 tiles need enough of them to occupy the 256 CUs; smaller problems use 128 x 128
     const bool fits32 = (int64_t)M * K * 2 < ((int64_t)1 << 32) && (int64_t)N * K < ((int64_t)1 << 32);  // 32-bit operand offsets
     const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
+    if constexpr (A_MODE == 0 && DT_OUT != F32) {
+        // tall tiles: dense A, 16-bit output, no bias, whole tiles only, enough of them to occupy the chip
+        const int64_t tall_tiles = (int64_t)(M / UM) * (N / UN);
+        if (fits32 && bias == nullptr && M % UM == 0 && N % UN == 0 && K % (2 * UK) == 0 && K >= 4 * UK && tall_tiles >= TALL_MIN_TILES &&
+            (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
+            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
+            auto kern = mxfp_gemm_tall_kernel<FW, DT_OUT>;
+            static bool attr_done = false;
+            if (!attr_done) {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, U_LDS_BYTES);
+                if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
+                attr_done = true;
+            }
+            const int cus = device_cu_count();
+            if (cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
+            const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
+                               w_elements, y, M, N, K, M / UM, N / UN);
+            return check_launch("mxfp_gemm");
+        }
+    }
     if (use_big) {
         const bool guard_k = K % TK != 0;
         auto kern = guard_k ? mxfp_gemm_kernel<A_MODE, FA, FW, DT_OUT, true> : mxfp_gemm_kernel<A_MODE, FA, FW, DT_OUT, false>;
@@ -524,14 +563,8 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
             attr_set[guard_k] = true;
         }
-        static int n_cus = 0;
-        if (n_cus == 0) {
-            int dev = 0;
-            hipDeviceProp_t prop;
-            if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-                return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
-            n_cus = prop.multiProcessorCount > 8 ? prop.multiProcessorCount : 8;
-        }
+        const int n_cus = device_cu_count();
+        if (n_cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
         // one persistent workgroup per CU (rounded down to a multiple of 8 XCD slots), never more than tiles
         const int64_t want = big_tiles < n_cus ? ((big_tiles + 7) / 8) * 8 : (n_cus / 8) * 8;
         const unsigned grid = (unsigned)want;
