@@ -66,16 +66,18 @@ struct Composer {
         const float a = decode_f32((w >> (16 * p)) & 0xFFu, f) * s_wide, b = decode_f32((w >> (16 * p + 8)) & 0xFFu, f) * s_wide;
         return cvt_pk_bf16(a, b);
     }
-    // 4 codes (one dword) -> 4 bf16 (two dwords), any code, any scale < 255
+    // codes 0,1 (pair_lo) / 2,3 (pair_hi) of a dword of 4 codes -> 2 bf16, any code, any scale < 255
+    __device__ inline uint32_t pair_lo(uint32_t w) const {
+        if (E >= 5) return bf16_pair_wide(w, 0);
+        return bf16_pair(__builtin_amdgcn_perm(0u, w << PRE, 0x010C000Cu));  // top bits of every byte are zero: no spill between bytes
+    }
+    __device__ inline uint32_t pair_hi(uint32_t w) const {
+        if (E >= 5) return bf16_pair_wide(w, 1);
+        return bf16_pair(__builtin_amdgcn_perm(0u, w << PRE, 0x030C020Cu));
+    }
     __device__ inline void pair2(uint32_t w, uint32_t& o0, uint32_t& o1) const {
-        if (E >= 5) {
-            o0 = bf16_pair_wide(w, 0);
-            o1 = bf16_pair_wide(w, 1);
-        } else {
-            const uint32_t ws = w << PRE;  // top bits of every byte are zero: no spill between bytes
-            o0 = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x010C000Cu));
-            o1 = bf16_pair(__builtin_amdgcn_perm(0u, ws, 0x030C020Cu));
-        }
+        o0 = pair_lo(w);
+        o1 = pair_hi(w);
     }
     // 16 codes (one 128-bit word) of one block -> 16 bf16 (two 128-bit words), any code, any scale < 255
     __device__ inline void run16(const uint4& codes, uint4& lo, uint4& hi) const {
@@ -535,9 +537,9 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     if constexpr (A_MODE == 0 && DT_OUT != F32) {
         // tall tiles: dense A, 16-bit output, no bias, whole tiles only, enough of them to occupy the chip
         const int64_t tall_tiles = (int64_t)(M / UM) * (N / UN);
-        if (fits32 && bias == nullptr && M % UM == 0 && N % UN == 0 && K % (2 * UK) == 0 && K >= 4 * UK && tall_tiles >= TALL_MIN_TILES &&
+        if (fits32 && bias == nullptr && M % UM == 0 && N % UN == 0 && K % UMAC == 0 && tall_tiles >= TALL_MIN_TILES &&
             (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
-            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
+            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0) {
             auto kern = mxfp_gemm_tall_kernel<FW, DT_OUT>;
             static bool attr_done = false;
             if (!attr_done) {

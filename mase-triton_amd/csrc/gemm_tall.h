@@ -1,52 +1,67 @@
-// Tall-tile MXFP GEMM kernel for gfx950: 512 (M) x 128 (N) x 32 (K) tiles, dense bf16 A, 16-bit output, no bias.
+// Tall-tile MXFP GEMM kernel for gfx950: 512 (M) x 128 (N) tiles, dense bf16 A, 16-bit output, no bias.
 //
 // Why this shape.  One wavefront can issue only about three other instructions per 32-cycle
 // 32x32x16 MFMA without slowing the matrix pipe, so the K loop has to be lean:
-//   * the dense A slab goes from global memory straight into LDS (global_load_lds_dwordx4, no
-//     VGPRs, no ds_write), four slabs deep;
+//   * the dense A operand goes from global memory straight into LDS (global_load_lds_dwordx4, no
+//     VGPRs, no ds_write), always as whole 128-byte lines: a CU's vector memory path moves about
+//     2.5 cycles per cache line an instruction touches, whatever part of the line is used, so
+//     64-byte row pieces would halve its rate;
 //   * the MXFP weight slab is composed to bf16 once per 512 output rows instead of once per 256;
-//   * all global traffic is issued by hand (inline asm) three K-steps ahead and waited for with
-//     one s_waitcnt per step, so the compiler inserts no conservative waits of its own;
-//   * every step is laid out by hand in 16 slots of two MFMAs each, the other work spread over
+//   * all global traffic is issued by hand (inline asm) and waited for with explicit s_waitcnt
+//     counts, so the compiler inserts no conservative waits of its own;
+//   * every K step is laid out by hand in 16 slots of two MFMAs each, the other work spread over
 //     them one vector-memory instruction at a time (a burst of them stalls the issuing wave for
 //     as long as the address unit needs to drain it).
 // Four wavefronts stacked along M, each 128 x 128 (4 x 4 MFMA tiles, 256 accumulator AGPRs).  A wave
 // only ever reads the 128 A rows it loaded itself; the 128-row W slab is shared by all four.
 //
-// A workgroup walks its tiles as ONE stream of K steps: the last three steps of a tile already
-// fetch the first three slabs of the next one, the output tile is converted and stored between two
-// steps, and its stores drain while the next tile is being multiplied.  Vector-memory operations
-// complete in issue order, so a wait only has to let the younger ones stay outstanding.
+// A workgroup walks its tiles as ONE stream of macro steps of 128 k (four K steps of 32): the last
+// macro step of a tile already fetches the first operands of the next one, the output tile is
+// converted and stored between two steps, and its stores drain while the next tile is being
+// multiplied.  Vector-memory operations complete in issue order, so a wait only has to let the
+// younger ones stay outstanding.
 //
-// LDS (160 KB): A stages [4][4 waves][128 rows][64 B], W stages [2][128 rows][64 B], and 4 KB per
-// wave to turn the accumulator layout into whole 128-byte output lines.  Rows of 64 bytes carry no
-// padding (the DMA writes 1 KB contiguous per instruction); the 16-byte chunk c of row r is kept
-// at position c ^ ((r >> 2) & 3), which makes the 128-bit fragment reads of 16 consecutive rows
-// hit 16 distinct bank groups.
+// LDS (160 KB):
+//   A   [2 stages][4 waves][128 rows][128 B]  stage d holds k 64d .. 64d+63 of the macro step; the
+//       16-byte chunk c of row r sits at position c ^ (r & 7) (conflict-free 128-bit fragment reads)
+//   W   [2 stages][128 rows][64 B]            composed bf16 of one K step, chunk c at c ^ ((r >> 2) & 3)
+//   out [4 waves][32 rows][128 B]             turns the accumulator layout into whole output lines
 //
-// Step kt (slab kt is being multiplied; A slab s -> stage s % 4 counted over the whole stream,
-// W slab s -> stage s % 2, its raw codes in register set s % 2):
-//   top         s_waitcnt: slab kt+1 has landed (W codes in registers, A rows in LDS)
-//   slots 0-7   MFMAs on k 0..15 of slab kt | read fragments k 16..31 of slab kt | compose W slab
-//               kt+1 into its stage | issue the W loads and the first A DMAs of slab kt+3
-//   barrier
-//   slots 8-15  MFMAs on k 16..31 | read fragments k 0..15 of slab kt+1 | remaining A DMAs
+// Macro step m, K step S = 0..3 (slab 4m+S is multiplied; A stage S/2; W stage S%2):
+//   slots 0-7   MFMAs k 0..15 | read fragments k 16..31 of slab S (slots 0-3) | compose W slab S+1, two codes a slot
+//   slot  8     write composed W slab S+1 to its stage
+//   slots 8-9   read the A fragments k 0..15 of slab S+1;  barrier after slot 9;  slots 10-11 the W fragments
+//   slots 8-15  MFMAs k 16..31
+// Global traffic of macro step m (per wave), in issue order:
+//   S=0 slots 0-3    A stage 1 of m   (last 4 of 16 DMAs; the first 12 were issued in S=3 of m-1)
+//   S=0 slot 6       W codes (4 x 16 B per thread) and scales (4 bytes) of macro step m+1
+//   S=1 slots 4-15   A stage 0 of m+1 (first 12)      [stage 0 was last read in S=1 slots 0-3]
+//   S=2 slots 0-3    A stage 0 of m+1 (last 4)
+//   S=3 slots 4-15   A stage 1 of m+1 (first 12)      [stage 1 was last read in S=3 slots 0-3]
+// Waits: S=1 slot 8 needs A stage 1 of m (9 younger operations); top of S=3 needs the W registers
+// of m+1 (16 younger); S=3 slot 8 needs A stage 0 of m+1 (4 younger).
 // (included from gemm_impl.h, inside namespace mase, after the shared helpers)
 
 constexpr int UM = 512, UN = 128, UK = 32;
-constexpr int U_A_STAGES = 4, U_W_STAGES = 2;
-constexpr int U_A_STAGE_BYTES = UM * UK * 2;  // 32 KB
-constexpr int U_W_STAGE_BYTES = UN * UK * 2;  // 8 KB
-constexpr int U_OUT_WAVE_BYTES = 32 * 128;    // 32 rows x 64 outputs of 2 bytes
+constexpr int UMAC = 128;                         // k per macro step: four K steps, one 128-byte line of W codes, two of A
+constexpr int U_A_STAGES = 2, U_W_STAGES = 2;
+constexpr int U_A_STAGE_BYTES = UM * 64 * 2;      // 64 KB: 512 rows x 64 k
+constexpr int U_A_WAVE_BYTES = 128 * 128;         // one wave's 128 rows of a stage
+constexpr int U_W_STAGE_BYTES = UN * UK * 2;      // 8 KB: 128 rows x 32 k, composed
+constexpr int U_OUT_WAVE_BYTES = 32 * 128;        // 32 rows x 64 outputs of 2 bytes
 constexpr int U_LDS_BYTES = U_A_STAGES * U_A_STAGE_BYTES + U_W_STAGES * U_W_STAGE_BYTES + 4 * U_OUT_WAVE_BYTES;  // 160 KB
-constexpr int U_VMEM_PER_STEP = 10;    // 1 code load + 1 scale load + 8 DMAs per wave
-constexpr int U_STORES_PER_TILE = 32;  // 16-byte output stores per lane and tile
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // 64 lanes x 16 bytes from per-lane global addresses (sbase + voff) to LDS [lds_addr, lds_addr + 1024)
 __device__ inline void dma_1kb(uint32_t lds_addr, uint32_t voff, const void* sbase) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+}
+// the same with M0 left as the previous dma_1kb_set_m0 / dma_1kb set it: LDS [m0 + OFF, m0 + OFF + 1024) from
+// (sbase + voff + OFF); the immediate offset counts on both sides, so the caller pre-subtracts it from voff
+template <int OFF>
+__device__ inline void dma_1kb_keep_m0(uint32_t voff, const void* sbase) {
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(voff), "s"(sbase), "n"(OFF) : "memory");
 }
 __device__ inline void async_load16(u32x4& dst, uint32_t voff, const void* sbase) {
     asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
@@ -104,33 +119,38 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
     void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    const uint32_t lds_a = (uint32_t)(uintptr_t)lds;
-    uint8_t* const lds_w_ptr = lds + U_A_STAGES * U_A_STAGE_BYTES;
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kblocks = K / 32, ksteps = K / UK;  // the launcher guarantees an even ksteps >= 4
+    const int kblocks = K / 32, nmac = K / UMAC;  // the launcher guarantees K % 128 == 0
+    const uint32_t lds_aw = (uint32_t)(uintptr_t)lds + (uint32_t)wave * U_A_WAVE_BYTES;  // this wave's rows of stage 0
+    uint8_t* const lds_a_ptr = lds + wave * U_A_WAVE_BYTES;
+    uint8_t* const lds_w_ptr = lds + U_A_STAGES * U_A_STAGE_BYTES;
     uint8_t* const lds_out = lds_w_ptr + U_W_STAGES * U_W_STAGE_BYTES + wave * U_OUT_WAVE_BYTES;
 
     // ---- per-lane constants
-    // A DMA: instruction i of a wave covers its rows 16i .. 16i+15; lane l fills position l & 3 of row
-    // 16i + (l >> 2), which must hold chunk (l & 3) ^ (row >> 2 & 3) = (l & 3) ^ (l >> 4 & 3)
-    uint32_t a_voff[8];
+    // A DMA: instruction i of a wave covers its rows 8i .. 8i+7; lane l fills position l & 7 of row
+    // 8i + (l >> 3), which must hold chunk (l & 7) ^ (row & 7) = (l & 7) ^ (l >> 3)
+    uint32_t a_voff[16];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        a_voff[i] = (uint32_t)(16 * i + (lane >> 2)) * (uint32_t)K * 2u + (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);
-    // W staging: thread t owns codes [16 h, 16 h + 16) of row t >> 1, h = t & 1
+    for (int i = 0; i < 16; ++i)
+        a_voff[i] = (uint32_t)(8 * i + (lane >> 3)) * (uint32_t)K * 2u + (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16) -
+                    (uint32_t)((i & 3) * 1024);  // DMAs 4q+1 .. 4q+3 reuse the M0 of DMA 4q and add an immediate instead
+    // A fragment reads: lane (g = l >> 5, r = l & 31) reads chunk 2qq + g of row 32 t + r, qq = k / 16 within the stage
+    uint32_t fa_off[4];
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) fa_off[qq] = (uint32_t)(lane & 31) * 128u + (uint32_t)(((2 * qq + (lane >> 5)) ^ (lane & 7)) * 16);
+    // W staging: thread t owns codes [16 h, 16 h + 16) of row t >> 1 in every K step, h = t & 1
     const int w_row = tid >> 1, w_half = tid & 1;
     const uint32_t w_voff = (uint32_t)w_row * (uint32_t)K + (uint32_t)w_half * 16u;
     const uint32_t ws_voff = (uint32_t)w_row * (uint32_t)kblocks;
     const uint32_t w_swz = (uint32_t)((w_row >> 2) & 3);
     const uint32_t w_lds_off0 = (uint32_t)w_row * 64u + (((2u * w_half) ^ w_swz) * 16u);
     const uint32_t w_lds_off1 = (uint32_t)w_row * 64u + (((2u * w_half + 1u) ^ w_swz) * 16u);
-    // fragment reads: lane (g = l >> 5, r = l & 31) reads chunk 2q + g of row 32 t + r
+    // W fragment reads: lane (g, r) reads chunk 2q + g of row 32 t + r
     const uint32_t f_swz = (uint32_t)((lane >> 2) & 3);
-    const uint32_t f_row = (uint32_t)(lane & 31) * 64u;
-    const uint32_t f_off_q0 = f_row + ((((uint32_t)(lane >> 5)) ^ f_swz) * 16u);
-    const uint32_t f_off_q1 = f_row + (((2u + (uint32_t)(lane >> 5)) ^ f_swz) * 16u);
+    const uint32_t fw_off_q0 = (uint32_t)(lane & 31) * 64u + ((((uint32_t)(lane >> 5)) ^ f_swz) * 16u);
+    const uint32_t fw_off_q1 = (uint32_t)(lane & 31) * 64u + (((2u + (uint32_t)(lane >> 5)) ^ f_swz) * 16u);
+
     const int n_tiles = tiles_m * tiles_n;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int slots = gridDim.x >> 3;
@@ -155,27 +175,32 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     int local = blockIdx.x >> 3;
     if (!has_tile(local)) return;
     TallTile cur = tile_at(local), next = cur;
-    int gbase = 0;  // stream number of the current tile's slab 0 (mod 4 is all that matters)
 
-    u32x4 rw[2];
-    uint32_t sw[2];
-    // W codes + scale of `slab` of tile `t` into register set `set`
-    auto issue_w = [&](const TallTile& t, int slab, auto set_c) {
-        constexpr int set = decltype(set_c)::value;
-        async_load16(rw[set], w_voff, t.w + (size_t)slab * UK);
-        async_load_u8(sw[set], ws_voff, t.ws + slab);
+    // raw W codes and scales: `wc` serves K steps 1..3 of the current macro step (index = step), `wn` is the
+    // landing area of the next macro step's (its step 0 is composed during step 3 of the current one)
+    u32x4 wc[4], wn[4];
+    uint32_t sc, sn;
+    auto issue_w_codes = [&](const uint8_t* w_src, auto q_c) {
+        constexpr int q = decltype(q_c)::value;
+        async_load16(wn[q], w_voff, w_src + q * 32);
     };
-    // DMA i (rows 16i .. 16i+15 of the wave) of the slab at `src` into the stage at `dst`
-    auto issue_a = [&](const uint8_t* src, uint32_t dst, int i) { dma_1kb(dst + i * 1024, a_voff[i], src); };
-    auto a_src_of = [&](const TallTile& t, int slab) { return t.a + (size_t)slab * (UK * 2); };
-    auto a_dst_of = [&](int stream_slab) {
-        return lds_a + (uint32_t)(stream_slab & (U_A_STAGES - 1)) * U_A_STAGE_BYTES + (uint32_t)wave * (128 * 64);
+    auto issue_w_scales = [&](const uint8_t* ws_src) {
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(sn) : "v"(ws_voff), "s"(ws_src) : "memory");
     };
-    auto compose_all = [&](int w_stage, auto set_c) {
-        constexpr int set = decltype(set_c)::value;
+    auto issue_w = [&](const uint8_t* w_src, const uint8_t* ws_src) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) async_load16(wn[q], w_voff, w_src + q * 32);
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(sn) : "v"(ws_voff), "s"(ws_src) : "memory");
+    };
+    // DMA i (rows 8i .. 8i+7 of the wave) of the 64-k half at `src` into stage `stage`
+    auto issue_a = [&](const uint8_t* src, int stage, auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        if (i % 4 == 0) dma_1kb(lds_aw + (uint32_t)stage * U_A_STAGE_BYTES + (uint32_t)i * 1024u, a_voff[i], src);
+        else dma_1kb_keep_m0<(i % 4) * 1024>(a_voff[i], src);
+    };
+    auto compose_to = [&](const u32x4& codes, uint32_t scale, int w_stage) {
         uint4 lo, hi;
-        const uint4 codes = make_uint4(rw[set].x, rw[set].y, rw[set].z, rw[set].w);
-        Composer<FW>::template compose16<true>(codes, sw[set], lo, hi);
+        Composer<FW>::template compose16<true>(make_uint4(codes.x, codes.y, codes.z, codes.w), scale, lo, hi);
         uint8_t* const st = lds_w_ptr + w_stage * U_W_STAGE_BYTES;
         *reinterpret_cast<uint4*>(st + w_lds_off0) = lo;
         *reinterpret_cast<uint4*>(st + w_lds_off1) = hi;
@@ -184,54 +209,55 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     floatx16 acc[4][4];  // [n-tile j][m-tile i]
     bf16x8 fa0[4], fw0[4], fa1[4], fw1[4];
 
-    // ---- prologue of the stream: slabs 0..2 of the first tile landed, W slab 0 composed,
-    //      fragments k 0..15 of slab 0 in registers
+    // ---- prologue of the stream: what a macro step expects to find: A stage 0 landed, the first 12 DMAs
+    //      of A stage 1 issued, W slab 0 composed, wc = the macro step's codes, fragments k 0..15 of slab 0
     {
-        issue_w(cur, 0, IntC<0>{});
-#pragma unroll
-        for (int i = 0; i < 8; ++i) issue_a(a_src_of(cur, 0), a_dst_of(0), i);
-        issue_w(cur, 1, IntC<1>{});
-#pragma unroll
-        for (int i = 0; i < 8; ++i) issue_a(a_src_of(cur, 1), a_dst_of(1), i);
-        wait_vmcnt<U_VMEM_PER_STEP>(rw[0], sw[0]);
-        compose_all(0, IntC<0>{});
-        issue_w(cur, 2, IntC<0>{});
-#pragma unroll
-        for (int i = 0; i < 8; ++i) issue_a(a_src_of(cur, 2), a_dst_of(2), i);
-        wait_vmcnt<0>(rw[1], sw[1]);
-        wait_vmcnt<0>(rw[0], sw[0]);
+        issue_w(cur.w, cur.ws);
+        static_for<16>([&](auto i_c) { issue_a(cur.a, 0, i_c); });
+        wait_vmcnt<0>(wn[0], sn);
+        wait_vmcnt<0>(wn[1], sn);
+        wait_vmcnt<0>(wn[2], sn);
+        wait_vmcnt<0>(wn[3], sn);
+        static_for<6>([&](auto i_c) { issue_a(cur.a + 128, 1, i_c); });
+        compose_to(wn[0], sn & 0xFFu, 0);
+        wc[1] = wn[1];
+        wc[2] = wn[2];
+        wc[3] = wn[3];
+        sc = sn;
         lds_barrier();
-        const uint8_t* const pa = lds + wave * (128 * 64) + f_off_q0;
-        const uint8_t* const pw = lds_w_ptr + f_off_q0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) fa0[i] = *reinterpret_cast<const bf16x8*>(pa + i * 2048);
+        for (int i = 0; i < 4; ++i) fa0[i] = *reinterpret_cast<const bf16x8*>(lds_a_ptr + fa_off[0] + i * 4096);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) fw0[j] = *reinterpret_cast<const bf16x8*>(pw + j * 2048);
+        for (int j = 0; j < 4; ++j) fw0[j] = *reinterpret_cast<const bf16x8*>(lds_w_ptr + fw_off_q0 + j * 2048);
     }
 
-    // one K step; FIRST: the accumulators start from zero; WAITN: operations younger than slab kt+1
-    auto step = [&](auto first_c, auto set_c, auto wait_c, int kt) {
+    // pointers of the macro step in flight: a1_cur = second 64-k half of the current macro step; *_nxt = the
+    // next macro step (of this tile or, past its end, of the next one)
+    const uint8_t *a1_cur, *a0_nxt, *a1_nxt, *w_nxt, *ws_nxt;
+
+    // K step S of a macro step; FIRST: the accumulators start from zero
+    auto step = [&](auto s_c, auto first_c) {
+        constexpr int S = decltype(s_c)::value;
         constexpr bool FIRST = decltype(first_c)::value != 0;
-        constexpr int set = decltype(set_c)::value;  // (kt + 1) & 1
-        constexpr int WAITN = decltype(wait_c)::value;
-        wait_vmcnt<WAITN>(rw[set], sw[set]);
+        constexpr int WST_NOW = S & 1, WST_NEXT = (S + 1) & 1;
+        constexpr int AST_NOW = S >> 1, QQ1 = 2 * (S & 1) + 1;                      // fragments k 16..31 of slab S
+        constexpr int AST_NEXT = ((S + 1) >> 1) & 1, QQ0 = 2 * ((S + 1) & 1);        // fragments k 0..15 of slab S+1
+        const uint8_t* const pa1 = lds_a_ptr + AST_NOW * U_A_STAGE_BYTES + fa_off[QQ1];
+        const uint8_t* const pw1 = lds_w_ptr + WST_NOW * U_W_STAGE_BYTES + fw_off_q1;
+        const uint8_t* const pa0 = lds_a_ptr + AST_NEXT * U_A_STAGE_BYTES + fa_off[QQ0];
+        const uint8_t* const pw0 = lds_w_ptr + WST_NEXT * U_W_STAGE_BYTES + fw_off_q0;
+        uint8_t* const wst = lds_w_ptr + WST_NEXT * U_W_STAGE_BYTES;
 
-        const int s_now = gbase + kt;
-        const uint8_t* const pa1 = lds + (s_now & 3) * U_A_STAGE_BYTES + wave * (128 * 64) + f_off_q1;
-        const uint8_t* const pw1 = lds_w_ptr + (set ^ 1) * U_W_STAGE_BYTES + f_off_q1;
-        const uint8_t* const pa0 = lds + ((s_now + 1) & 3) * U_A_STAGE_BYTES + wave * (128 * 64) + f_off_q0;
-        const uint8_t* const pw0 = lds_w_ptr + set * U_W_STAGE_BYTES + f_off_q0;
-        uint8_t* const wst = lds_w_ptr + set * U_W_STAGE_BYTES;
-        int s3 = kt + 3;
-        const bool wrap = s3 >= ksteps;
-        if (wrap) s3 -= ksteps;
-        const uint8_t* const a_src = (wrap ? next.a : cur.a) + (size_t)s3 * (UK * 2);
-        const uint8_t* const w_src = (wrap ? next.w : cur.w) + (size_t)s3 * UK;
-        const uint8_t* const ws_src = (wrap ? next.ws : cur.ws) + s3;
-        const uint32_t a_dst = a_dst_of(s_now + 3);
-
-        const Composer<FW> cmp(sw[set]);
-        const uint32_t cw[4] = {rw[set].x, rw[set].y, rw[set].z, rw[set].w};
+        if (S == 3) {  // the next macro step's codes and scales are about to be composed / copied
+            wait_vmcnt<17>(wn[0], sn);
+            wait_vmcnt<17>(wn[1], sn);
+            wait_vmcnt<17>(wn[2], sn);
+            wait_vmcnt<17>(wn[3], sn);
+        }
+        const u32x4& codes = S == 3 ? wn[0] : wc[(S + 1) & 3];
+        const uint32_t scale = S == 3 ? (sn & 0xFFu) : ((sc >> (8 * ((S + 1) & 3))) & 0xFFu);
+        const Composer<FW> cmp(scale);
+        const uint32_t cw[4] = {codes.x, codes.y, codes.z, codes.w};
         uint32_t o[8];
 
         auto mm = [&](const bf16x8(&af)[4], const bf16x8(&wf)[4], int j, int i, bool zero) {
@@ -244,112 +270,156 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
                 acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], af[i], acc[j][i], 0, 0, 0);
             }
         };
+        // the global traffic of slot `slot` of this step
+        auto vmem = [&](auto slot_c) {
+            constexpr int slot = decltype(slot_c)::value;
+            // A: one DMA every second slot.  Stage 0 (of the next macro step): S1 slots 4..14, S2, S3 slots 0..2;
+            // stage 1: S3 slots 4..14, S0 of the next macro step, S1 slots 0..2
+            if constexpr (slot % 2 == 0) {
+                constexpr int h = slot / 2;
+                if constexpr (S == 3 && h >= 2) issue_a(a1_nxt, 1, IntC<h - 2>{});
+                if constexpr (S == 0) issue_a(a1_cur, 1, IntC<6 + h>{});
+                if constexpr (S == 1 && h < 2) issue_a(a1_cur, 1, IntC<14 + h>{});
+                if constexpr (S == 1 && h >= 2) issue_a(a0_nxt, 0, IntC<h - 2>{});
+                if constexpr (S == 2) issue_a(a0_nxt, 0, IntC<6 + h>{});
+                if constexpr (S == 3 && h < 2) issue_a(a0_nxt, 0, IntC<14 + h>{});
+            }
+            // W codes and scales of the next macro step: S0, odd slots 5..13
+            if constexpr (S == 0 && slot >= 5 && slot <= 11 && slot % 2 == 1) issue_w_codes(w_nxt, IntC<(slot - 5) / 2>{});
+            if constexpr (S == 0 && slot == 13) issue_w_scales(ws_nxt);
+        };
+        auto mm2 = [&](auto slot_c) {
+            constexpr int slot = decltype(slot_c)::value, k = slot & 7, j = k >> 1, i = 2 * (k & 1);
+            if (slot < 8) {
+                mm(fa0, fw0, j, i, FIRST);
+                mm(fa0, fw0, j, i + 1, FIRST);
+            } else {
+                mm(fa1, fw1, j, i, false);
+                mm(fa1, fw1, j, i + 1, false);
+            }
+        };
 #define U_SLOT_END() __builtin_amdgcn_sched_barrier(0)
-        // ---- slots 0..7: k 0..15
+        // ---- slots 0..7: MFMAs k 0..15; fragments k 16..31 of this slab; one pair of the next W slab per slot
+        auto pair_at = [&](auto k_c) {
+            constexpr int k = decltype(k_c)::value;
+            if (k & 1) o[k] = cmp.pair_hi(cw[k >> 1]);
+            else o[k] = cmp.pair_lo(cw[k >> 1]);
+        };
         fa1[0] = *reinterpret_cast<const bf16x8*>(pa1);
-        fa1[1] = *reinterpret_cast<const bf16x8*>(pa1 + 2048);
-        cmp.pair2(cw[0], o[0], o[1]);
-        mm(fa0, fw0, 0, 0, FIRST);
-        mm(fa0, fw0, 0, 1, FIRST);
+        fa1[1] = *reinterpret_cast<const bf16x8*>(pa1 + 4096);
+        pair_at(IntC<0>{});
+        vmem(IntC<0>{});
+        mm2(IntC<0>{});
         U_SLOT_END();
-        fa1[2] = *reinterpret_cast<const bf16x8*>(pa1 + 4096);
-        fa1[3] = *reinterpret_cast<const bf16x8*>(pa1 + 6144);
-        cmp.pair2(cw[1], o[2], o[3]);
-        mm(fa0, fw0, 0, 2, FIRST);
-        mm(fa0, fw0, 0, 3, FIRST);
+        fa1[2] = *reinterpret_cast<const bf16x8*>(pa1 + 8192);
+        fa1[3] = *reinterpret_cast<const bf16x8*>(pa1 + 12288);
+        pair_at(IntC<1>{});
+        vmem(IntC<1>{});
+        mm2(IntC<1>{});
         U_SLOT_END();
         fw1[0] = *reinterpret_cast<const bf16x8*>(pw1);
         fw1[1] = *reinterpret_cast<const bf16x8*>(pw1 + 2048);
-        cmp.pair2(cw[2], o[4], o[5]);
-        mm(fa0, fw0, 1, 0, FIRST);
-        mm(fa0, fw0, 1, 1, FIRST);
+        pair_at(IntC<2>{});
+        vmem(IntC<2>{});
+        mm2(IntC<2>{});
         U_SLOT_END();
         fw1[2] = *reinterpret_cast<const bf16x8*>(pw1 + 4096);
         fw1[3] = *reinterpret_cast<const bf16x8*>(pw1 + 6144);
-        cmp.pair2(cw[3], o[6], o[7]);
-        mm(fa0, fw0, 1, 2, FIRST);
-        mm(fa0, fw0, 1, 3, FIRST);
+        pair_at(IntC<3>{});
+        vmem(IntC<3>{});
+        mm2(IntC<3>{});
         U_SLOT_END();
+        // in steps 1 and 3 the A stage read in slots 0..3 is handed back to the DMA engine from slot 4 on; its
+        // writes must not pass those reads
+        if (S & 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        pair_at(IntC<4>{});
+        vmem(IntC<4>{});
+        mm2(IntC<4>{});
+        U_SLOT_END();
+        pair_at(IntC<5>{});
+        vmem(IntC<5>{});
+        mm2(IntC<5>{});
+        U_SLOT_END();
+        pair_at(IntC<6>{});
+        vmem(IntC<6>{});
+        mm2(IntC<6>{});
+        U_SLOT_END();
+        pair_at(IntC<7>{});
+        vmem(IntC<7>{});
+        mm2(IntC<7>{});
+        U_SLOT_END();
+        // ---- slots 8..15: MFMAs k 16..31; the composed slab goes to LDS; fragments k 0..15 of the next slab
         {
             uint4 lo = make_uint4(o[0], o[1], o[2], o[3]), hi = make_uint4(o[4], o[5], o[6], o[7]);
-            Composer<FW>::fix255(sw[set], make_uint4(cw[0], cw[1], cw[2], cw[3]), lo, hi);
+            Composer<FW>::fix255(scale, make_uint4(cw[0], cw[1], cw[2], cw[3]), lo, hi);
             *reinterpret_cast<uint4*>(wst + w_lds_off0) = lo;
             *reinterpret_cast<uint4*>(wst + w_lds_off1) = hi;
         }
+        if (S == 3) {
+            wc[1] = wn[1];
+            wc[2] = wn[2];
+            wc[3] = wn[3];
+            sc = sn;
+        }
+        vmem(IntC<8>{});
+        mm2(IntC<8>{});
         U_SLOT_END();
-        async_load16(rw[set], w_voff, w_src);  // the set's old contents were consumed above
-        async_load_u8(sw[set], ws_voff, ws_src);
-        mm(fa0, fw0, 2, 0, FIRST);
-        mm(fa0, fw0, 2, 1, FIRST);
+        vmem(IntC<9>{});
+        mm2(IntC<9>{});
         U_SLOT_END();
-        issue_a(a_src, a_dst, 0);
-        mm(fa0, fw0, 2, 2, FIRST);
-        mm(fa0, fw0, 2, 3, FIRST);
-        U_SLOT_END();
-        issue_a(a_src, a_dst, 1);
-        mm(fa0, fw0, 3, 0, FIRST);
-        mm(fa0, fw0, 3, 1, FIRST);
-        U_SLOT_END();
-        issue_a(a_src, a_dst, 2);
-        mm(fa0, fw0, 3, 2, FIRST);
-        mm(fa0, fw0, 3, 3, FIRST);
-        U_SLOT_END();
-        lds_barrier();  // every wave's part of W slab kt+1 is in LDS; W slab kt is no longer read
-        U_SLOT_END();
-        // ---- slots 8..15: k 16..31
-        fa0[0] = *reinterpret_cast<const bf16x8*>(pa0);
-        fa0[1] = *reinterpret_cast<const bf16x8*>(pa0 + 2048);
-        issue_a(a_src, a_dst, 3);
-        mm(fa1, fw1, 0, 0, false);
-        mm(fa1, fw1, 0, 1, false);
-        U_SLOT_END();
-        fa0[2] = *reinterpret_cast<const bf16x8*>(pa0 + 4096);
-        fa0[3] = *reinterpret_cast<const bf16x8*>(pa0 + 6144);
-        issue_a(a_src, a_dst, 4);
-        mm(fa1, fw1, 0, 2, false);
-        mm(fa1, fw1, 0, 3, false);
+        lds_barrier();  // every wave's part of W slab S+1 is in LDS; W slab S is no longer read
         U_SLOT_END();
         fw0[0] = *reinterpret_cast<const bf16x8*>(pw0);
         fw0[1] = *reinterpret_cast<const bf16x8*>(pw0 + 2048);
-        issue_a(a_src, a_dst, 5);
-        mm(fa1, fw1, 1, 0, false);
-        mm(fa1, fw1, 1, 1, false);
+        vmem(IntC<10>{});
+        mm2(IntC<10>{});
         U_SLOT_END();
         fw0[2] = *reinterpret_cast<const bf16x8*>(pw0 + 4096);
         fw0[3] = *reinterpret_cast<const bf16x8*>(pw0 + 6144);
-        issue_a(a_src, a_dst, 6);
-        mm(fa1, fw1, 1, 2, false);
-        mm(fa1, fw1, 1, 3, false);
+        vmem(IntC<11>{});
+        mm2(IntC<11>{});
         U_SLOT_END();
-        issue_a(a_src, a_dst, 7);
-        mm(fa1, fw1, 2, 0, false);
-        mm(fa1, fw1, 2, 1, false);
+        // the A stage read next has landed: steps 1 and 3 start a stage whose last DMA was issued in slot 2
+        if (S & 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        fa0[0] = *reinterpret_cast<const bf16x8*>(pa0);
+        fa0[1] = *reinterpret_cast<const bf16x8*>(pa0 + 4096);
+        vmem(IntC<12>{});
+        mm2(IntC<12>{});
         U_SLOT_END();
-        mm(fa1, fw1, 2, 2, false);
-        mm(fa1, fw1, 2, 3, false);
-        mm(fa1, fw1, 3, 0, false);
-        mm(fa1, fw1, 3, 1, false);
-        mm(fa1, fw1, 3, 2, false);
-        mm(fa1, fw1, 3, 3, false);
+        fa0[2] = *reinterpret_cast<const bf16x8*>(pa0 + 8192);
+        fa0[3] = *reinterpret_cast<const bf16x8*>(pa0 + 12288);
+        vmem(IntC<13>{});
+        mm2(IntC<13>{});
+        U_SLOT_END();
+        vmem(IntC<14>{});
+        mm2(IntC<14>{});
+        U_SLOT_END();
+        vmem(IntC<15>{});
+        mm2(IntC<15>{});
         U_SLOT_END();
 #undef U_SLOT_END
     };
-
-    // after a tile's stores, the first two steps of the next tile may leave them outstanding
-    typedef IntC<U_VMEM_PER_STEP> WaitSteady;
-    typedef IntC<U_VMEM_PER_STEP + U_STORES_PER_TILE> WaitAfterStores;
+    auto macro_step = [&](int mi, auto first_c) {
+        a1_cur = cur.a + (size_t)mi * (UMAC * 2) + 128;
+        const bool wrap = mi + 1 == nmac;
+        const int mn = wrap ? 0 : mi + 1;
+        a0_nxt = (wrap ? next.a : cur.a) + (size_t)mn * (UMAC * 2);
+        a1_nxt = a0_nxt + 128;
+        w_nxt = (wrap ? next.w : cur.w) + (size_t)mn * UMAC;
+        ws_nxt = (wrap ? next.ws : cur.ws) + mn * (UMAC / 32);
+        step(IntC<0>{}, first_c);
+        step(IntC<1>{}, IntC<0>{});
+        step(IntC<2>{}, IntC<0>{});
+        step(IntC<3>{}, IntC<0>{});
+    };
 
     for (;;) {
         const int next_local = local + slots;
         const bool more = has_tile(next_local);
-        if (more) next = tile_at(next_local);  // else the look-ahead re-reads this tile's first slabs (unused)
+        if (more) next = tile_at(next_local);  // else the look-ahead re-reads this tile's first operands (unused)
 
-        step(IntC<1>{}, IntC<1>{}, WaitAfterStores{}, 0);
-        step(IntC<0>{}, IntC<0>{}, WaitAfterStores{}, 1);
-        for (int kt = 2; kt < ksteps; kt += 2) {
-            step(IntC<0>{}, IntC<1>{}, WaitSteady{}, kt);
-            step(IntC<0>{}, IntC<0>{}, WaitSteady{}, kt + 1);
-        }
+        macro_step(0, IntC<1>{});
+        for (int mi = 1; mi < nmac; ++mi) macro_step(mi, IntC<0>{});
 
         // ---- output: lane holds, for tile (j, i) and g = 0..3, y[m][n .. n+3] with
         //      m = m0 + wave*128 + i*32 + lane%32,  n = n0 + j*32 + 8*g + 4*(lane/32).
@@ -358,7 +428,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         uint8_t* const y_wave = static_cast<uint8_t*>(y) + ((size_t)(cur.m0 + wave * 128) * N + cur.n0) * 2;
         // output staging (per wave, 32 rows of 128 bytes, 16-byte chunk c of row r at position c ^ (r & 7)):
         // a lane writes 8 bytes of row l & 31 and reads 16 bytes of row 8 t + (l >> 3).  The lane number goes
-        // through an empty asm so that these addresses are recomputed here instead of living in registers
+        // through an asm so that these addresses are recomputed here instead of living in registers
         // through the K loop.
         uint32_t ol = (uint32_t)lane;
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(ol));  // also: the last MFMA results are readable after this
@@ -380,16 +450,17 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
                     const u32x4 v = *reinterpret_cast<const u32x4*>(lds_out + o_rd_off + t * 1024);
                     async_store16(o_st_voff, y_wave + ((size_t)(i * 32 + 8 * t) * N + jh * 64) * 2, v);
                 });
-                __builtin_amdgcn_sched_barrier(0);  // one pass at a time: keeps the accumulator reads from piling up in VGPRs
+                __builtin_amdgcn_sched_barrier(0);  // one pass at a time
             });
         });
 
         if (!more) break;
         cur = next;
         local = next_local;
-        gbase = (gbase + ksteps) & 3;
     }
-    // the look-ahead loads of the last steps still target LDS and registers: let them finish
-    wait_vmcnt<0>(rw[0], sw[0]);
-    wait_vmcnt<0>(rw[1], sw[1]);
+    // the look-ahead loads of the last macro step still target LDS and registers: let them finish
+    wait_vmcnt<0>(wn[0], sn);
+    wait_vmcnt<0>(wn[1], sn);
+    wait_vmcnt<0>(wn[2], sn);
+    wait_vmcnt<0>(wn[3], sn);
 }
