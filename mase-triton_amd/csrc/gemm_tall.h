@@ -23,23 +23,24 @@
 //
 // LDS (160 KB):
 //   A   [2 stages][4 waves][128 rows][128 B]  stage d holds k 64d .. 64d+63 of the macro step; the
-//       16-byte chunk c of row r sits at position c ^ (r & 7) (conflict-free 128-bit fragment reads)
-//   W   [2 stages][128 rows][64 B]            composed bf16 of one K step, chunk c at c ^ ((r >> 2) & 3)
-//   out [4 waves][32 rows][128 B]             turns the accumulator layout into whole output lines
+//       16-byte chunk c of row r sits at position c ^ ((r >> 1) & 7): the LDS serves a 128-bit read 16 lanes
+//       at a time from 64 banks, and 16 consecutive rows then land in 16 different 16-byte bank groups
+//   W   [2 stages][128 rows][128 B]           composed bf16, same split of the macro step and same swizzle.  A wave
+//       composes rows 32w .. 32w+31; between tiles it uses that part of stage 1 to turn the accumulator
+//       layout into whole output lines
 //
-// Macro step m, K step S = 0..3 (slab 4m+S is multiplied; A stage S/2; W stage S%2):
-//   slots 0-7   MFMAs k 0..15 | read fragments k 16..31 of slab S (slots 0-3) | compose W slab S+1, two codes a slot
-//   slot  8     write composed W slab S+1 to its stage
-//   slots 8-9   read the A fragments k 0..15 of slab S+1;  barrier after slot 9;  slots 10-11 the W fragments
-//   slots 8-15  MFMAs k 16..31
-// Global traffic of macro step m (per wave), in issue order:
-//   S=0 slots 0-3    A stage 1 of m   (last 4 of 16 DMAs; the first 12 were issued in S=3 of m-1)
-//   S=0 slot 6       W codes (4 x 16 B per thread) and scales (4 bytes) of macro step m+1
-//   S=1 slots 4-15   A stage 0 of m+1 (first 12)      [stage 0 was last read in S=1 slots 0-3]
-//   S=2 slots 0-3    A stage 0 of m+1 (last 4)
-//   S=3 slots 4-15   A stage 1 of m+1 (first 12)      [stage 1 was last read in S=3 slots 0-3]
-// Waits: S=1 slot 8 needs A stage 1 of m (9 younger operations); top of S=3 needs the W registers
-// of m+1 (16 younger); S=3 slot 8 needs A stage 0 of m+1 (4 younger).
+// Macro step m, K step S = 0..3 (slab 4m+S is multiplied; A and W stage S/2):
+//   slots 0-7    MFMAs k 0..15 | read fragments k 16..31 of slab S (slots 0-3) | compose W slab S+2, two codes a slot
+//   slot  8      write the composed W slab to its stage (S0, S1: stage 1; S2, S3: stage 0 of macro step m+1)
+//   slot  9      S1, S3 only: barrier (the W stage written last is complete, the other one no longer read)
+//   slots 10-13  read the W, then the A fragments k 0..15 of slab S+1
+//   slots 8-15   MFMAs k 16..31
+// Global traffic of macro step m (per wave): one A DMA every second slot -
+//   S3 of m-1 slots 4..14, S0, S1 slots 0..2    A stage 1 of m     [stage 1 was last read in S3 slots 0-3]
+//   S1 slots 4..14, S2, S3 slots 0..2           A stage 0 of m+1   [stage 0 was last read in S1 slots 0-3]
+//   S0 slots 5..13 (odd)                        W codes (4 x 16 B per thread) and scales (4 bytes) of m+1
+// Waits: S1 and S3 slot 12 need the A stage whose last DMA went out in their slot 2 (4 younger operations);
+// the top of S2 needs the W registers of m+1 (9 younger).
 // (included from gemm_impl.h, inside namespace mase, after the shared helpers)
 
 constexpr int UM = 512, UN = 128, UK = 32;
@@ -47,9 +48,9 @@ constexpr int UMAC = 128;                         // k per macro step: four K st
 constexpr int U_A_STAGES = 2, U_W_STAGES = 2;
 constexpr int U_A_STAGE_BYTES = UM * 64 * 2;      // 64 KB: 512 rows x 64 k
 constexpr int U_A_WAVE_BYTES = 128 * 128;         // one wave's 128 rows of a stage
-constexpr int U_W_STAGE_BYTES = UN * UK * 2;      // 8 KB: 128 rows x 32 k, composed
+constexpr int U_W_STAGE_BYTES = UN * 64 * 2;      // 16 KB: 128 rows x 64 k, composed
 constexpr int U_OUT_WAVE_BYTES = 32 * 128;        // 32 rows x 64 outputs of 2 bytes
-constexpr int U_LDS_BYTES = U_A_STAGES * U_A_STAGE_BYTES + U_W_STAGES * U_W_STAGE_BYTES + 4 * U_OUT_WAVE_BYTES;  // 160 KB
+constexpr int U_LDS_BYTES = U_A_STAGES * U_A_STAGE_BYTES + U_W_STAGES * U_W_STAGE_BYTES;  // 160 KB
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -125,31 +126,35 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     const uint32_t lds_aw = (uint32_t)(uintptr_t)lds + (uint32_t)wave * U_A_WAVE_BYTES;  // this wave's rows of stage 0
     uint8_t* const lds_a_ptr = lds + wave * U_A_WAVE_BYTES;
     uint8_t* const lds_w_ptr = lds + U_A_STAGES * U_A_STAGE_BYTES;
-    uint8_t* const lds_out = lds_w_ptr + U_W_STAGES * U_W_STAGE_BYTES + wave * U_OUT_WAVE_BYTES;
+    // output staging: the wave's own 32 rows of W stage 1, which nobody reads between the last barrier of a tile
+    // and this wave's next write of them
+    uint8_t* const lds_out = lds_w_ptr + U_W_STAGE_BYTES + wave * U_OUT_WAVE_BYTES;
 
     // ---- per-lane constants
     // A DMA: instruction i of a wave covers its rows 8i .. 8i+7; lane l fills position l & 7 of row
-    // 8i + (l >> 3), which must hold chunk (l & 7) ^ (row & 7) = (l & 7) ^ (l >> 3)
+    // 8i + (l >> 3), which must hold chunk (l & 7) ^ (row >> 1 & 7) = (l & 7) ^ ((4i + (l >> 4)) & 7)
     uint32_t a_voff[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-        a_voff[i] = (uint32_t)(8 * i + (lane >> 3)) * (uint32_t)K * 2u + (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16) -
+        a_voff[i] = (uint32_t)(8 * i + (lane >> 3)) * (uint32_t)K * 2u + (uint32_t)(((lane & 7) ^ ((4 * i + (lane >> 4)) & 7)) * 16) -
                     (uint32_t)((i & 3) * 1024);  // DMAs 4q+1 .. 4q+3 reuse the M0 of DMA 4q and add an immediate instead
     // A fragment reads: lane (g = l >> 5, r = l & 31) reads chunk 2qq + g of row 32 t + r, qq = k / 16 within the stage
     uint32_t fa_off[4];
 #pragma unroll
-    for (int qq = 0; qq < 4; ++qq) fa_off[qq] = (uint32_t)(lane & 31) * 128u + (uint32_t)(((2 * qq + (lane >> 5)) ^ (lane & 7)) * 16);
+    for (int qq = 0; qq < 4; ++qq)
+        fa_off[qq] = (uint32_t)(lane & 31) * 128u + (uint32_t)(((2 * qq + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16);
     // W staging: thread t owns codes [16 h, 16 h + 16) of row t >> 1 in every K step, h = t & 1
     const int w_row = tid >> 1, w_half = tid & 1;
     const uint32_t w_voff = (uint32_t)w_row * (uint32_t)K + (uint32_t)w_half * 16u;
     const uint32_t ws_voff = (uint32_t)w_row * (uint32_t)kblocks;
-    const uint32_t w_swz = (uint32_t)((w_row >> 2) & 3);
-    const uint32_t w_lds_off0 = (uint32_t)w_row * 64u + (((2u * w_half) ^ w_swz) * 16u);
-    const uint32_t w_lds_off1 = (uint32_t)w_row * 64u + (((2u * w_half + 1u) ^ w_swz) * 16u);
-    // W fragment reads: lane (g, r) reads chunk 2q + g of row 32 t + r
-    const uint32_t f_swz = (uint32_t)((lane >> 2) & 3);
-    const uint32_t fw_off_q0 = (uint32_t)(lane & 31) * 64u + ((((uint32_t)(lane >> 5)) ^ f_swz) * 16u);
-    const uint32_t fw_off_q1 = (uint32_t)(lane & 31) * 64u + (((2u + (uint32_t)(lane >> 5)) ^ f_swz) * 16u);
+    // its 16 bf16 of K step p (0 / 1 within the 64-k stage) are chunks 4p + 2h and 4p + 2h + 1 of the row
+    uint32_t w_lds_off[2][2];
+#pragma unroll
+    for (int pp = 0; pp < 2; ++pp)
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+            w_lds_off[pp][e] = (uint32_t)w_row * 128u + (uint32_t)(((4 * pp + 2 * w_half + e) ^ ((w_row >> 1) & 7)) * 16);
+    // W fragment reads use the same offsets as A's (same row length and swizzle)
 
     const int n_tiles = tiles_m * tiles_n;
     const int per_xcd = (n_tiles + 7) >> 3;
@@ -176,8 +181,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     if (!has_tile(local)) return;
     TallTile cur = tile_at(local), next = cur;
 
-    // raw W codes and scales: `wc` serves K steps 1..3 of the current macro step (index = step), `wn` is the
-    // landing area of the next macro step's (its step 0 is composed during step 3 of the current one)
+    // raw W codes and scales: `wn` is the landing area of the next macro step's (its slabs 0, 1 are composed
+    // during steps 2, 3 of the current one), `wc[2..3]`, `sc` keep slabs 2, 3 of the current one
     u32x4 wc[4], wn[4];
     uint32_t sc, sn;
     auto issue_w_codes = [&](const uint8_t* w_src, auto q_c) {
@@ -198,19 +203,19 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         if (i % 4 == 0) dma_1kb(lds_aw + (uint32_t)stage * U_A_STAGE_BYTES + (uint32_t)i * 1024u, a_voff[i], src);
         else dma_1kb_keep_m0<(i % 4) * 1024>(a_voff[i], src);
     };
-    auto compose_to = [&](const u32x4& codes, uint32_t scale, int w_stage) {
+    auto compose_to = [&](const u32x4& codes, uint32_t scale, int w_stage, int pp) {
         uint4 lo, hi;
         Composer<FW>::template compose16<true>(make_uint4(codes.x, codes.y, codes.z, codes.w), scale, lo, hi);
         uint8_t* const st = lds_w_ptr + w_stage * U_W_STAGE_BYTES;
-        *reinterpret_cast<uint4*>(st + w_lds_off0) = lo;
-        *reinterpret_cast<uint4*>(st + w_lds_off1) = hi;
+        *reinterpret_cast<uint4*>(st + w_lds_off[pp][0]) = lo;
+        *reinterpret_cast<uint4*>(st + w_lds_off[pp][1]) = hi;
     };
 
     floatx16 acc[4][4];  // [n-tile j][m-tile i]
     bf16x8 fa0[4], fw0[4], fa1[4], fw1[4];
 
-    // ---- prologue of the stream: what a macro step expects to find: A stage 0 landed, the first 12 DMAs
-    //      of A stage 1 issued, W slab 0 composed, wc = the macro step's codes, fragments k 0..15 of slab 0
+    // ---- prologue of the stream: what a macro step expects to find: A stage 0 landed, the first 6 DMAs
+    //      of A stage 1 issued, W slabs 0, 1 composed, wc = the codes of slabs 2, 3, fragments k 0..15 of slab 0
     {
         issue_w(cur.w, cur.ws);
         static_for<16>([&](auto i_c) { issue_a(cur.a, 0, i_c); });
@@ -219,8 +224,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         wait_vmcnt<0>(wn[2], sn);
         wait_vmcnt<0>(wn[3], sn);
         static_for<6>([&](auto i_c) { issue_a(cur.a + 128, 1, i_c); });
-        compose_to(wn[0], sn & 0xFFu, 0);
-        wc[1] = wn[1];
+        compose_to(wn[0], sn & 0xFFu, 0, 0);
+        compose_to(wn[1], (sn >> 8) & 0xFFu, 0, 1);
         wc[2] = wn[2];
         wc[3] = wn[3];
         sc = sn;
@@ -228,7 +233,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 #pragma unroll
         for (int i = 0; i < 4; ++i) fa0[i] = *reinterpret_cast<const bf16x8*>(lds_a_ptr + fa_off[0] + i * 4096);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) fw0[j] = *reinterpret_cast<const bf16x8*>(lds_w_ptr + fw_off_q0 + j * 2048);
+        for (int j = 0; j < 4; ++j) fw0[j] = *reinterpret_cast<const bf16x8*>(lds_w_ptr + fa_off[0] + j * 4096);
     }
 
     // pointers of the macro step in flight: a1_cur = second 64-k half of the current macro step; *_nxt = the
@@ -239,23 +244,25 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     auto step = [&](auto s_c, auto first_c) {
         constexpr int S = decltype(s_c)::value;
         constexpr bool FIRST = decltype(first_c)::value != 0;
-        constexpr int WST_NOW = S & 1, WST_NEXT = (S + 1) & 1;
+        // this step composes slab S+2 (S0, S1: second 64-k half of this macro step, W stage 1; S2, S3: first half
+        // of the next macro step, W stage 0)
+        constexpr int WST_WRITE = S < 2 ? 1 : 0, PP = S & 1;
         constexpr int AST_NOW = S >> 1, QQ1 = 2 * (S & 1) + 1;                      // fragments k 16..31 of slab S
         constexpr int AST_NEXT = ((S + 1) >> 1) & 1, QQ0 = 2 * ((S + 1) & 1);        // fragments k 0..15 of slab S+1
         const uint8_t* const pa1 = lds_a_ptr + AST_NOW * U_A_STAGE_BYTES + fa_off[QQ1];
-        const uint8_t* const pw1 = lds_w_ptr + WST_NOW * U_W_STAGE_BYTES + fw_off_q1;
+        const uint8_t* const pw1 = lds_w_ptr + AST_NOW * U_W_STAGE_BYTES + fa_off[QQ1];
         const uint8_t* const pa0 = lds_a_ptr + AST_NEXT * U_A_STAGE_BYTES + fa_off[QQ0];
-        const uint8_t* const pw0 = lds_w_ptr + WST_NEXT * U_W_STAGE_BYTES + fw_off_q0;
-        uint8_t* const wst = lds_w_ptr + WST_NEXT * U_W_STAGE_BYTES;
+        const uint8_t* const pw0 = lds_w_ptr + AST_NEXT * U_W_STAGE_BYTES + fa_off[QQ0];
+        uint8_t* const wst = lds_w_ptr + WST_WRITE * U_W_STAGE_BYTES;
 
-        if (S == 3) {  // the next macro step's codes and scales are about to be composed / copied
-            wait_vmcnt<17>(wn[0], sn);
-            wait_vmcnt<17>(wn[1], sn);
-            wait_vmcnt<17>(wn[2], sn);
-            wait_vmcnt<17>(wn[3], sn);
+        if (S == 2) {  // the next macro step's codes and scales are about to be composed
+            wait_vmcnt<9>(wn[0], sn);
+            wait_vmcnt<9>(wn[1], sn);
+            wait_vmcnt<9>(wn[2], sn);
+            wait_vmcnt<9>(wn[3], sn);
         }
-        const u32x4& codes = S == 3 ? wn[0] : wc[(S + 1) & 3];
-        const uint32_t scale = S == 3 ? (sn & 0xFFu) : ((sc >> (8 * ((S + 1) & 3))) & 0xFFu);
+        const u32x4& codes = S < 2 ? wc[(S + 2) & 3] : wn[(S + 2) & 3];
+        const uint32_t scale = ((S < 2 ? sc : sn) >> (8 * ((S + 2) & 3))) & 0xFFu;
         const Composer<FW> cmp(scale);
         const uint32_t cw[4] = {codes.x, codes.y, codes.z, codes.w};
         uint32_t o[8];
@@ -318,13 +325,13 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         mm2(IntC<1>{});
         U_SLOT_END();
         fw1[0] = *reinterpret_cast<const bf16x8*>(pw1);
-        fw1[1] = *reinterpret_cast<const bf16x8*>(pw1 + 2048);
+        fw1[1] = *reinterpret_cast<const bf16x8*>(pw1 + 4096);
         pair_at(IntC<2>{});
         vmem(IntC<2>{});
         mm2(IntC<2>{});
         U_SLOT_END();
-        fw1[2] = *reinterpret_cast<const bf16x8*>(pw1 + 4096);
-        fw1[3] = *reinterpret_cast<const bf16x8*>(pw1 + 6144);
+        fw1[2] = *reinterpret_cast<const bf16x8*>(pw1 + 8192);
+        fw1[3] = *reinterpret_cast<const bf16x8*>(pw1 + 12288);
         pair_at(IntC<3>{});
         vmem(IntC<3>{});
         mm2(IntC<3>{});
@@ -352,11 +359,10 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         {
             uint4 lo = make_uint4(o[0], o[1], o[2], o[3]), hi = make_uint4(o[4], o[5], o[6], o[7]);
             Composer<FW>::fix255(scale, make_uint4(cw[0], cw[1], cw[2], cw[3]), lo, hi);
-            *reinterpret_cast<uint4*>(wst + w_lds_off0) = lo;
-            *reinterpret_cast<uint4*>(wst + w_lds_off1) = hi;
+            *reinterpret_cast<uint4*>(wst + w_lds_off[PP][0]) = lo;
+            *reinterpret_cast<uint4*>(wst + w_lds_off[PP][1]) = hi;
         }
         if (S == 3) {
-            wc[1] = wn[1];
             wc[2] = wn[2];
             wc[3] = wn[3];
             sc = sn;
@@ -367,15 +373,16 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         vmem(IntC<9>{});
         mm2(IntC<9>{});
         U_SLOT_END();
-        lds_barrier();  // every wave's part of W slab S+1 is in LDS; W slab S is no longer read
+        // S1: W stage 1 is complete and W stage 0 is no longer read; S3: the other way round
+        if (S & 1) lds_barrier();
         U_SLOT_END();
         fw0[0] = *reinterpret_cast<const bf16x8*>(pw0);
-        fw0[1] = *reinterpret_cast<const bf16x8*>(pw0 + 2048);
+        fw0[1] = *reinterpret_cast<const bf16x8*>(pw0 + 4096);
         vmem(IntC<10>{});
         mm2(IntC<10>{});
         U_SLOT_END();
-        fw0[2] = *reinterpret_cast<const bf16x8*>(pw0 + 4096);
-        fw0[3] = *reinterpret_cast<const bf16x8*>(pw0 + 6144);
+        fw0[2] = *reinterpret_cast<const bf16x8*>(pw0 + 8192);
+        fw0[3] = *reinterpret_cast<const bf16x8*>(pw0 + 12288);
         vmem(IntC<11>{});
         mm2(IntC<11>{});
         U_SLOT_END();
@@ -445,10 +452,14 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
                     const uint32_t chunk = (uint32_t)(jj * 4 + g) ^ (o_row & 7u);
                     *reinterpret_cast<uint2*>(lds_out + o_row * 128u + chunk * 16u + o_half * 8u) = p;
                 });
+                u32x4 v[4];
                 static_for<4>([&](auto t_c) {
                     constexpr int t = decltype(t_c)::value;
-                    const u32x4 v = *reinterpret_cast<const u32x4*>(lds_out + o_rd_off + t * 1024);
-                    async_store16(o_st_voff, y_wave + ((size_t)(i * 32 + 8 * t) * N + jh * 64) * 2, v);
+                    v[t] = *reinterpret_cast<const u32x4*>(lds_out + o_rd_off + t * 1024);
+                });
+                static_for<4>([&](auto t_c) {
+                    constexpr int t = decltype(t_c)::value;
+                    async_store16(o_st_voff, y_wave + ((size_t)(i * 32 + 8 * t) * N + jh * 64) * 2, v[t]);
                 });
                 __builtin_amdgcn_sched_barrier(0);  // one pass at a time
             });

@@ -140,6 +140,52 @@ def test_mxfp_linear_vs_cpu_reference_path(mh):
     assert rel_fro(y, y_ref) <= REL_FRO_TOL
 
 
+@pytest.mark.parametrize("MNK,w_tag,odt", [
+    ((4096, 2048, 128), "MXFP8_E4M3_fn", torch.bfloat16),    # 128 tiles, a single 128-k macro step per tile
+    ((2048, 8320, 384), "OCP_MXFP6_E3M2", torch.bfloat16),   # 260 tiles: some workgroups take two, one XCD is short
+    ((8192, 2048, 1024), "OCP_MXFP4_E2M1", torch.float16),   # one tile per workgroup, fp16 output
+    ((1536, 16384, 256), "MXFP8_E5M2_fn", torch.bfloat16),   # 3 tile rows: the last group of tile rows is a single row
+    ((16384, 1024, 512), "OCP_MXFP6_E2M3", torch.bfloat16),  # tall problem: 32 x 8 tiles
+])
+def test_gemm_large_tile_shapes(mh, MNK, w_tag, odt):
+    """Shapes that take the 512 x 128 tile kernel (dense A, 16-bit output, no bias, whole tiles): the whole output
+    against an fp32 dequantize-then-matmul on the GPU, and a sample of it against float64 accumulation."""
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    we, wm = PRESETS[w_tag]
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    w_sc, w_el = oracle.extract_mxfp(w, 32, we, wm)
+    w_dq = oracle.compose_mxfp(w_sc, w_el, 32, we, wm, True, torch.bfloat16).view(N, K)
+    y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, w_tag), None, M, N, K, odt)
+    assert y.shape == (M, N) and y.dtype == odt
+    y_gpu = (x_dq.to(DEV).float() @ w_dq.to(DEV).float().T).to(odt)
+    assert rel_fro(y, y_gpu) <= REL_FRO_TOL
+    rows = torch.arange(0, M, 61)
+    cols = torch.arange(0, N, 37)
+    y_ref = oracle.matmul_nt(x_dq[rows], w_dq[cols]).to(odt)
+    assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref) <= REL_FRO_TOL
+
+
+def test_gemm_large_tile_special_values(mh):
+    """Scale 255 (a block that held an inf) on the 512 x 128 tile kernel: that output column is NaN, the rest finite."""
+    M, N, K = 4096, 2048, 256
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    w[777, 200] = float("inf")
+    w[5, 3] = float("nan")
+    w_sc, w_el = oracle.extract_mxfp(w, 32, 4, 3)
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), None,
+                         M, N, K, torch.bfloat16).cpu()
+    bad = torch.zeros(N, dtype=torch.bool)
+    bad[777] = bad[5] = True
+    assert y[:, bad].isnan().all()
+    assert y[:, ~bad].isfinite().all()
+
+
 def test_config_c4_full_size(mh):
     """x [16384,4096] . W [14336,4096]^T, both MXFP8 E4M3.  The whole output is compared with
     the GPU dequantize-then-matmul (fp32 accumulate, bf16 out); a sample of rows and columns
