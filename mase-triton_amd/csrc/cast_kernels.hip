@@ -11,27 +11,61 @@
 namespace mase {
 
 constexpr int kThreads = 256;
+// 128-bit steps per lane and launch: one is fastest on every measured size (more, smaller workgroups in flight)
+#ifndef MASE_UNROLL_SMALL
+#define MASE_UNROLL_SMALL 1
+#endif
+#ifndef MASE_UNROLL_MXFP
+#define MASE_UNROLL_MXFP 1
+#endif
+#ifndef MASE_UNROLL_PACKED
+#define MASE_UNROLL_PACKED 1
+#endif
 
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
 
 // ------------------------------------------------------------------------------ vector I/O
+// 128- and 64-bit accesses of the streaming kernels.  Every byte is touched once, so loads and stores are
+// marked non-temporal (no reuse to keep in the caches); measured faster on all kernels but the fp32 -> fp32
+// fused minifloat pass, which passes NT = false.
+typedef uint32_t u32v4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32v2 __attribute__((ext_vector_type(2)));
+template <bool NT = true>
+__device__ inline uint4 ld128(const void* p) {
+    if (NT) {
+        const u32v4 v = __builtin_nontemporal_load(static_cast<const u32v4*>(p));
+        return make_uint4(v.x, v.y, v.z, v.w);
+    }
+    return *static_cast<const uint4*>(p);
+}
+__device__ inline uint2 ld64(const void* p) {
+    const u32v2 v = __builtin_nontemporal_load(static_cast<const u32v2*>(p));
+    return make_uint2(v.x, v.y);
+}
+template <bool NT = true>
+__device__ inline void st128(void* p, uint4 v) {
+    if (NT) __builtin_nontemporal_store(u32v4{v.x, v.y, v.z, v.w}, static_cast<u32v4*>(p));
+    else *static_cast<uint4*>(p) = v;
+}
+__device__ inline void st64(void* p, uint2 v) { __builtin_nontemporal_store(u32v2{v.x, v.y}, static_cast<u32v2*>(p)); }
+
 // EPT elements starting at element index `off` of a flat array, as fp32 bit patterns.
-template <int DT, int EPT>
+template <int DT, int EPT, bool NT = true>
 __device__ inline void load_bits(const void* base, int64_t off, uint32_t (&u)[EPT]) {
     if (DT == F32) {
         const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint32_t*>(base) + off);
 #pragma unroll
         for (int v = 0; v < EPT / 4; ++v) {
-            const uint4 r = p[v];
+            const uint4 r = ld128<NT>(p + v);
             u[4 * v + 0] = r.x; u[4 * v + 1] = r.y; u[4 * v + 2] = r.z; u[4 * v + 3] = r.w;
         }
     } else {
         const uint4* p = reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + off);
 #pragma unroll
         for (int v = 0; v < EPT / 8; ++v) {
-            const uint4 r = p[v];
+            const uint4 r = ld128<NT>(p + v);
             const uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -62,13 +96,13 @@ __device__ inline uint32_t pack_f16(float a, float b) {
     return f32_bits_to_half_bits(f32_bits(a)) | (f32_bits_to_half_bits(f32_bits(b)) << 16);
 }
 
-template <int DT, int EPT>
+template <int DT, int EPT, bool NT = true>
 __device__ inline void store_vals(void* base, int64_t off, const float (&y)[EPT]) {
     if (DT == F32) {
         uint4* p = reinterpret_cast<uint4*>(static_cast<float*>(base) + off);
 #pragma unroll
         for (int v = 0; v < EPT / 4; ++v)
-            p[v] = make_uint4(f32_bits(y[4 * v]), f32_bits(y[4 * v + 1]), f32_bits(y[4 * v + 2]), f32_bits(y[4 * v + 3]));
+            st128<NT>(p + v, make_uint4(f32_bits(y[4 * v]), f32_bits(y[4 * v + 1]), f32_bits(y[4 * v + 2]), f32_bits(y[4 * v + 3])));
     } else {
         uint4* p = reinterpret_cast<uint4*>(static_cast<uint16_t*>(base) + off);
 #pragma unroll
@@ -78,7 +112,7 @@ __device__ inline void store_vals(void* base, int64_t off, const float (&y)[EPT]
             for (int j = 0; j < 4; ++j)
                 w[j] = DT == BF16 ? pack_bf16(y[8 * v + 2 * j], y[8 * v + 2 * j + 1])
                                   : pack_f16(y[8 * v + 2 * j], y[8 * v + 2 * j + 1]);
-            p[v] = make_uint4(w[0], w[1], w[2], w[3]);
+            st128<NT>(p + v, make_uint4(w[0], w[1], w[2], w[3]));
         }
     }
 }
@@ -111,7 +145,7 @@ __global__ __launch_bounds__(kThreads) void extract_minifloat_kernel(const void*
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 w[j] = encode_f32_bits(u[r][2 * j], f) | (encode_f32_bits(u[r][2 * j + 1], f) << 16);
-            *reinterpret_cast<uint4*>(codes + c * EPT) = make_uint4(w[0], w[1], w[2], w[3]);
+            st128(codes + c * EPT, make_uint4(w[0], w[1], w[2], w[3]));
         }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n % EPT)) {
@@ -130,7 +164,7 @@ __global__ __launch_bounds__(kThreads) void compose_minifloat_kernel(const uint1
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
         const int64_t c = chunk0 + (int64_t)r * kThreads;
-        if (c < n_chunks) raw[r] = *reinterpret_cast<const uint4*>(codes + c * EPT);
+        if (c < n_chunks) raw[r] = ld128(codes + c * EPT);
     }
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
@@ -161,7 +195,7 @@ __global__ __launch_bounds__(kThreads) void qdq_minifloat_kernel(const void* x, 
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
         const int64_t c = chunk0 + (int64_t)r * kThreads;
-        if (c < n_chunks) load_bits<DT_IN, EPT>(x, c * EPT, u[r]);
+        if (c < n_chunks) load_bits<DT_IN, EPT, false>(x, c * EPT, u[r]);
     }
     // the scalar tail reads before anything is written, so that `out` may alias `x`
     uint32_t tail_bits = 0;
@@ -174,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void qdq_minifloat_kernel(const void* x, 
             float y[EPT];
 #pragma unroll
             for (int j = 0; j < EPT; ++j) y[j] = decode_f32(encode_f32_bits(u[r][j], f), f);
-            store_vals<DT_OUT, EPT>(out, c * EPT, y);
+            store_vals<DT_OUT, EPT, false>(out, c * EPT, y);
         }
     }
     if (has_tail) store_val_scalar<DT_OUT>(out, n_chunks * EPT + threadIdx.x, decode_f32(encode_f32_bits(tail_bits, f), f));
@@ -233,8 +267,8 @@ __global__ __launch_bounds__(kThreads) void extract_mxfp_kernel(const void* __re
 #pragma unroll
             for (int j = 0; j < EPT / 4; ++j)
                 w[j] = code[4 * j] | (code[4 * j + 1] << 8) | (code[4 * j + 2] << 16) | (code[4 * j + 3] << 24);
-            if constexpr (EPT == 16) *reinterpret_cast<uint4*>(elements + c * EPT) = make_uint4(w[0], w[1], w[2], w[3]);
-            else *reinterpret_cast<uint2*>(elements + c * EPT) = make_uint2(w[0], w[1]);
+            if constexpr (EPT == 16) st128(elements + c * EPT, make_uint4(w[0], w[1], w[2], w[3]));
+            else st64(elements + c * EPT, make_uint2(w[0], w[1]));
             if ((c & (lpb - 1)) == 0) scales[c >> lpb_shift] = (uint8_t)scale;
         }
     }
@@ -323,7 +357,7 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
         const int64_t c = chunk0 + (int64_t)r * kThreads;
-        raw[r] = c < n_chunks ? x[c] : make_uint4(0, 0, 0, 0);
+        raw[r] = c < n_chunks ? ld128(x + c) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
@@ -361,10 +395,10 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
         if (c < n_chunks) {
             if (MODE == 0) {
                 // o[j] holds two codes in the low bytes of its halves: gather the 8 code bytes
-                elements[c] = make_uint2(__builtin_amdgcn_perm(o[1], o[0], 0x06040200u), __builtin_amdgcn_perm(o[3], o[2], 0x06040200u));
+                st64(elements + c, make_uint2(__builtin_amdgcn_perm(o[1], o[0], 0x06040200u), __builtin_amdgcn_perm(o[3], o[2], 0x06040200u)));
                 if ((c & 3) == 0) scales[c >> 2] = (uint8_t)scale;
             } else {
-                out[c] = make_uint4(o[0], o[1], o[2], o[3]);
+                st128(out + c, make_uint4(o[0], o[1], o[2], o[3]));
             }
         }
     }
@@ -401,10 +435,10 @@ __global__ __launch_bounds__(kThreads) void compose_mxfp_kernel(const uint8_t* _
         const int64_t c = chunk0 + (int64_t)r * kThreads;
         if (c < n_chunks) {
             if constexpr (EPT == 16) {
-                const uint4 v = *reinterpret_cast<const uint4*>(elements + c * EPT);
+                const uint4 v = ld128(elements + c * EPT);
                 w[r][0] = v.x; w[r][1] = v.y; w[r][2] = v.z; w[r][3] = v.w;
             } else {
-                const uint2 v = *reinterpret_cast<const uint2*>(elements + c * EPT);
+                const uint2 v = ld64(elements + c * EPT);
                 w[r][0] = v.x; w[r][1] = v.y;
             }
             sc[r] = scales[c / chunks_per_block];
@@ -513,7 +547,7 @@ int mase_hip_extract_minifloat(const void* x, int x_dtype, uint16_t* codes, int6
     if (!x || !codes) return fail(ERR_INVALID, "null pointer");
     if (!aligned(x, 16) || !aligned(codes, 16)) return fail(ERR_INVALID, "x and codes must be 16-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = MASE_UNROLL_SMALL;
     const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
         return dispatch_dtype(x_dtype, [&](auto dt) {
@@ -533,7 +567,7 @@ int mase_hip_compose_minifloat(const uint16_t* codes, void* out, int out_dtype, 
     if (!codes || !out) return fail(ERR_INVALID, "null pointer");
     if (!aligned(codes, 16) || !aligned(out, 16)) return fail(ERR_INVALID, "codes and out must be 16-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = MASE_UNROLL_SMALL;
     const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, RN, [&](auto f) {
         return dispatch_dtype(out_dtype, [&](auto dt) {
@@ -555,7 +589,7 @@ int mase_hip_qdq_minifloat(const void* x, int x_dtype, void* out, int out_dtype,
     if (!aligned(x, 16) || !aligned(out, 16)) return fail(ERR_INVALID, "x and out must be 16-byte aligned");
     if (x == out && dtype_size(x_dtype) != dtype_size(out_dtype)) return fail(ERR_INVALID, "in-place use needs equal element sizes");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = MASE_UNROLL_SMALL;
     const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
         return dispatch_dtype(x_dtype, [&](auto di) {
@@ -575,13 +609,13 @@ int mase_hip_extract_mxfp(const void* x, int x_dtype, uint8_t* scales, uint8_t* 
     if (n == 0) return OK;
     if (!x || !scales || !elements) return fail(ERR_INVALID, "null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int EPT = 8, UNROLL = 4;
+    constexpr int EPT = 8, UNROLL = MASE_UNROLL_MXFP;
     const int B = block_size;
     const bool vec = B % EPT == 0 && pow2(B / EPT) && B / EPT <= 64 && aligned(x, 16) && aligned(elements, 8);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
         if constexpr (decltype(f)::kStatic) {
             if (x_dtype == BF16 && B == 32 && vec) {
-                constexpr int U = 4;
+                constexpr int U = MASE_UNROLL_PACKED;
                 hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 0>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
                                    static_cast<const uint4*>(x), scales, reinterpret_cast<uint2*>(elements), nullptr, n / 8, f);
                 return check_launch("extract_mxfp");
@@ -609,16 +643,13 @@ int mase_hip_compose_mxfp(const uint8_t* scales, const uint8_t* elements, void* 
     if (n == 0) return OK;
     if (!scales || !elements || !out) return fail(ERR_INVALID, "null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = MASE_UNROLL_SMALL;
     const int B = block_size;
-    const bool al = aligned(elements, 16) && aligned(out, 16);
+    const bool al = aligned(elements, 8) && aligned(out, 16);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, RN, [&](auto f) {
         return dispatch_dtype(out_dtype, [&](auto dt) {
-            if (al && B % 16 == 0) {
-                hipLaunchKernelGGL((compose_mxfp_kernel<decltype(dt)::value, decltype(f), 16, UNROLL>),
-                                   dim3(grid_for(n / 16, UNROLL * kThreads)), dim3(kThreads), 0, s, scales, elements, out, n, B / 16,
-                                   f);
-            } else if (al && B % 8 == 0) {
+            // 8 codes per lane: a wavefront then stores 1 KB contiguous per instruction (16 per lane would leave gaps)
+            if (al && B % 8 == 0) {
                 hipLaunchKernelGGL((compose_mxfp_kernel<decltype(dt)::value, decltype(f), 8, UNROLL>),
                                    dim3(grid_for(n / 8, UNROLL * kThreads)), dim3(kThreads), 0, s, scales, elements, out, n, B / 8, f);
             } else {
@@ -639,13 +670,13 @@ int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int6
     if (!x || !out) return fail(ERR_INVALID, "null pointer");
     if (x == out && dtype_size(x_dtype) != dtype_size(out_dtype)) return fail(ERR_INVALID, "in-place use needs equal element sizes");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int EPT = 8, UNROLL = 4;
+    constexpr int EPT = 8, UNROLL = MASE_UNROLL_MXFP;
     const int B = block_size;
     const bool vec = B % EPT == 0 && pow2(B / EPT) && B / EPT <= 64 && aligned(x, 16) && aligned(out, 16);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
         if constexpr (decltype(f)::kStatic) {
             if (x_dtype == BF16 && out_dtype == BF16 && B == 32 && vec) {
-                constexpr int U = 4;
+                constexpr int U = MASE_UNROLL_PACKED;
                 hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 1>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
                                    static_cast<const uint4*>(x), nullptr, nullptr, static_cast<uint4*>(out), n / 8, f);
                 return check_launch("qdq_mxfp");
