@@ -535,9 +535,9 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     const bool fits32 = (int64_t)M * K * 2 < ((int64_t)1 << 32) && (int64_t)N * K < ((int64_t)1 << 32);  // 32-bit operand offsets
     const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
     if constexpr (A_MODE == 0 && DT_OUT != F32) {
-        // tall tiles: dense A, 16-bit output, no bias, whole tiles only, enough of them to occupy the chip
+        // tall tiles: dense A, 16-bit output, whole tiles only, enough of them to occupy the chip
         const int64_t tall_tiles = (int64_t)(M / UM) * (N / UN);
-        if (fits32 && bias == nullptr && M % UM == 0 && N % UN == 0 && K % UMAC == 0 && tall_tiles >= TALL_MIN_TILES &&
+        if (fits32 && M % UM == 0 && N % UN == 0 && K % UMAC == 0 && tall_tiles >= TALL_MIN_TILES &&
             (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
             (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0) {
             auto kern = mxfp_gemm_tall_kernel<FW, DT_OUT>;
@@ -551,7 +551,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             if (cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
             hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                               w_elements, y, M, N, K, M / UM, N / UN);
+                               w_elements, bias, bias_dtype, y, M, N, K, M / UM, N / UN);
             return check_launch("mxfp_gemm");
         }
     }

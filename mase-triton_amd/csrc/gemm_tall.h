@@ -1,4 +1,4 @@
-// Tall-tile MXFP GEMM kernel for gfx950: 512 (M) x 128 (N) tiles, dense bf16 A, 16-bit output, no bias.
+// Tall-tile MXFP GEMM kernel for gfx950: 512 (M) x 128 (N) tiles, dense bf16 A, 16-bit output.
 //
 // Why this shape.  One wavefront can issue only about three other instructions per 32-cycle
 // 32x32x16 MFMA without slowing the matrix pipe, so the K loop has to be lean:
@@ -118,7 +118,7 @@ struct TallTile {
 template <class FW, int DT_OUT>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_tall_kernel(
     const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -442,28 +442,48 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         const uint32_t o_row = ol & 31u, o_half = ol >> 5;
         const uint32_t o_rd_off = (ol >> 3) * 128u + (((ol & 7u) ^ (ol >> 3)) * 16u);
         const uint32_t o_st_voff = ((ol >> 3) * (uint32_t)N + (ol & 7u) * 8u) * 2u;
-        static_for<4>([&](auto i_c) {
-            static_for<2>([&](auto jh_c) {
-                constexpr int i = decltype(i_c)::value, jh = decltype(jh_c)::value;
-                static_for<8>([&](auto jg_c) {
-                    constexpr int jj = decltype(jg_c)::value >> 2, g = decltype(jg_c)::value & 3, j = 2 * jh + jj;
-                    const uint2 p = pack_out4<DT_OUT>(acc_read(acc[j][i][4 * g]), acc_read(acc[j][i][4 * g + 1]),
-                                                      acc_read(acc[j][i][4 * g + 2]), acc_read(acc[j][i][4 * g + 3]));
-                    const uint32_t chunk = (uint32_t)(jj * 4 + g) ^ (o_row & 7u);
-                    *reinterpret_cast<uint2*>(lds_out + o_row * 128u + chunk * 16u + o_half * 8u) = p;
+        auto write_tile = [&](auto has_bias_c) {
+            constexpr bool HAS_BIAS = decltype(has_bias_c)::value != 0;
+            // the tile's 128 bias values, two per lane: column c sits in register c / 64 of lane c % 64
+            float bv[2] = {0.0f, 0.0f};
+            if (HAS_BIAS) {
+                bv[0] = load_bias(bias, bias_dtype, cur.n0 + (int)ol);
+                bv[1] = load_bias(bias, bias_dtype, cur.n0 + 64 + (int)ol);
+            }
+            static_for<4>([&](auto i_c) {
+                static_for<2>([&](auto jh_c) {
+                    constexpr int i = decltype(i_c)::value, jh = decltype(jh_c)::value;
+                    static_for<8>([&](auto jg_c) {
+                        constexpr int jj = decltype(jg_c)::value >> 2, g = decltype(jg_c)::value & 3, j = 2 * jh + jj;
+                        float r[4];
+                        static_for<4>([&](auto t_c) {
+                            constexpr int t = decltype(t_c)::value, col = 32 * j + 8 * g + t;  // + 4 for the upper half-wave
+                            r[t] = acc_read(acc[j][i][4 * g + t]);
+                            if (HAS_BIAS) {
+                                const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv[col >> 6]), col & 63));
+                                const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv[col >> 6]), (col + 4) & 63));
+                                r[t] += o_half ? hi : lo;
+                            }
+                        });
+                        const uint2 p = pack_out4<DT_OUT>(r[0], r[1], r[2], r[3]);
+                        const uint32_t chunk = (uint32_t)(jj * 4 + g) ^ (o_row & 7u);
+                        *reinterpret_cast<uint2*>(lds_out + o_row * 128u + chunk * 16u + o_half * 8u) = p;
+                    });
+                    u32x4 v[4];
+                    static_for<4>([&](auto t_c) {
+                        constexpr int t = decltype(t_c)::value;
+                        v[t] = *reinterpret_cast<const u32x4*>(lds_out + o_rd_off + t * 1024);
+                    });
+                    static_for<4>([&](auto t_c) {
+                        constexpr int t = decltype(t_c)::value;
+                        async_store16(o_st_voff, y_wave + ((size_t)(i * 32 + 8 * t) * N + jh * 64) * 2, v[t]);
+                    });
+                    __builtin_amdgcn_sched_barrier(0);  // one pass at a time
                 });
-                u32x4 v[4];
-                static_for<4>([&](auto t_c) {
-                    constexpr int t = decltype(t_c)::value;
-                    v[t] = *reinterpret_cast<const u32x4*>(lds_out + o_rd_off + t * 1024);
-                });
-                static_for<4>([&](auto t_c) {
-                    constexpr int t = decltype(t_c)::value;
-                    async_store16(o_st_voff, y_wave + ((size_t)(i * 32 + 8 * t) * N + jh * 64) * 2, v[t]);
-                });
-                __builtin_amdgcn_sched_barrier(0);  // one pass at a time
             });
-        });
+        };
+        if (bias) write_tile(IntC<1>{});
+        else write_tile(IntC<0>{});
 
         if (!more) break;
         cur = next;
