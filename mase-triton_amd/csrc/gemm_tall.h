@@ -35,12 +35,12 @@
 //   slot  9      S1, S3 only: barrier (the W stage written last is complete, the other one no longer read)
 //   slots 10-13  read the W, then the A fragments k 0..15 of slab S+1
 //   slots 8-15   MFMAs k 16..31
-// Global traffic of macro step m (per wave): one A DMA every second slot -
-//   S3 of m-1 slots 4..14, S0, S1 slots 0..2    A stage 1 of m     [stage 1 was last read in S3 slots 0-3]
-//   S1 slots 4..14, S2, S3 slots 0..2           A stage 0 of m+1   [stage 0 was last read in S1 slots 0-3]
-//   S0 slots 5..13 (odd)                        W codes (4 x 16 B per thread) and scales (4 bytes) of m+1
-// Waits: S1 and S3 slot 12 need the A stage whose last DMA went out in their slot 2 (4 younger operations);
-// the top of S2 needs the W registers of m+1 (9 younger).
+// Global traffic of macro step m (per wave): one A DMA per slot in slots 8..15 of every step -
+//   S3 of m-1 and S0     A stage 1 of m     [stage 1 was last read in S3 slots 0-3]
+//   S1 and S2            A stage 0 of m+1   [stage 0 was last read in S1 slots 0-3]
+//   S0 slots 0..4        W codes (4 x 16 B per thread) and scales (4 bytes) of m+1
+// Waits: S1 and S3 slot 12 need the A stage whose last DMA went out in the previous step's slot 15 (4 younger
+// operations); the top of S2 needs the W registers of m+1 (16 younger).
 // (included from gemm_impl.h, inside namespace mase, after the shared helpers)
 
 constexpr int UM = 512, UN = 128, UK = 32;
@@ -185,6 +185,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     // during steps 2, 3 of the current one), `wc[2..3]`, `sc` keep slabs 2, 3 of the current one
     u32x4 wc[4], wn[4];
     uint32_t sc, sn;
+    bool any255_cur = true, any255_nxt = true;  // wave-uniform: a scale of 255 among the macro step's four
     auto issue_w_codes = [&](const uint8_t* w_src, auto q_c) {
         constexpr int q = decltype(q_c)::value;
         async_load16(wn[q], w_voff, w_src + q * 32);
@@ -214,7 +215,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     floatx16 acc[4][4];  // [n-tile j][m-tile i]
     bf16x8 fa0[4], fw0[4], fa1[4], fw1[4];
 
-    // ---- prologue of the stream: what a macro step expects to find: A stage 0 landed, the first 6 DMAs
+    // ---- prologue of the stream: what a macro step expects to find: A stage 0 landed, the first 8 DMAs
     //      of A stage 1 issued, W slabs 0, 1 composed, wc = the codes of slabs 2, 3, fragments k 0..15 of slab 0
     {
         issue_w(cur.w, cur.ws);
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         wait_vmcnt<0>(wn[1], sn);
         wait_vmcnt<0>(wn[2], sn);
         wait_vmcnt<0>(wn[3], sn);
-        static_for<6>([&](auto i_c) { issue_a(cur.a + 128, 1, i_c); });
+        static_for<8>([&](auto i_c) { issue_a(cur.a + 128, 1, i_c); });
         compose_to(wn[0], sn & 0xFFu, 0, 0);
         compose_to(wn[1], (sn >> 8) & 0xFFu, 0, 1);
         wc[2] = wn[2];
@@ -256,10 +257,14 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         uint8_t* const wst = lds_w_ptr + WST_WRITE * U_W_STAGE_BYTES;
 
         if (S == 2) {  // the next macro step's codes and scales are about to be composed
-            wait_vmcnt<9>(wn[0], sn);
-            wait_vmcnt<9>(wn[1], sn);
-            wait_vmcnt<9>(wn[2], sn);
-            wait_vmcnt<9>(wn[3], sn);
+            wait_vmcnt<16>(wn[0], sn);
+            wait_vmcnt<16>(wn[1], sn);
+            wait_vmcnt<16>(wn[2], sn);
+            wait_vmcnt<16>(wn[3], sn);
+            // does any wavefront lane hold a scale of 255 (a block that held inf / NaN) among these four?  Checked once
+            // per macro step; the patch-up code below runs only then.
+            const uint32_t inv = ~sn;
+            any255_nxt = __builtin_amdgcn_ballot_w64(((inv - 0x01010101u) & sn & 0x80808080u) != 0u) != 0;
         }
         const u32x4& codes = S < 2 ? wc[(S + 2) & 3] : wn[(S + 2) & 3];
         const uint32_t scale = ((S < 2 ? sc : sn) >> (8 * ((S + 2) & 3))) & 0xFFu;
@@ -280,20 +285,18 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         // the global traffic of slot `slot` of this step
         auto vmem = [&](auto slot_c) {
             constexpr int slot = decltype(slot_c)::value;
-            // A: one DMA every second slot.  Stage 0 (of the next macro step): S1 slots 4..14, S2, S3 slots 0..2;
-            // stage 1: S3 slots 4..14, S0 of the next macro step, S1 slots 0..2
-            if constexpr (slot % 2 == 0) {
-                constexpr int h = slot / 2;
-                if constexpr (S == 3 && h >= 2) issue_a(a1_nxt, 1, IntC<h - 2>{});
-                if constexpr (S == 0) issue_a(a1_cur, 1, IntC<6 + h>{});
-                if constexpr (S == 1 && h < 2) issue_a(a1_cur, 1, IntC<14 + h>{});
-                if constexpr (S == 1 && h >= 2) issue_a(a0_nxt, 0, IntC<h - 2>{});
-                if constexpr (S == 2) issue_a(a0_nxt, 0, IntC<6 + h>{});
-                if constexpr (S == 3 && h < 2) issue_a(a0_nxt, 0, IntC<14 + h>{});
+            // A: one DMA per slot in the second half of every step (the first half carries the compose).
+            // Stage 0 of the next macro step in S1, S2; stage 1 in S3 and S0 of the next macro step.
+            if constexpr (slot >= 8) {
+                constexpr int h = slot - 8;
+                if constexpr (S == 3) issue_a(a1_nxt, 1, IntC<h>{});
+                if constexpr (S == 0) issue_a(a1_cur, 1, IntC<8 + h>{});
+                if constexpr (S == 1) issue_a(a0_nxt, 0, IntC<h>{});
+                if constexpr (S == 2) issue_a(a0_nxt, 0, IntC<8 + h>{});
             }
-            // W codes and scales of the next macro step: S0, odd slots 5..13
-            if constexpr (S == 0 && slot >= 5 && slot <= 11 && slot % 2 == 1) issue_w_codes(w_nxt, IntC<(slot - 5) / 2>{});
-            if constexpr (S == 0 && slot == 13) issue_w_scales(ws_nxt);
+            // W codes and scales of the next macro step: S0, slots 0..4
+            if constexpr (S == 0 && slot < 4) issue_w_codes(w_nxt, IntC<slot>{});
+            if constexpr (S == 0 && slot == 4) issue_w_scales(ws_nxt);
         };
         auto mm2 = [&](auto slot_c) {
             constexpr int slot = decltype(slot_c)::value, k = slot & 7, j = k >> 1, i = 2 * (k & 1);
@@ -336,9 +339,6 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         vmem(IntC<3>{});
         mm2(IntC<3>{});
         U_SLOT_END();
-        // in steps 1 and 3 the A stage read in slots 0..3 is handed back to the DMA engine from slot 4 on; its
-        // writes must not pass those reads
-        if (S & 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
         pair_at(IntC<4>{});
         vmem(IntC<4>{});
         mm2(IntC<4>{});
@@ -355,14 +355,18 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         vmem(IntC<7>{});
         mm2(IntC<7>{});
         U_SLOT_END();
-        // ---- slots 8..15: MFMAs k 16..31; the composed slab goes to LDS; fragments k 0..15 of the next slab
+        // ---- slots 8..15: MFMAs k 16..31; the composed slab goes to LDS; fragments k 0..15 of the next slab.
+        //      In steps 1 and 3 the A stage read in slots 0..3 is handed back to the DMA engine from here on; its
+        //      writes must not pass those reads
+        if (S & 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
         {
             uint4 lo = make_uint4(o[0], o[1], o[2], o[3]), hi = make_uint4(o[4], o[5], o[6], o[7]);
-            Composer<FW>::fix255(scale, make_uint4(cw[0], cw[1], cw[2], cw[3]), lo, hi);
+            if (S < 2 ? any255_cur : any255_nxt) Composer<FW>::fix255(scale, make_uint4(cw[0], cw[1], cw[2], cw[3]), lo, hi);
             *reinterpret_cast<uint4*>(wst + w_lds_off[PP][0]) = lo;
             *reinterpret_cast<uint4*>(wst + w_lds_off[PP][1]) = hi;
         }
         if (S == 3) {
+            any255_cur = any255_nxt;
             wc[2] = wn[2];
             wc[3] = wn[3];
             sc = sn;
