@@ -100,7 +100,30 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     gemm_ms = sum(event_ms(pairs)) / args.steps
     flop = 2.0 * M * N * K
+    # context, not the metric: the same step with backend="separate" (fused QDQ of x, compose W to bf16 in HBM, then
+    # the vendor library's dense bf16 GEMM through F.linear), and that dense GEMM alone on the dequantised operands
+    sep = dict(call, backend="separate")
+    for _ in range(max(3, args.warmup // 2)):
+        MXFP_F.mxfp_linear(**sep)
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for _ in range(args.steps):
+        MXFP_F.mxfp_linear(**sep)
+    torch.cuda.synchronize()
+    sep_ms = (time.perf_counter() - t2) * 1e3 / args.steps
+    a_dq = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
+    w_dq = kernels.compose_mxfp_tensor(w_sc, w_el, fmt, torch.bfloat16).view(N, K)
+    for _ in range(5):
+        torch.nn.functional.linear(a_dq, w_dq)
+    torch.cuda.synchronize()
+    t3 = time.perf_counter()
+    for _ in range(args.steps):
+        torch.nn.functional.linear(a_dq, w_dq)
+    torch.cuda.synchronize()
+    dense_ms = (time.perf_counter() - t3) * 1e3 / args.steps
+    del a_dq, w_dq
     return {
+        "separate_ms": sep_ms, "dense_ms": dense_ms,
         "ms_per_step": ms_per_step,
         "tflops_step": flop / (ms_per_step * 1e-3) / 1e12,
         "gemm_ms": gemm_ms,
@@ -331,6 +354,14 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(lin["tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": GEMM_C4_TRAFFIC_BYTES,
                      "kernel": "mxfp_gemm_tall_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4)},
+        "context": {
+            "separate_backend_ms_per_step": round(lin["separate_ms"], 4),
+            "separate_backend_TFLOPs": round(2.0 * M * N * K / (lin["separate_ms"] * 1e-3) / 1e12, 2),
+            "vendor_dense_bf16_gemm_ms": round(lin["dense_ms"], 4),
+            "vendor_dense_bf16_gemm_TFLOPs": round(2.0 * M * N * K / (lin["dense_ms"] * 1e-3) / 1e12, 2),
+            "note": "same shape on the same GPU: backend='separate' = QDQ x + compose W to bf16 in HBM + library GEMM "
+                    "(weights held dequantised during the call); dense = the library's bf16 GEMM alone",
+        },
     }
     if not args.skip_hbm:
         result["hbm_kernels"] = bench_hbm(

@@ -411,6 +411,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 }
 
 #include "gemm_tall.h"
+#include "gemm_skinny.h"
 
 // ---------------------------------------------------------------------------------------------
 // Small-shape kernel: 128 x 128 x 32 tiles, single LDS buffer.  Used when the problem cannot
@@ -513,7 +514,7 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
 }
 
 #ifndef TALL_MIN_TILES
-#define TALL_MIN_TILES 128
+#define TALL_MIN_TILES 96
 #endif
 inline int device_cu_count() {
     static int n_cus = 0;
@@ -534,6 +535,12 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     // 256 x 256 tiles need enough of them to occupy the 256 CUs; smaller problems use 128 x 128
     const bool fits32 = (int64_t)M * K * 2 < ((int64_t)1 << 32) && (int64_t)N * K < ((int64_t)1 << 32);  // 32-bit operand offsets
     const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
+    if constexpr (A_MODE == 0) {
+        // few rows of A: bound by streaming W; one workgroup per 32 rows of W
+        if (M <= 128 && N % SK_N == 0 && K % SK_MAC == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
+            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0)
+            return launch_gemm_skinny<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+    }
     if constexpr (A_MODE == 0 && DT_OUT != F32) {
         // tall tiles: dense A, 16-bit output, whole tiles only, enough of them to occupy the chip
         const int64_t tall_tiles = (int64_t)(M / UM) * (N / UN);

@@ -1,0 +1,184 @@
+// Skinny MXFP GEMM kernel for gfx950: M <= 128 (decode / small-batch shapes), dense bf16 A, MXFP W.
+//
+// With few rows of A the product is bound by streaming W from HBM, and the point of the fused path is
+// that W is read as one byte per element and never written back as bf16.  One workgroup owns 32 rows of
+// W (N / 32 workgroups, several resident per CU) and walks K in macro steps of 128:
+//   * W codes come as whole 128-byte lines (lane = 16 codes of one row), are composed to bf16 in
+//     registers and written to LDS in the MFMA fragment-friendly layout below;
+//   * the matching 128 k of all A rows come global -> LDS by DMA (whole lines; A is small and stays in L2);
+//   * the macro step's eight 16-k MFMA steps are split over the four wavefronts (two each, all rows),
+//     so every wavefront ends with partial sums that are added through LDS once, at the end.
+// The loads of macro step m+D (W codes and scales into registers, A by DMA into one of D+1 LDS stages) are issued
+// before the MFMAs of step m; HBM latency is covered by this depth, since a CU holds fewer than two of these
+// workgroups when N / 32 is a few hundred.  All of them are inline asm, waited for with a counted s_waitcnt
+// (vector memory completes in issue order).  The composed W is double buffered; one barrier per macro step.
+//
+// LDS rows are 256 bytes (128 k of bf16), the 16-byte chunk c of row r at position c ^ (r & 15): the LDS
+// serves a 128-bit read 16 lanes at a time from 64 banks, and 16 consecutive rows then hit 16 different
+// bank groups.
+// (included from gemm_impl.h, inside namespace mase, after gemm_tall.h, whose asm helpers it uses)
+
+constexpr int SK_N = 32;        // W rows per workgroup
+constexpr int SK_MAC = 128;     // k per macro step
+constexpr int SK_ROW = 256;     // bytes per LDS row
+
+template <class FW, int DT_OUT, int MT, int D>
+__global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
+    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K) {
+    constexpr int R = D + 1;                                  // ring size: registers sets of W, LDS stages of A
+    constexpr int OPS = 2 * MT + 2;                           // vector-memory operations per wavefront and macro step
+    constexpr int A_STAGE = 32 * MT * SK_ROW, W_STAGE = SK_N * SK_ROW;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    uint8_t* const lds_a = lds;                    // [R][32 MT rows][256 B]
+    uint8_t* const lds_w = lds + R * A_STAGE;      // [2][32 rows][256 B]
+    const uint32_t lds_a_addr = (uint32_t)(uintptr_t)lds;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n0 = blockIdx.x * SK_N;
+    const int kblocks = K / 32, nmac = K / SK_MAC;
+
+    // A DMA: instruction i (of 8 MT per macro step, 2 MT per wavefront) covers tile rows 4i .. 4i+3; lane l fills
+    // position l & 15 of row 4i + (l >> 4), which must hold chunk (l & 15) ^ (row & 15).  Rows past M re-read row M-1.
+    uint32_t a_voff[2 * MT];
+#pragma unroll
+    for (int j = 0; j < 2 * MT; ++j) {
+        const int row = 4 * (wave * 2 * MT + j) + (lane >> 4);
+        a_voff[j] = (uint32_t)min(row, M - 1) * (uint32_t)K * 2u + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
+    }
+    // W: the wavefront loads rows 8w .. 8w+7 as whole lines, lane = 16 codes (16 k) of row 8w + (l >> 3)
+    const int w_row = wave * 8 + (lane >> 3), w_chunk = lane & 7;
+    const uint8_t* const w_base = w_elements + (size_t)(n0 + wave * 8) * K;          // wave-uniform
+    const uint8_t* const ws_base = w_scales + (size_t)(n0 + wave * 8) * kblocks;
+    const uint32_t w_voff = (uint32_t)(lane >> 3) * (uint32_t)K + (uint32_t)w_chunk * 16u;
+    const uint32_t ws_voff = (uint32_t)(lane >> 3) * (uint32_t)kblocks + (uint32_t)(w_chunk >> 1);
+    const uint32_t w_lds_off0 = (uint32_t)w_row * SK_ROW + (uint32_t)(((2 * w_chunk) ^ (w_row & 15)) * 16);
+    const uint32_t w_lds_off1 = (uint32_t)w_row * SK_ROW + (uint32_t)(((2 * w_chunk + 1) ^ (w_row & 15)) * 16);
+    // fragment reads: lane (g = l >> 5, r = l & 31) reads chunk 2q + g of row 32 t + r; this wavefront owns q = 2w, 2w+1
+    uint32_t f_off[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+        f_off[e] = (uint32_t)(lane & 31) * SK_ROW + (uint32_t)(((2 * (2 * wave + e) + (lane >> 5)) ^ (lane & 15)) * 16);
+
+    floatx16 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
+
+    u32x4 w_raw[R];
+    uint32_t w_scale[R];
+    // loads of macro step `mac` into ring slot `slot_c`; past the end the last macro step is read again (unused),
+    // which keeps the number of operations per step, and with it the wait counts, the same
+    auto issue_loads = [&](int mac, auto slot_c) {
+        constexpr int slot = decltype(slot_c)::value;
+        const int mc = min(mac, nmac - 1);
+        async_load16(w_raw[slot], w_voff, w_base + (size_t)mc * SK_MAC);
+        async_load_u8(w_scale[slot], ws_voff, ws_base + mc * (SK_MAC / 32));
+        const uint8_t* const a_src = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)mc * (SK_MAC * 2);
+        const uint32_t dst = lds_a_addr + (uint32_t)slot * A_STAGE + (uint32_t)wave * (2 * MT * 1024);
+#pragma unroll
+        for (int j = 0; j < 2 * MT; ++j) dma_1kb(dst + j * 1024, a_voff[j], a_src);
+    };
+    // the loads of the macro step in ring slot `slot_c` have arrived (D - 1 younger steps may still be in flight):
+    // compose its W into stage `mac & 1`
+    auto stage_w = [&](int mac, auto slot_c) {
+        constexpr int slot = decltype(slot_c)::value;
+        wait_vmcnt<(D - 1) * OPS>(w_raw[slot], w_scale[slot]);
+        uint4 lo, hi;
+        Composer<FW>::template compose16<true>(make_uint4(w_raw[slot].x, w_raw[slot].y, w_raw[slot].z, w_raw[slot].w),
+                                               w_scale[slot], lo, hi);
+        uint8_t* const st = lds_w + (mac & 1) * W_STAGE;
+        *reinterpret_cast<uint4*>(st + w_lds_off0) = lo;
+        *reinterpret_cast<uint4*>(st + w_lds_off1) = hi;
+    };
+
+    static_for<D>([&](auto d_c) { issue_loads(decltype(d_c)::value, d_c); });
+    stage_w(0, IntC<0>{});
+    for (int base = 0; base < nmac; base += R) {
+        static_for<R>([&](auto r_c) {
+            constexpr int r = decltype(r_c)::value;
+            const int mac = base + r;
+            if (mac < nmac) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront's LDS reads and writes are done
+                __builtin_amdgcn_s_barrier();        // W stage mac & 1 and A slot r are complete; slot r - 1 is no longer read
+                issue_loads(mac + D, IntC<(r + D) % R>{});
+                const uint8_t* const pa = lds_a + r * A_STAGE;
+                const uint8_t* const pw = lds_w + (mac & 1) * W_STAGE;
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const bf16x8 wf = *reinterpret_cast<const bf16x8*>(pw + f_off[e]);
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) {
+                        const bf16x8 af = *reinterpret_cast<const bf16x8*>(pa + t * (32 * SK_ROW) + f_off[e]);
+                        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, af, acc[t], 0, 0, 0);
+                    }
+                }
+                stage_w(mac + 1, IntC<(r + 1) % R>{});  // (past the end: composes the re-read step into the unused stage)
+            }
+        });
+    }
+    // the look-ahead loads still target LDS and registers: let them finish
+    wait_vmcnt<0>(w_raw[0], w_scale[0]);
+
+    // ---- add the four wavefronts' partial sums: wavefronts 1..3 park theirs in LDS ([w-1][t][v][lane]), 0 adds
+    __syncthreads();  // every fragment read is done: the stages can be reused
+    float* const red = reinterpret_cast<float*>(lds);
+    if (wave != 0) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) red[(((wave - 1) * MT + t) * 16 + v) * 64 + lane] = acc[t][v];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll 1
+    for (int w = 0; w < 3; ++w)  // one wavefront's sums at a time: all three at once would cost 48 MT registers
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[t][v] += red[((w * MT + t) * 16 + v) * 64 + lane];
+
+    // lane holds, for m-tile t and g = 0..3, y[m][n .. n+3] with m = 32 t + lane % 32, n = n0 + 8 g + 4 (lane / 32)
+    const bool vec_ok = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int n = n0 + 8 * g + 4 * (lane >> 5);
+        float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (bias)
+            for (int t = 0; t < 4; ++t) b[t] = load_bias(bias, bias_dtype, n + t);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int m = 32 * t + (lane & 31);
+            if (m < M) {
+                const float r[4] = {acc[t][4 * g] + b[0], acc[t][4 * g + 1] + b[1], acc[t][4 * g + 2] + b[2], acc[t][4 * g + 3] + b[3]};
+                store_out4<DT_OUT>(y, (int64_t)m * N + n, r, vec_ok, 4);
+            }
+        }
+    }
+}
+
+template <class FW, int DT_OUT>
+int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
+                       void* y, int M, int N, int K, hipStream_t s) {
+    const dim3 grid((unsigned)(N / SK_N));
+    auto go = [&](auto mt_c) {
+        constexpr int MT = decltype(mt_c)::value;
+        constexpr int D = MT == 1 ? 4 : MT == 2 ? 2 : 1;  // look-ahead in macro steps: the A stages must leave LDS for two workgroups per CU
+        constexpr int lds_bytes = (D + 1) * 32 * MT * SK_ROW + 2 * SK_N * SK_ROW;
+        auto kern = mxfp_gemm_skinny_kernel<FW, DT_OUT, MT, D>;
+        static bool attr_done = false;
+        if (!attr_done) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
+            attr_done = true;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
+                           bias, bias_dtype, y, M, N, K);
+        return check_launch("mxfp_gemm");
+    };
+    if (M <= 32) return go(IntC<1>{});
+    if (M <= 64) return go(IntC<2>{});
+    return go(IntC<4>{});
+}

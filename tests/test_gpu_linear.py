@@ -211,6 +211,51 @@ def test_gemm_large_tile_special_values(mh):
     assert y[:, ~bad].isfinite().all()
 
 
+@pytest.mark.parametrize("MNK,w_tag,odt,with_bias", [
+    ((1, 1024, 128), "MXFP8_E4M3_fn", torch.bfloat16, False),     # one row, a single macro step
+    ((16, 2048, 640), "OCP_MXFP4_E2M1", torch.float32, True),     # 5 macro steps: the look-ahead ring wraps once
+    ((33, 512, 1024), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # two m-tiles, the second almost empty
+    ((64, 96, 256), "MXFP8_E5M2_fn", torch.float16, False),       # three workgroups
+    ((100, 1024, 2048), "OCP_MXFP6_E2M3", torch.bfloat16, False), # four m-tiles, ragged
+    ((128, 4096, 1536), "MXFP8_E4M3_fn", torch.float32, True),
+])
+def test_gemm_few_rows(mh, MNK, w_tag, odt, with_bias):
+    """M <= 128 with N % 32 == 0 and K % 128 == 0 takes the kernel that streams W once (one workgroup per 32 rows of W,
+    K split over its wavefronts, partial sums added through LDS)."""
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
+    we, wm = PRESETS[w_tag]
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    w_sc, w_el = oracle.extract_mxfp(w, 32, we, wm)
+    w_dq = oracle.compose_mxfp(w_sc, w_el, 32, we, wm, True, torch.bfloat16).view(N, K)
+    y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, w_tag),
+                         None if b is None else b.to(DEV), M, N, K, odt)
+    assert y.shape == (M, N) and y.dtype == odt
+    y_ref = oracle.matmul_nt(x_dq, w_dq)
+    if b is not None:
+        y_ref = y_ref + b.float()
+    assert rel_fro(y, y_ref.to(odt)) <= (1e-5 if odt == torch.float32 else REL_FRO_TOL)
+
+
+def test_gemm_few_rows_special_values(mh):
+    M, N, K = 8, 256, 384
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    w[77, 300] = float("inf")
+    w_sc, w_el = oracle.extract_mxfp(w, 32, 4, 3)
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), None,
+                         M, N, K, torch.float32).cpu()
+    assert y[:, 77].isnan().all()
+    keep = torch.ones(N, dtype=torch.bool)
+    keep[77] = False
+    assert y[:, keep].isfinite().all()
+
+
 def test_config_c4_full_size(mh):
     """x [16384,4096] . W [14336,4096]^T, both MXFP8 E4M3.  The whole output is compared with
     the GPU dequantize-then-matmul (fp32 accumulate, bf16 out); a sample of rows and columns
