@@ -543,8 +543,9 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     }
     if constexpr (A_MODE == 0 && DT_OUT != F32) {
         // tall tiles: dense A, 16-bit output, whole tiles only, enough of them to occupy the chip
-        const int64_t tall_tiles = (int64_t)(M / UM) * (N / UN);
-        if (fits32 && M % UM == 0 && N % UN == 0 && K % UMAC == 0 && tall_tiles >= TALL_MIN_TILES &&
+        const int tall_tiles_m = (M + UM - 1) / UM;
+        const int64_t tall_tiles = (int64_t)tall_tiles_m * (N / UN);
+        if (fits32 && M >= UM && N % UN == 0 && K % UMAC == 0 && tall_tiles >= TALL_MIN_TILES &&
             (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
             (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0) {
             auto kern = mxfp_gemm_tall_kernel<FW, DT_OUT>;
@@ -558,7 +559,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             if (cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
             hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                               w_elements, bias, bias_dtype, y, M, N, K, M / UM, N / UN);
+                               w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN);
             return check_launch("mxfp_gemm");
         }
     }

@@ -169,7 +169,9 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         const int rows = min(tiles_m - first_m, GROUP);
         const int rr = pos % in_group;
         TallTile t;
-        t.m0 = (first_m + rr % rows) * UM;
+        // M need not be a multiple of 512: the last tile row is shifted up to end at row M - 1; the rows it shares with
+        // its neighbour are computed twice, identically
+        t.m0 = min((first_m + rr % rows) * UM, M - UM);
         t.n0 = (rr / rows) * UN;
         t.a = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)(t.m0 + wave * 128) * K) * 2;
         t.w = w_elements + (size_t)t.n0 * K;

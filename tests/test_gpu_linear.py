@@ -146,6 +146,8 @@ def test_mxfp_linear_vs_cpu_reference_path(mh):
     ((8192, 2048, 1024), "OCP_MXFP4_E2M1", torch.float16),   # one tile per workgroup, fp16 output
     ((1536, 16384, 256), "MXFP8_E5M2_fn", torch.bfloat16),   # 3 tile rows: the last group of tile rows is a single row
     ((16384, 1024, 512), "OCP_MXFP6_E2M3", torch.bfloat16),  # tall problem: 32 x 8 tiles
+    ((1000, 8192, 256), "MXFP8_E4M3_fn", torch.bfloat16),    # M not a multiple of 512: the last tile row is shifted up
+    ((3001, 2048, 384), "OCP_MXFP6_E3M2", torch.float16),    # 6 tile rows, the last one overlapping by 71 rows
 ])
 def test_gemm_large_tile_shapes(mh, MNK, w_tag, odt):
     """Shapes that take the 512 x 128 tile kernel (dense A, 16-bit output, no bias, whole tiles): the whole output
