@@ -19,47 +19,59 @@
 // (included from gemm_impl.h, inside namespace mase, after gemm_tall.h, whose asm helpers it uses)
 
 constexpr int SK_N = 32;        // W rows per workgroup
-constexpr int SK_MAC = 128;     // k per macro step
-constexpr int SK_ROW = 256;     // bytes per LDS row
+constexpr int SK_MAC = 128;     // k granularity the launcher requires
 
-template <class FW, int DT_OUT, int MT, int D>
+template <class FW, int DT_OUT, int MT, int D, int L, int AR>
 __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
     const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K) {
+    // L = 128-byte lines of W codes per row and macro step: the macro step covers KM = 128 L k, LDS rows are 256 L bytes
+    // AR = rows of A kept per m-tile: 32, or 16 when M <= 16 (rows 16..31 of the MFMA operand then re-read rows 0..15)
+    static_assert(AR == 32 || (AR == 16 && MT == 1), "16-row stages only with one m-tile");
+    constexpr int KM = 128 * L, ROW = 2 * KM, CH = ROW / 16;
     constexpr int R = D + 1;                                  // ring size: registers sets of W, LDS stages of A
-    constexpr int OPS = 2 * MT + 2;                           // vector-memory operations per wavefront and macro step
-    constexpr int A_STAGE = 32 * MT * SK_ROW, W_STAGE = SK_N * SK_ROW;
+    constexpr int A_DMAS = AR * MT * ROW / 1024 / 4;          // A DMAs per wavefront and macro step
+    constexpr int OPS = A_DMAS + 2 * L;                       // vector-memory operations per wavefront and macro step
+    constexpr int A_STAGE = AR * MT * ROW, W_STAGE = SK_N * ROW;
+    constexpr int QW = KM / 16 / 4;                           // 16-k MFMA steps per wavefront and macro step
+    static_assert((D - 1) * OPS < 64, "vmcnt is a 6-bit counter");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    uint8_t* const lds_a = lds;                    // [R][32 MT rows][256 B]
-    uint8_t* const lds_w = lds + R * A_STAGE;      // [2][32 rows][256 B]
+    uint8_t* const lds_a = lds;                    // [R][32 MT rows][ROW]
+    uint8_t* const lds_w = lds + R * A_STAGE;      // [2][32 rows][ROW]
     const uint32_t lds_a_addr = (uint32_t)(uintptr_t)lds;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n0 = blockIdx.x * SK_N;
-    const int kblocks = K / 32, nmac = K / SK_MAC;
+    const int kblocks = K / 32, nmac = K / KM;
 
-    // A DMA: instruction i (of 8 MT per macro step, 2 MT per wavefront) covers tile rows 4i .. 4i+3; lane l fills
-    // position l & 15 of row 4i + (l >> 4), which must hold chunk (l & 15) ^ (row & 15).  Rows past M re-read row M-1.
-    uint32_t a_voff[2 * MT];
+    // A DMA: an instruction moves 1 KB = 1024 / ROW rows; lane l fills position l % CH of row (1 KB index) * (1024 / ROW)
+    // + l / CH, which must hold chunk (l % CH) ^ (row & 15).  Rows past M re-read row M - 1.
+    uint32_t a_voff[A_DMAS];
 #pragma unroll
-    for (int j = 0; j < 2 * MT; ++j) {
-        const int row = 4 * (wave * 2 * MT + j) + (lane >> 4);
-        a_voff[j] = (uint32_t)min(row, M - 1) * (uint32_t)K * 2u + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
+    for (int j = 0; j < A_DMAS; ++j) {
+        const int row = (wave * A_DMAS + j) * (1024 / ROW) + lane / CH;
+        a_voff[j] = (uint32_t)min(row, M - 1) * (uint32_t)K * 2u + (uint32_t)((((lane % CH) ^ (row & 15))) * 16);
     }
-    // W: the wavefront loads rows 8w .. 8w+7 as whole lines, lane = 16 codes (16 k) of row 8w + (l >> 3)
+    // W: the wavefront loads rows 8w .. 8w+7 as whole lines, lane = 16 codes (16 k) of row 8w + (l >> 3), L times
     const int w_row = wave * 8 + (lane >> 3), w_chunk = lane & 7;
     const uint8_t* const w_base = w_elements + (size_t)(n0 + wave * 8) * K;          // wave-uniform
     const uint8_t* const ws_base = w_scales + (size_t)(n0 + wave * 8) * kblocks;
     const uint32_t w_voff = (uint32_t)(lane >> 3) * (uint32_t)K + (uint32_t)w_chunk * 16u;
     const uint32_t ws_voff = (uint32_t)(lane >> 3) * (uint32_t)kblocks + (uint32_t)(w_chunk >> 1);
-    const uint32_t w_lds_off0 = (uint32_t)w_row * SK_ROW + (uint32_t)(((2 * w_chunk) ^ (w_row & 15)) * 16);
-    const uint32_t w_lds_off1 = (uint32_t)w_row * SK_ROW + (uint32_t)(((2 * w_chunk + 1) ^ (w_row & 15)) * 16);
-    // fragment reads: lane (g = l >> 5, r = l & 31) reads chunk 2q + g of row 32 t + r; this wavefront owns q = 2w, 2w+1
-    uint32_t f_off[2];
+    uint32_t w_lds_off[L][2];
 #pragma unroll
-    for (int e = 0; e < 2; ++e)
-        f_off[e] = (uint32_t)(lane & 31) * SK_ROW + (uint32_t)(((2 * (2 * wave + e) + (lane >> 5)) ^ (lane & 15)) * 16);
+    for (int li = 0; li < L; ++li)
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+            w_lds_off[li][e] = (uint32_t)w_row * ROW + (uint32_t)(((16 * li + 2 * w_chunk + e) ^ (w_row & 15)) * 16);
+    // fragment reads: lane (g = l >> 5, r = l & 31) reads chunk 2q + g of row 32 t + r; this wavefront owns q = QW w .. QW w + QW - 1
+    uint32_t f_off[QW], fa_off[QW];
+#pragma unroll
+    for (int e = 0; e < QW; ++e) {
+        f_off[e] = (uint32_t)(lane & 31) * ROW + (uint32_t)(((2 * (QW * wave + e) + (lane >> 5)) ^ (lane & 15)) * 16);
+        fa_off[e] = (uint32_t)(lane & (AR - 1)) * ROW + (uint32_t)(((2 * (QW * wave + e) + (lane >> 5)) ^ (lane & 15)) * 16);
+    }
 
     floatx16 acc[MT];
 #pragma unroll
@@ -67,31 +79,43 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
 
-    u32x4 w_raw[R];
-    uint32_t w_scale[R];
+    u32x4 w_raw[R][L];
+    uint32_t w_scale[R][L];
+    // workgroups start at different macro steps of K (and wrap around): at any moment they then read different
+    // columns of W, i.e. addresses that do not all differ by multiples of the row pitch and so spread over the
+    // memory channels
+    const int rot = (int)(blockIdx.x % (unsigned)nmac);
     // loads of macro step `mac` into ring slot `slot_c`; past the end the last macro step is read again (unused),
     // which keeps the number of operations per step, and with it the wait counts, the same
     auto issue_loads = [&](int mac, auto slot_c) {
         constexpr int slot = decltype(slot_c)::value;
-        const int mc = min(mac, nmac - 1);
-        async_load16(w_raw[slot], w_voff, w_base + (size_t)mc * SK_MAC);
-        async_load_u8(w_scale[slot], ws_voff, ws_base + mc * (SK_MAC / 32));
-        const uint8_t* const a_src = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)mc * (SK_MAC * 2);
-        const uint32_t dst = lds_a_addr + (uint32_t)slot * A_STAGE + (uint32_t)wave * (2 * MT * 1024);
+        int mc = min(mac, nmac - 1) + rot;
+        if (mc >= nmac) mc -= nmac;
 #pragma unroll
-        for (int j = 0; j < 2 * MT; ++j) dma_1kb(dst + j * 1024, a_voff[j], a_src);
+        for (int li = 0; li < L; ++li) {
+            async_load16(w_raw[slot][li], w_voff, w_base + (size_t)mc * KM + li * 128);
+            async_load_u8(w_scale[slot][li], ws_voff, ws_base + mc * (KM / 32) + li * 4);
+        }
+        const uint8_t* const a_src = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)mc * (KM * 2);
+        const uint32_t dst = lds_a_addr + (uint32_t)slot * A_STAGE + (uint32_t)wave * (A_DMAS * 1024);
+#pragma unroll
+        for (int j = 0; j < A_DMAS; ++j) dma_1kb(dst + j * 1024, a_voff[j], a_src);
     };
     // the loads of the macro step in ring slot `slot_c` have arrived (D - 1 younger steps may still be in flight):
     // compose its W into stage `mac & 1`
     auto stage_w = [&](int mac, auto slot_c) {
         constexpr int slot = decltype(slot_c)::value;
-        wait_vmcnt<(D - 1) * OPS>(w_raw[slot], w_scale[slot]);
-        uint4 lo, hi;
-        Composer<FW>::template compose16<true>(make_uint4(w_raw[slot].x, w_raw[slot].y, w_raw[slot].z, w_raw[slot].w),
-                                               w_scale[slot], lo, hi);
+        wait_vmcnt<(D - 1) * OPS>(w_raw[slot][0], w_scale[slot][0]);
+        if (L == 2) wait_vmcnt<(D - 1) * OPS>(w_raw[slot][L - 1], w_scale[slot][L - 1]);
         uint8_t* const st = lds_w + (mac & 1) * W_STAGE;
-        *reinterpret_cast<uint4*>(st + w_lds_off0) = lo;
-        *reinterpret_cast<uint4*>(st + w_lds_off1) = hi;
+#pragma unroll
+        for (int li = 0; li < L; ++li) {
+            uint4 lo, hi;
+            Composer<FW>::template compose16<true>(make_uint4(w_raw[slot][li].x, w_raw[slot][li].y, w_raw[slot][li].z, w_raw[slot][li].w),
+                                                   w_scale[slot][li], lo, hi);
+            *reinterpret_cast<uint4*>(st + w_lds_off[li][0]) = lo;
+            *reinterpret_cast<uint4*>(st + w_lds_off[li][1]) = hi;
+        }
     };
 
     static_for<D>([&](auto d_c) { issue_loads(decltype(d_c)::value, d_c); });
@@ -106,21 +130,40 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
                 issue_loads(mac + D, IntC<(r + D) % R>{});
                 const uint8_t* const pa = lds_a + r * A_STAGE;
                 const uint8_t* const pw = lds_w + (mac & 1) * W_STAGE;
+                if constexpr (MT <= 2) {
+                    // few MFMAs: the fragment reads go out, the next step's W is composed while they are in flight, then
+                    // the MFMAs (nothing waits for their results before the next step's MFMAs)
+                    bf16x8 wf[QW], af[QW][MT];
 #pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const bf16x8 wf = *reinterpret_cast<const bf16x8*>(pw + f_off[e]);
+                    for (int e = 0; e < QW; ++e) {
+                        wf[e] = *reinterpret_cast<const bf16x8*>(pw + f_off[e]);
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        const bf16x8 af = *reinterpret_cast<const bf16x8*>(pa + t * (32 * SK_ROW) + f_off[e]);
-                        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, af, acc[t], 0, 0, 0);
+                        for (int t = 0; t < MT; ++t) af[e][t] = *reinterpret_cast<const bf16x8*>(pa + t * (32 * ROW) + fa_off[e]);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
+                    stage_w(mac + 1, IntC<(r + 1) % R>{});  // (past the end: composes the re-read step into the unused stage)
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int e = 0; e < QW; ++e)
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[e], af[e][t], acc[t], 0, 0, 0);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < QW; ++e) {
+                        const bf16x8 wf = *reinterpret_cast<const bf16x8*>(pw + f_off[e]);
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) {
+                            const bf16x8 af = *reinterpret_cast<const bf16x8*>(pa + t * (32 * ROW) + fa_off[e]);
+                            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, af, acc[t], 0, 0, 0);
+                        }
+                    }
+                    stage_w(mac + 1, IntC<(r + 1) % R>{});
                 }
-                stage_w(mac + 1, IntC<(r + 1) % R>{});  // (past the end: composes the re-read step into the unused stage)
             }
         });
     }
     // the look-ahead loads still target LDS and registers: let them finish
-    wait_vmcnt<0>(w_raw[0], w_scale[0]);
+    wait_vmcnt<0>(w_raw[0][0], w_scale[0][0]);
 
     // ---- add the four wavefronts' partial sums: wavefronts 1..3 park theirs in LDS ([w-1][t][v][lane]), 0 adds
     __syncthreads();  // every fragment read is done: the stages can be reused
@@ -159,15 +202,138 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// M <= 64: the same product with no workgroup barrier in the K loop.  Wavefront w of a workgroup owns the k
+// range [32 w, 32 w + 32) of every 128-k macro step, for all 32 rows of W and all rows of A:
+//   * a lane (g = l >> 5, r = l & 31) loads the 16 codes of W row r at k 16 g .. 16 g + 15 of that range, composes
+//     them in registers, and uses codes 0..7 / 8..15 directly as its MFMA operand of the range's first / second
+//     16-k step: an MFMA may pair the k values of a step in any order as long as both operands use the same one,
+//     so the A fragment of lane (g, r') is read from k 16 g + 8 e .. + 7 as well;
+//   * the matching 64-byte pieces of the A rows come by DMA into a ring of LDS slots private to the wavefront.
+// Every wavefront is its own stream with loads D macro steps ahead; the partial sums meet once at the end.
+template <class FW, int DT_OUT, int MT, int R>
+__global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_stream_kernel(
+    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K) {
+    constexpr int D = R - 1;                      // look-ahead in macro steps
+    constexpr int OPS = 2 + 2 * MT;               // vector-memory operations per wavefront and macro step
+    constexpr int SLOT = 32 * MT * 64;            // one macro step's A piece of a wavefront: 32 MT rows x 64 B
+    static_assert(D * OPS < 64, "vmcnt is a 6-bit counter");
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n0 = blockIdx.x * SK_N;
+    const int kblocks = K / 32, nmac = K / SK_MAC;
+    uint8_t* const ring = lds + wave * (R * SLOT);                                  // [R][32 MT rows][64 B]
+    const uint32_t ring_addr = (uint32_t)(uintptr_t)lds + (uint32_t)wave * (R * SLOT);
+
+    // A DMA: instruction j (of 2 MT) covers rows 16 j .. 16 j + 15; lane l fills position l & 3 of row 16 j + (l >> 2),
+    // which must hold chunk (l & 3) ^ ((row >> 2) & 3).  Rows past M re-read row M - 1.
+    uint32_t a_voff[2 * MT];
+#pragma unroll
+    for (int j = 0; j < 2 * MT; ++j) {
+        const int row = 16 * j + (lane >> 2);
+        a_voff[j] = (uint32_t)min(row, M - 1) * (uint32_t)K * 2u + (uint32_t)(((lane & 3) ^ ((row >> 2) & 3)) * 16);
+    }
+    const uint8_t* const a_base = reinterpret_cast<const uint8_t*>(a_dense) + wave * 64;       // k = 32 w
+    const uint8_t* const w_base = w_elements + (size_t)n0 * K + wave * 32;
+    const uint8_t* const ws_base = w_scales + (size_t)n0 * kblocks + wave;
+    const uint32_t w_voff = (uint32_t)(lane & 31) * (uint32_t)K + (uint32_t)(lane >> 5) * 16u;
+    const uint32_t ws_voff = (uint32_t)(lane & 31) * (uint32_t)kblocks;
+    // A fragment of 16-k step e: chunk 2 g + e of row 32 t + r
+    uint32_t f_off[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+        f_off[e] = (uint32_t)(lane & 31) * 64u + (uint32_t)(((2 * (lane >> 5) + e) ^ ((lane >> 2) & 3)) * 16);
+
+    floatx16 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
+
+    u32x4 w_raw[R];
+    uint32_t w_scale[R];
+    // past the end the last macro step is read again (unused): the number of operations per step stays the same
+    auto issue_loads = [&](int mac, auto slot_c) {
+        constexpr int slot = decltype(slot_c)::value;
+        const int mc = min(mac, nmac - 1);
+        async_load16(w_raw[slot], w_voff, w_base + (size_t)mc * SK_MAC);
+        async_load_u8(w_scale[slot], ws_voff, ws_base + mc * (SK_MAC / 32));
+        const uint8_t* const a_src = a_base + (size_t)mc * (SK_MAC * 2);
+#pragma unroll
+        for (int j = 0; j < 2 * MT; ++j) dma_1kb(ring_addr + (uint32_t)slot * SLOT + j * 1024, a_voff[j], a_src);
+    };
+
+    static_for<D>([&](auto d_c) { issue_loads(decltype(d_c)::value, d_c); });
+    for (int base = 0; base < nmac; base += R) {
+        static_for<R>([&](auto r_c) {
+            constexpr int r = decltype(r_c)::value;
+            const int mac = base + r;
+            if (mac < nmac) {
+                issue_loads(mac + D, IntC<(r + D) % R>{});            // into the slot consumed one step ago
+                wait_vmcnt<D * OPS>(w_raw[r], w_scale[r]);             // this step's loads have arrived
+                uint4 lo, hi;
+                Composer<FW>::template compose16<true>(make_uint4(w_raw[r].x, w_raw[r].y, w_raw[r].z, w_raw[r].w), w_scale[r], lo, hi);
+                const bf16x8 wf0 = __builtin_bit_cast(bf16x8, lo), wf1 = __builtin_bit_cast(bf16x8, hi);
+                const uint8_t* const pa = ring + r * SLOT;
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const bf16x8 af0 = *reinterpret_cast<const bf16x8*>(pa + t * 2048 + f_off[0]);
+                    const bf16x8 af1 = *reinterpret_cast<const bf16x8*>(pa + t * 2048 + f_off[1]);
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf0, af0, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf1, af1, acc[t], 0, 0, 0);
+                }
+                // the slot is handed back to the DMA engine in the next step: its reads must have returned
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+            }
+        });
+    }
+    wait_vmcnt<0>(w_raw[0], w_scale[0]);  // the look-ahead loads still target LDS and registers
+
+    // ---- add the four wavefronts' partial sums: wavefronts 1..3 park theirs in LDS ([w-1][t][v][lane]), 0 adds
+    __syncthreads();
+    float* const red = reinterpret_cast<float*>(lds);
+    if (wave != 0) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) red[(((wave - 1) * MT + t) * 16 + v) * 64 + lane] = acc[t][v];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll 1
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[t][v] += red[((w * MT + t) * 16 + v) * 64 + lane];
+    const bool vec_ok = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int n = n0 + 8 * g + 4 * (lane >> 5);
+        float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (bias)
+            for (int t = 0; t < 4; ++t) b[t] = load_bias(bias, bias_dtype, n + t);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int m = 32 * t + (lane & 31);
+            if (m < M) {
+                const float r[4] = {acc[t][4 * g] + b[0], acc[t][4 * g + 1] + b[1], acc[t][4 * g + 2] + b[2], acc[t][4 * g + 3] + b[3]};
+                store_out4<DT_OUT>(y, (int64_t)m * N + n, r, vec_ok, 4);
+            }
+        }
+    }
+}
+
 template <class FW, int DT_OUT>
 int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
                        void* y, int M, int N, int K, hipStream_t s) {
     const dim3 grid((unsigned)(N / SK_N));
-    auto go = [&](auto mt_c) {
-        constexpr int MT = decltype(mt_c)::value;
-        constexpr int D = MT == 1 ? 4 : MT == 2 ? 2 : 1;  // look-ahead in macro steps: the A stages must leave LDS for two workgroups per CU
-        constexpr int lds_bytes = (D + 1) * 32 * MT * SK_ROW + 2 * SK_N * SK_ROW;
-        auto kern = mxfp_gemm_skinny_kernel<FW, DT_OUT, MT, D>;
+    auto go_stream = [&](auto mt_c, auto r_c) {
+        constexpr int MT = decltype(mt_c)::value, R = decltype(r_c)::value;
+        constexpr int lds_bytes = 4 * R * 32 * MT * 64;   // >= the 12 MT KB the final reduction needs
+        auto kern = mxfp_gemm_stream_kernel<FW, DT_OUT, MT, R>;
         static bool attr_done = false;
         if (!attr_done) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -178,6 +344,39 @@ int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8
                            bias, bias_dtype, y, M, N, K);
         return check_launch("mxfp_gemm");
     };
+    auto go = [&](auto mt_c) {
+        constexpr int MT = decltype(mt_c)::value;
+        // look-ahead D (macro steps) and lines per row L: the A stages must leave LDS for two workgroups per CU
+        constexpr int D = MT == 1 ? 4 : MT == 2 ? 2 : 1, L = 1, AR = 32;
+        constexpr int lds_bytes = (D + 1) * AR * MT * 256 * L + 2 * SK_N * 256 * L;
+        auto kern = mxfp_gemm_skinny_kernel<FW, DT_OUT, MT, D, L, AR>;
+        static bool attr_done = false;
+        if (!attr_done) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
+            attr_done = true;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
+                           bias, bias_dtype, y, M, N, K);
+        return check_launch("mxfp_gemm");
+    };
+    // few workgroups (at most one per two CUs): the barrier-free kernel, whose weakness is address-unit load per CU
+    if (M <= 32 && N / SK_N <= 128) return go_stream(IntC<1>{}, IntC<6>{});
+    if (M <= 64 && N / SK_N <= 128) return go_stream(IntC<2>{}, IntC<4>{});
+    if (M <= 16) {  // 16-row A stages leave LDS for a look-ahead of 8 macro steps
+        constexpr int D = 8, L = 1, AR = 16;
+        constexpr int lds_bytes = (D + 1) * AR * 256 * L + 2 * SK_N * 256 * L;
+        auto kern = mxfp_gemm_skinny_kernel<FW, DT_OUT, 1, D, L, AR>;
+        static bool attr16_done = false;
+        if (!attr16_done) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
+            attr16_done = true;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
+                           bias, bias_dtype, y, M, N, K);
+        return check_launch("mxfp_gemm");
+    }
     if (M <= 32) return go(IntC<1>{});
     if (M <= 64) return go(IntC<2>{});
     return go(IntC<4>{});

@@ -220,6 +220,9 @@ def test_gemm_large_tile_special_values(mh):
     ((64, 96, 256), "MXFP8_E5M2_fn", torch.float16, False),       # three workgroups
     ((100, 1024, 2048), "OCP_MXFP6_E2M3", torch.bfloat16, False), # four m-tiles, ragged
     ((128, 4096, 1536), "MXFP8_E4M3_fn", torch.float32, True),
+    ((8, 8192, 1024), "MXFP8_E4M3_fn", torch.bfloat16, False),    # many workgroups, M <= 16: 16-row A stages, look-ahead 8
+    ((24, 6144, 896), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # many workgroups, 16 < M <= 32; 7 macro steps
+    ((64, 8192, 512), "OCP_MXFP4_E2M1", torch.float16, False),    # many workgroups, two m-tiles
 ])
 def test_gemm_few_rows(mh, MNK, w_tag, odt, with_bias):
     """M <= 128 with N % 32 == 0 and K % 128 == 0 takes the kernel that streams W once (one workgroup per 32 rows of W,
