@@ -1,0 +1,35 @@
+"""Static check of the kernels that count their own outstanding vector-memory operations (inline-asm loads,
+stores and DMAs waited for with hand-written s_waitcnt vmcnt(N)): a register spill would add scratch
+loads and stores that those counts do not know about, so these kernels must compile without scratch.
+Cross-compiles one weight format for gfx950 (no GPU needed)."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "mase-triton_amd", "csrc")
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not available")
+def test_counted_wait_kernels_use_no_scratch(tmp_path):
+    out = tmp_path / "gemm_w_e4m3.s"
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "--cuda-device-only", "-S", os.path.join(CSRC, "gemm_w_e4m3.hip"), "-o", str(out)]
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=600)
+    text = out.read_text()
+    names = re.findall(r"^(_ZN4mase\w+):\s*; @", text, re.M)
+    scratch = re.findall(r"; ScratchSize: (\d+)", text)
+    assert len(names) == len(scratch) > 0
+    checked = 0
+    for name, size in zip(names, scratch):
+        if any(tag in name for tag in ("gemm_tall_kernel", "gemm_skinny_kernel", "gemm_stream_kernel")):
+            assert int(size) == 0, f"{name} spills ({size} bytes of scratch): its s_waitcnt counts would be wrong"
+            checked += 1
+    assert checked >= 6
+    # M0 carries the LDS address of the DMAs between inline-asm statements: nothing else may write it
+    m0_writes = [ln for ln in text.splitlines() if re.search(r"\bm0\b", ln) and not ln.strip().startswith(";")]
+    assert all(re.match(r"\s*s_mov_b32 m0, s\d+", ln) for ln in m0_writes), m0_writes[:5]
