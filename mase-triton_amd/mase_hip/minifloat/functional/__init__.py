@@ -1,5 +1,5 @@
 from .cast import compose_minifloat_component, extract_minifloat_component, quantize_dequantize
-from .linear import minifloat_linear
+from .linear import gemm_weight_eligible, minifloat_linear, narrow_weight_codes
 from .matmul import minifloat_matmul
 
 __all__ = [

@@ -1,9 +1,17 @@
 """Minifloat-quantised linear (API of src/mase_triton/minifloat/functional/linear.py:108-171).
 
 ``layer_type`` spells which operands are quantised: X or Xq, W or Wq, B or Bq.  Activations
-are quantise-dequantised on the fly; weights and biases arrive as uint16 codes.  Both backends
-dequantise and call the dense GEMM; "fused" uses the single-pass QDQ kernel for activations
-(the reference raises NotImplementedError for it).
+are quantise-dequantised on the fly; weights and biases arrive as uint16 codes.
+
+backend="separate" follows the reference literally: dequantise every operand, then
+``torch.nn.functional.linear``.
+backend="fused" (NotImplementedError in the reference, :127-128) uses the single-pass QDQ kernel
+for activations and, when the weight format is one the MXFP GEMM decodes (at most 8 bits wide,
+see ``_GEMM_WEIGHT_FORMATS``), never builds the dense weight: a minifloat code is an MXFP
+element whose block scale is 2^0, so the codes are narrowed to one byte each and the GEMM
+composes them to bf16 in registers on their way to the MFMA units.  Such values have at most
+four significant bits, so the bf16 operands are exact and the result differs from "separate"
+only by the summation order.  Other formats fall back to compose + dense GEMM.
 """
 from __future__ import annotations
 
@@ -12,10 +20,55 @@ from typing import Literal
 import torch
 from torch import Tensor
 
+from ...mxfp import kernels as mxfp_kernels
+from ...mxfp.meta import MXFPMeta
+from .. import kernels
 from ..meta import MinifloatMeta, MinifloatTensorMeta
 from .cast import compose_minifloat_component, extract_minifloat_component, quantize_dequantize
 
 _LAYER_TYPES = ("XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq")
+
+
+# (exp_bits, frac_bits) of the element formats the GEMM kernels are instantiated for
+_GEMM_WEIGHT_FORMATS = ((4, 3), (5, 2), (2, 3), (3, 2), (2, 1))
+_UNIT_SCALE = 127  # E8M0 code of 2^0
+
+
+def narrow_weight_codes(w_element: Tensor, w_tensor_meta: MinifloatTensorMeta) -> tuple[Tensor, Tensor]:
+    """uint16 minifloat codes [N, K] -> (uint8 unit scales [N*K/32], uint8 codes [N, K]) for the
+    MXFP GEMM.  Only the low ``1 + exp_bits + frac_bits`` bits of a code carry meaning, as in
+    the decode of the reference (src/mase_triton/minifloat/fake.py:97-123)."""
+    assert w_element.dtype == torch.uint16
+    codes = w_element.contiguous().view(torch.uint8).view(*w_element.shape, 2)[..., 0].contiguous()
+    n_bits = w_tensor_meta.meta.n_bits
+    if n_bits < 8:
+        codes &= (1 << n_bits) - 1
+    scales = torch.full((w_element.numel() // 32,), _UNIT_SCALE, dtype=torch.uint8, device=w_element.device)
+    return scales, codes
+
+
+def gemm_weight_eligible(w_tensor_meta: MinifloatTensorMeta) -> bool:
+    """Can the MXFP GEMM decode this weight?  Finite-only format of a supported width, 2-D,
+    in_features a multiple of the 32-element block."""
+    m = w_tensor_meta.meta
+    return (m.is_finite and (m.exp_bits, m.frac_bits) in _GEMM_WEIGHT_FORMATS
+            and len(w_tensor_meta.shape) == 2 and w_tensor_meta.shape[1] % 32 == 0)
+
+
+def _gemm_eligible(x: Tensor, x_meta: MinifloatMeta | None, w_tensor_meta: MinifloatTensorMeta,
+                   b: Tensor | None) -> bool:
+    """The MFMA path computes on bf16 operands: a dense X must already be bf16, a quantised X
+    must be in a format bf16 holds exactly."""
+    if x.device.type != "cuda" or not gemm_weight_eligible(w_tensor_meta):
+        return False
+    if x.dtype not in (torch.bfloat16, torch.float32) or getattr(torch, w_tensor_meta.dtype) != x.dtype:
+        return False
+    if x_meta is None:
+        if x.dtype != torch.bfloat16:
+            return False
+    elif x_meta.exp_bits > 8 or x_meta.frac_bits > 7:
+        return False
+    return b is None or b.dtype in (torch.bfloat16, torch.float16, torch.float32)
 
 
 def _check_backend(backend: str) -> None:
@@ -34,20 +87,47 @@ def minifloat_linear(
     b_tensor_meta: MinifloatTensorMeta | None,
     layer_type: Literal["XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq"],
     backend: Literal["separate", "fused"],
+    _narrowed: tuple[Tensor, Tensor] | None = None,
 ) -> Tensor:
+    """``_narrowed`` (not in the reference's signature): the result of ``narrow_weight_codes``
+    for this weight, kept by a caller that applies the same weight many times."""
     if layer_type not in _LAYER_TYPES:
         raise NotImplementedError(f"Layer type {layer_type} not implemented")
     _check_backend(backend)
-    if layer_type.startswith("Xq"):
+    quantised_x = layer_type.startswith("Xq")
+    quantised_w = "Wq" in layer_type
+    if layer_type.endswith("Bq"):
+        # as in the reference (:22-25, :49-52): the quantised bias is used only when a dense `b`
+        # is passed as well; with b=None (what MinifloatLinearPTQ passes) no bias is added
+        b = compose_minifloat_component(b_element, b_tensor_meta) if b is not None else None
+
+    if backend == "fused" and quantised_w and _gemm_eligible(x, x_meta if quantised_x else None, w_tensor_meta, b):
+        if _narrowed is None:
+            _narrowed = narrow_weight_codes(w_element, w_tensor_meta)
+        return _fused_gemm(x, x_meta if quantised_x else None, _narrowed, w_tensor_meta, b)
+
+    if quantised_x:
         if backend == "fused":
             x = quantize_dequantize(x, x_meta)
         else:
             x_element, x_tensor_meta = extract_minifloat_component(x, x_meta)
             x = compose_minifloat_component(x_element, x_tensor_meta)
-    if "Wq" in layer_type:
+    if quantised_w:
         w = compose_minifloat_component(w_element, w_tensor_meta)
-    if layer_type.endswith("Bq"):
-        # as in the reference (:22-25, :49-52): the quantised bias is used only when a dense `b`
-        # is passed as well; with b=None (what MinifloatLinearPTQ passes) no bias is added
-        b = compose_minifloat_component(b_element, b_tensor_meta) if b is not None else None
     return torch.nn.functional.linear(x, w, b)
+
+
+def _fused_gemm(x: Tensor, x_meta: MinifloatMeta | None, narrowed: tuple[Tensor, Tensor],
+                w_tensor_meta: MinifloatTensorMeta, bias: Tensor | None) -> Tensor:
+    out_features, in_features = w_tensor_meta.shape
+    assert x.shape[-1] == in_features
+    scales, codes = narrowed
+    wm = w_tensor_meta.meta
+    gemm_meta = MXFPMeta(block_size=32, scale_exp_bits=8, element_exp_bits=wm.exp_bits,
+                         element_frac_bits=wm.frac_bits, element_is_finite=True, round_mode="rn")
+    a = x.reshape(-1, in_features)
+    if x_meta is not None:
+        a = kernels.quantize_dequantize(a, x_meta, torch.bfloat16)
+    y = mxfp_kernels.mxfp_gemm(a, None, None, None, scales, codes, gemm_meta, bias,
+                               a.shape[0], out_features, in_features, x.dtype)
+    return y.view(*x.shape[:-1], out_features)

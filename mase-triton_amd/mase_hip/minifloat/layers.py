@@ -66,6 +66,7 @@ class MinifloatLinearPTQ(nn.Module):
         self.weight = self.bias = None
         self.w_element = self.w_tensor_meta = None
         self.b_element = self.b_tensor_meta = None
+        self._narrowed = self._narrowed_key = None
 
         if "Wq" in layer_type:
             if w_element is None:
@@ -88,6 +89,7 @@ class MinifloatLinearPTQ(nn.Module):
     def _apply(self, fn, recurse=True):
         before = {n: getattr(self, n).dtype for n in self._CODE_PARAMS if getattr(self, n) is not None}
         result = super()._apply(fn, recurse)
+        self._narrowed = self._narrowed_key = None
         for name, dt in before.items():
             now = getattr(self, name).dtype
             if now != dt:
@@ -98,12 +100,26 @@ class MinifloatLinearPTQ(nn.Module):
             self.b_tensor_meta = self.b_tensor_meta.create(device=self.b_element.device)
         return result
 
+    def _narrowed_weight(self):
+        """One-byte copy of the weight codes for the fused GEMM (not part of ``state_dict``),
+        rebuilt when ``w_element`` is replaced, written in place or moved."""
+        w = self.w_element
+        if (self.backend != "fused" or w is None or w.device.type != "cuda"
+                or not MinifloatF.gemm_weight_eligible(self.w_tensor_meta)):
+            return None
+        key = (w.data_ptr(), w._version, w.device)
+        if self._narrowed_key != key:
+            self._narrowed = MinifloatF.narrow_weight_codes(w, self.w_tensor_meta)
+            self._narrowed_key = key
+        return self._narrowed
+
     @torch.no_grad()
     def forward(self, input: Tensor) -> Tensor:
         return MinifloatF.minifloat_linear(
             x=input, x_meta=self.x_minifloat_meta, w=self.weight, w_element=self.w_element,
             w_tensor_meta=self.w_tensor_meta, b=self.bias, b_element=self.b_element,
-            b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend)
+            b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend,
+            _narrowed=self._narrowed_weight())
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "

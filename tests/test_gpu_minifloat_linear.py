@@ -1,0 +1,177 @@
+"""GPU parity tests for minifloat_linear / minifloat_matmul / MinifloatLinearPTQ.  The fused
+backend sends weights in the formats the MXFP GEMM decodes through that GEMM (codes narrowed to
+one byte, unit block scales); the rest goes compose -> dense GEMM.  Tolerance: relative
+Frobenius error <= 1e-3 against dequantize-then-matmul in fp64 on the checker's values, rounded
+once to the output dtype; fp32 outputs of the MFMA route are held to 1e-5."""
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+REL_FRO_TOL = 1e-3
+
+
+def rel_fro(y, y_ref):
+    y, y_ref = y.double().cpu(), y_ref.double().cpu()
+    return ((y - y_ref).norm() / y_ref.norm()).item()
+
+
+@pytest.fixture(scope="module")
+def mf():
+    import mase_hip.minifloat.functional as F
+    from mase_hip import _lib
+    from mase_hip.minifloat import meta
+    from mase_hip.minifloat.layers import MinifloatLinearPTQ
+
+    _lib.load()
+
+    class NS:
+        pass
+
+    ns = NS()
+    ns.F, ns.meta, ns.Layer = F, meta, MinifloatLinearPTQ
+    return ns
+
+
+def checker_linear(x, x_meta, w_codes, w_meta, bias):
+    """fp64 x_dq @ w_dq^T + b from the CPU checker's quantisation."""
+    x = x.cpu()
+    x_dq = x if x_meta is None else oracle.qdq_minifloat(x, x_meta.exp_bits, x_meta.frac_bits, x_meta.is_finite,
+                                                          x_meta.round_mode)
+    w_dq = oracle.compose_minifloat(w_codes.cpu(), w_meta.exp_bits, w_meta.frac_bits, w_meta.is_finite, torch.float32)
+    y = x_dq.double().reshape(-1, x.shape[-1]) @ w_dq.double().t()
+    if bias is not None:
+        y = y + bias.double().cpu()
+    return y.view(*x.shape[:-1], -1)
+
+
+W_TAGS = ["FP8_E4M3_fn", "FP8_E5M2_fn", "FP6_E2M3_fn", "FP6_E3M2_fn", "FP4_E2M1_fn"]
+
+
+@pytest.mark.parametrize("w_tag", W_TAGS)
+@pytest.mark.parametrize("MNK", [(96, 256, 512), (8, 128, 256), (200, 136, 96)])
+def test_minifloat_linear_fused_vs_checker(mf, w_tag, MNK):
+    """XqWqB through the MFMA route: every weight format the GEMM decodes, shapes that take the
+    few-row, the 256x256-tile and the bounds-checked kernels."""
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(3)
+    x = (2 * torch.randn(M, K, generator=g)).to(torch.bfloat16)
+    w = (0.5 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    x_meta, w_meta = mf.meta.FP8_E4M3_fn, getattr(mf.meta, w_tag)
+    w_codes, w_tm = mf.F.extract_minifloat_component(w.to(DEV), w_meta)
+    assert torch.equal(w_codes.cpu(), oracle.extract_minifloat(w, w_meta.exp_bits, w_meta.frac_bits))
+    y = mf.F.minifloat_linear(x=x.to(DEV), x_meta=x_meta, w=None, w_element=w_codes, w_tensor_meta=w_tm,
+                              b=b.to(DEV), b_element=None, b_tensor_meta=None, layer_type="XqWqB", backend="fused")
+    assert y.dtype == torch.bfloat16 and y.shape == (M, N)
+    assert rel_fro(y, checker_linear(x, x_meta, w_codes, w_meta, b).to(y.dtype)) <= REL_FRO_TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("layer_type", ["XqWqB", "XWqB", "XqWB", "XWB", "XqWqBq"])
+@pytest.mark.parametrize("bias", [True, False])
+def test_minifloat_layer_fused_matches_separate(mf, dtype, layer_type, bias):
+    M, N, K = 192, 256, 512
+    g = torch.Generator().manual_seed(7)
+    x = (torch.randn(3, M // 3, K, generator=g) * 3).to(dtype).to(DEV)
+    lin = torch.nn.Linear(K, N, bias=bias, dtype=dtype, device=DEV)
+    with torch.no_grad():
+        lin.weight.mul_(16)  # minifloat has no block scale: bring the weights into FP6's range
+    x_meta = mf.meta.FP8_E4M3_fn if layer_type.startswith("Xq") else None
+    w_meta = mf.meta.FP6_E3M2_fn if "Wq" in layer_type else None
+    b_meta = mf.meta.FP8_E4M3_fn if layer_type.endswith("Bq") and bias else None
+    fused = mf.Layer.from_linear(lin, x_meta, w_meta, b_meta, layer_type, "fused")
+    separate = mf.Layer.from_linear(lin, x_meta, w_meta, b_meta, layer_type, "separate")
+    y_f, y_s = fused(x), separate(x)
+    assert y_f.shape == (3, M // 3, N) and y_f.dtype == dtype
+    # a dense fp32 x is not rounded to bf16: that case stays on the dense route and is bit-equal
+    mfma_route = "Wq" in layer_type and (dtype == torch.bfloat16 or layer_type.startswith("Xq"))
+    if not mfma_route:
+        assert torch.equal(y_f, y_s)
+    assert rel_fro(y_f, y_s) <= (REL_FRO_TOL if dtype == torch.bfloat16 else 1e-5)
+
+
+def test_minifloat_linear_wide_formats_use_dense_route(mf):
+    """Weight formats wider than a byte, or with inf/NaN codes, are composed and multiplied by
+    the dense GEMM: bit-equal to the separate backend."""
+    M, N, K = 64, 128, 256
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16).to(DEV)
+    for w_meta in (mf.meta.MinifloatMeta(5, 6, True, "rn"), mf.meta.MinifloatMeta(4, 3, False, "rn")):
+        w_codes, w_tm = mf.F.extract_minifloat_component(w, w_meta)
+        assert not mf.F.gemm_weight_eligible(w_tm)
+        kw = dict(x=x, x_meta=mf.meta.FP8_E4M3_fn, w=None, w_element=w_codes, w_tensor_meta=w_tm, b=None,
+                  b_element=None, b_tensor_meta=None, layer_type="XqWqB")
+        y_f = mf.F.minifloat_linear(**kw, backend="fused")
+        y_s = mf.F.minifloat_linear(**kw, backend="separate")
+        assert torch.equal(y_f, y_s)
+        assert rel_fro(y_f, checker_linear(x, mf.meta.FP8_E4M3_fn, w_codes, w_meta, None).to(y_f.dtype)) <= REL_FRO_TOL
+
+
+def test_minifloat_linear_ignores_code_bits_above_the_format(mf):
+    """The decode reads only the low 1+E+M bits of a code (fake.py:97-123); so does the
+    narrowing to one byte."""
+    M, N, K = 32, 64, 128
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16).to(DEV)
+    w_meta = mf.meta.FP6_E2M3_fn
+    w_codes, w_tm = mf.F.extract_minifloat_component(w, w_meta)
+    noisy = (w_codes.to(torch.int32) | (torch.randint(0, 4, (N, K), generator=g).to(DEV) << 6)).to(torch.uint16)
+    kw = dict(x=x, x_meta=None, w=None, w_tensor_meta=w_tm, b=None, b_element=None, b_tensor_meta=None,
+              layer_type="XWqB", backend="fused")
+    assert torch.equal(mf.F.minifloat_linear(w_element=w_codes, **kw), mf.F.minifloat_linear(w_element=noisy, **kw))
+
+
+def test_minifloat_layer_large_and_few_rows(mf):
+    """One layer applied to a large batch (persistent large-tile kernel) and to a few rows
+    (weight-streaming kernel), checked against fp64 on the checker's values."""
+    N, K = 3072, 256
+    g = torch.Generator().manual_seed(13)
+    w = (0.05 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    lin = torch.nn.Linear(K, N, bias=True, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        lin.bias.copy_(b)
+    x_meta, w_meta = mf.meta.FP8_E4M3_fn, mf.meta.FP8_E4M3_fn
+    layer = mf.Layer.from_linear(lin, x_meta, w_meta, None, "XqWqB", "fused")
+    for M in (2048, 16):
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        y = layer(x.to(DEV))
+        assert rel_fro(y, checker_linear(x, x_meta, layer.w_element, w_meta, b).to(y.dtype)) <= REL_FRO_TOL
+
+
+def test_minifloat_layer_follows_weight_updates(mf):
+    """The one-byte copy of the codes kept by the layer is rebuilt when the codes change."""
+    N, K = 64, 128
+    lin = torch.nn.Linear(K, N, bias=False, dtype=torch.bfloat16, device=DEV)
+    layer = mf.Layer.from_linear(lin, None, mf.meta.FP8_E4M3_fn, None, "XWqB", "fused")
+    x = torch.randn(16, K, dtype=torch.bfloat16, device=DEV)
+    y0 = layer(x)
+    assert "_narrowed" not in layer.state_dict() and set(layer.state_dict()) == {"w_element"}
+    with torch.no_grad():
+        layer.w_element.copy_((layer.w_element.to(torch.int32) ^ 0x80).to(torch.uint16))  # flip every sign
+    y1 = layer(x)
+    assert torch.equal(y1, -y0)
+    cpu_layer = layer.to("cpu")
+    assert cpu_layer._narrowed is None
+
+
+@pytest.mark.parametrize("func_type", ["XW", "XqW", "XWq", "XqWq"])
+@pytest.mark.parametrize("backend", ["separate", "fused"])
+def test_minifloat_matmul(mf, func_type, backend):
+    g = torch.Generator().manual_seed(17)
+    a = torch.randn(4, 48, 96, generator=g).to(torch.bfloat16)
+    b = torch.randn(96, 80, generator=g).to(torch.bfloat16)
+    am, bm = mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn
+    y = mf.F.minifloat_matmul(a.to(DEV), b.to(DEV), am if "Xq" in func_type else None,
+                              bm if "Wq" in func_type else None, func_type, backend)
+    a_dq = oracle.qdq_minifloat(a, am.exp_bits, am.frac_bits) if "Xq" in func_type else a
+    b_dq = oracle.qdq_minifloat(b, bm.exp_bits, bm.frac_bits) if "Wq" in func_type else b
+    assert y.shape == (4, 48, 80) and y.dtype == torch.bfloat16
+    assert rel_fro(y, (a_dq.double() @ b_dq.double()).to(y.dtype)) <= REL_FRO_TOL
