@@ -113,6 +113,33 @@ int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int6
                       void* stream);
 
 /*
+ * Blocks along the middle axis of a row-major [outer, k_len, inner] tensor: block b of column
+ * (o, i) is x[o, 32*b .. 32*b+31, i].  Same scales and elements, in the same order
+ * (scales[outer, inner, k_len/32], elements[outer, inner, k_len]), as permuting the block axis
+ * last, copying and calling mase_hip_extract_mxfp, without the copy.
+ * Replaces extract_mxfp_components(tensor, block_dim, mxfp_meta) for block_dim other than the last
+ * axis  src/mase_triton/mxfp/functional/cast.py:11-44 with its flatten_for_quantize
+ * src/mase_triton/mxfp/helpers.py:4-24, as used on `other` by mxfp_matmul
+ * src/mase_triton/mxfp/functional/matmul.py:24-29.
+ * Needs block_size == 32 and k_len % 32 == 0 (a block never straddles columns), else -2.
+ */
+int mase_hip_extract_mxfp_strided(const void* x, int x_dtype, uint8_t* scales, uint8_t* elements,
+                                  int64_t outer, int64_t k_len, int64_t inner, int block_size,
+                                  int exp_bits, int frac_bits, int is_finite, int round_mode,
+                                  void* stream);
+
+/*
+ * out[outer, k_len, inner] = compose(extract(x)) with blocks along the middle axis, in one pass,
+ * written in x's own layout.  `out` may alias `x` when both dtypes have the same size.
+ * Replaces quantize_dequantize(tensor, block_dim, ...) for block_dim other than the last axis
+ * src/mase_triton/mxfp/functional/cast.py:103-129 (flatten, cast, permute back).
+ * Same restrictions as mase_hip_extract_mxfp_strided.
+ */
+int mase_hip_qdq_mxfp_strided(const void* x, int x_dtype, void* out, int out_dtype, int64_t outer,
+                              int64_t k_len, int64_t inner, int block_size, int exp_bits,
+                              int frac_bits, int is_finite, int round_mode, void* stream);
+
+/*
  * y[M,N] (out_dtype) = A[M,K] * W[N,K]^T (+ bias[N]), fp32 accumulation on bf16 MFMA.
  *
  *   A: either dense (a_dense != NULL, dtype a_dtype, row-major [M,K], NOT yet quantised: it is

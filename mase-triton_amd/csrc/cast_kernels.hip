@@ -513,6 +513,171 @@ __global__ __launch_bounds__(kThreads) void qdq_mxfp_block_kernel(const void* x,
     }
 }
 
+// ------------------------------------------------------------------------------ blocks along a non-last axis
+// The tensor is [outer, K, inner] row-major and blocks of 32 run along K (element stride
+// `inner`), K % 32 == 0: what the reference reaches by permuting the block axis last and
+// copying (src/mase_triton/mxfp/helpers.py:4-24) before its flat kernel.  Here a lane owns
+// adjacent positions of the inner axis and walks down K one block at a time; a block sits in
+// one lane's registers, so its maximum needs no cross-lane traffic, and adjacent lanes read
+// adjacent addresses of a row.  Outputs keep the reference's order: scales [outer, inner, K/32]
+// and elements [outer, inner, K] (extract), or the input's own layout (quantise-dequantise).
+// Work item (one per lane) -> (outer, group of kb_per k-blocks, chunk of the inner axis), chunk
+// fastest, so a short inner axis still fills a wavefront with several k-groups.
+struct StridedGeom {
+    int64_t K, inner, nkb;  // nkb = K / 32
+    int64_t chunks, kgroups, items;
+    int kb_per;
+};
+
+__device__ inline bool strided_origin(const StridedGeom& g, int vec, int64_t& o, int64_t& kb0, int64_t& i0) {
+    const int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t rest = item / g.chunks;
+    i0 = (item - rest * g.chunks) * vec;
+    o = rest / g.kgroups;
+    kb0 = (rest - o * g.kgroups) * g.kb_per;
+    return item < g.items;
+}
+
+// 32 codes (one per entry, low byte) -> 32 consecutive bytes at dst
+__device__ inline void store_block_codes(uint8_t* dst, const uint32_t (&code)[32], bool aligned16) {
+    if (aligned16) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            uint32_t w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int b = 16 * h + 4 * j;
+                w[j] = code[b] | (code[b + 1] << 8) | (code[b + 2] << 16) | (code[b + 3] << 24);
+            }
+            st128<false>(dst + 16 * h, make_uint4(w[0], w[1], w[2], w[3]));
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) dst[j] = (uint8_t)code[j];
+    }
+}
+
+// Any dtype, any format: one position of the inner axis per lane.  MODE 0 extract, 1 QDQ.
+template <int DT_IN, int DT_OUT, class F, int MODE>
+__global__ __launch_bounds__(kThreads) void mxfp_strided_kernel(const void* x, uint8_t* __restrict__ scales,
+                                                                 uint8_t* __restrict__ elements, void* out, StridedGeom g,
+                                                                 bool elements_aligned16, F f) {
+    int64_t o, kb0, i;
+    if (!strided_origin(g, 1, o, kb0, i)) return;
+    for (int q = 0; q < g.kb_per; ++q) {
+        const int64_t kb = kb0 + q;
+        if (kb >= g.nkb) break;
+        const int64_t first = (o * g.K + kb * 32) * g.inner + i;
+        uint32_t u[32], amax = 0;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            u[j] = load_bits_scalar<DT_IN>(x, first + j * g.inner);
+            const uint32_t a = u[j] & 0x7FFFFFFFu;
+            amax = a > amax ? a : amax;
+        }
+        const int se = shared_exponent<F, DT_IN != F32>(amax, f);
+        const uint32_t scale = amax < 0x00800000u ? 0u : (uint32_t)(se + 127);
+        uint32_t code[32];
+#pragma unroll
+        for (int j = 0; j < 32; ++j) code[j] = encode_mxfp_element(u[j], se, f);
+        if (MODE == 0) {
+            const int64_t col = o * g.inner + i;
+            store_block_codes(elements + col * g.K + kb * 32, code, elements_aligned16);
+            scales[col * g.nkb + kb] = (uint8_t)scale;
+        } else {
+            // the lane has read its whole block before it writes: in-place use is safe
+            const float sc = scale_f32(scale);
+#pragma unroll
+            for (int j = 0; j < 32; ++j) store_val_scalar<DT_OUT>(out, first + j * g.inner, mxfp_value(code[j], sc, f));
+        }
+    }
+}
+
+// bfloat16 in (and out), compile-time format: two positions of the inner axis per lane (one
+// 32-bit load per row), packed 16-bit arithmetic as in mxfp_bf16_b32_kernel with one scale per
+// 16-bit half.  Needs inner % 2 == 0 and 4-byte aligned x / out.
+template <class F, int MODE>
+__global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_kernel(const uint16_t* x, uint8_t* __restrict__ scales,
+                                                                      uint8_t* __restrict__ elements, uint16_t* out,
+                                                                      StridedGeom g, bool elements_aligned16, F f) {
+    int64_t o, kb0, i0;
+    if (!strided_origin(g, 2, o, kb0, i0)) return;
+    for (int q = 0; q < g.kb_per; ++q) {
+        const int64_t kb = kb0 + q;
+        if (kb >= g.nkb) break;
+        const int64_t first = (o * g.K + kb * 32) * g.inner + i0;
+        uint32_t h[32];
+        u16x2 m = {0, 0};
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            h[j] = *reinterpret_cast<const uint32_t*>(x + first + j * g.inner);
+            m = __builtin_elementwise_max(m, as_u16x2(h[j] & 0x7FFF7FFFu));
+        }
+        uint32_t amax[2], scale[2];
+        bool hard = false;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            amax[c] = m[c];
+            const int scale_n = max((int)(amax[c] >> 7) - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
+            hard |= amax[c] >= 0x7F80u || scale_n >= 151 || (MODE == 1 && amax[c] != 0u && scale_n <= fmt_bias(f));
+            scale[c] = (uint32_t)scale_n;
+        }
+        // res[j]: MODE 0 two codes (low byte of each half), MODE 1 two bf16 results
+        uint32_t res[32];
+        if (__builtin_amdgcn_ballot_w64(hard) == 0) {
+            const uint32_t lo = (uint32_t)(((int)scale[0] - fmt_bias(f)) << 7) & 0xFFFFu;
+            const uint32_t hi = (uint32_t)(((int)scale[1] - fmt_bias(f)) << 7) & 0xFFFFu;
+            const uint32_t ssb2 = lo | (hi << 16);
+#pragma unroll
+            for (int j = 0; j < 32; ++j) res[j] = MODE == 0 ? PackedBf16<F>::codes(h[j], ssb2) : PackedBf16<F>::qdq(h[j], ssb2);
+        } else {
+            // exact per-element routine
+            int se[2];
+            float sc[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const uint32_t amax32 = amax[t] << 16;
+                se[t] = shared_exponent<F, true>(amax32, f);
+                scale[t] = amax32 < 0x00800000u ? 0u : (uint32_t)(se[t] + 127);
+                sc[t] = scale_f32(scale[t]);
+            }
+#pragma unroll
+            for (int j = 0; j < 32; ++j) {
+                const uint32_t c0 = encode_mxfp_element(h[j] << 16, se[0], f);
+                const uint32_t c1 = encode_mxfp_element(h[j] & 0xFFFF0000u, se[1], f);
+                res[j] = MODE == 0 ? (c0 | (c1 << 16)) : pack_bf16(mxfp_value(c0, sc[0], f), mxfp_value(c1, sc[1], f));
+            }
+        }
+        if (MODE == 0) {
+            // bytes 0 / 2 of res[j] are the codes of the lane's first / second column in row j
+            uint32_t cd[2][8];
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                const uint32_t t01 = __builtin_amdgcn_perm(res[4 * w + 1], res[4 * w], 0x06020400u);
+                const uint32_t t23 = __builtin_amdgcn_perm(res[4 * w + 3], res[4 * w + 2], 0x06020400u);
+                cd[0][w] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+                cd[1][w] = __builtin_amdgcn_perm(t23, t01, 0x07060302u);
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int64_t col = o * g.inner + i0 + t;
+                uint8_t* dst = elements + col * g.K + kb * 32;
+                if (elements_aligned16) {
+                    st128<false>(dst, make_uint4(cd[t][0], cd[t][1], cd[t][2], cd[t][3]));
+                    st128<false>(dst + 16, make_uint4(cd[t][4], cd[t][5], cd[t][6], cd[t][7]));
+                } else {
+#pragma unroll
+                    for (int b = 0; b < 32; ++b) dst[b] = (uint8_t)(cd[t][b >> 2] >> (8 * (b & 3)));
+                }
+                scales[col * g.nkb + kb] = (uint8_t)scale[t];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 32; ++j) *reinterpret_cast<uint32_t*>(out + first + j * g.inner) = res[j];
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------ launch helpers
 inline unsigned grid_for(int64_t items, int per_block) {
     return (unsigned)((items + per_block - 1) / per_block);
@@ -696,5 +861,99 @@ int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int6
         });
     });
 }
+
+// Blocks along the middle axis of an [outer, K, inner] tensor (no counterpart kernel in the
+// reference, which permutes and copies first; same outputs as that route).
+static int strided_args(int64_t outer, int64_t k_len, int64_t inner, int block_size) {
+    if (outer < 0 || k_len < 0 || inner < 0) return fail(ERR_INVALID, "negative extent");
+    if (block_size != 32) return fail(ERR_UNSUPPORTED, "strided blocks need block_size 32");
+    if (k_len % 32 != 0) return fail(ERR_UNSUPPORTED, "strided blocks need the block axis to be a multiple of 32");
+    if (outer != 0 && k_len != 0 && inner != 0 && (outer > INT64_MAX / k_len || outer * k_len > INT64_MAX / inner))
+        return fail(ERR_INVALID, "extent overflow");
+    return OK;
+}
+
+// k-blocks handled in sequence by one lane: up to 4 (a lane then fills whole 128-byte lines of
+// codes), fewer while that leaves less than a few wavefronts per SIMD
+static StridedGeom strided_geom(int64_t outer, int64_t k_len, int64_t inner, int vec, unsigned& grid, bool& ok) {
+    StridedGeom g;
+    g.K = k_len; g.inner = inner; g.nkb = k_len / 32;
+    g.chunks = inner / vec;
+    int kb_per = 4;
+    while (kb_per > 1 && outer * ((g.nkb + kb_per - 1) / kb_per) * g.chunks < (int64_t)256 * 16 * 64) kb_per >>= 1;
+    g.kb_per = kb_per;
+    g.kgroups = (g.nkb + kb_per - 1) / kb_per;
+    g.items = outer * g.kgroups * g.chunks;
+    const int64_t blocks = (g.items + kThreads - 1) / kThreads;
+    ok = blocks <= 0x7FFFFFFFll;
+    grid = (unsigned)blocks;
+    return g;
+}
+
+int mase_hip_extract_mxfp_strided(const void* x, int x_dtype, uint8_t* scales, uint8_t* elements, int64_t outer,
+                                  int64_t k_len, int64_t inner, int block_size, int exp_bits, int frac_bits, int is_finite,
+                                  int round_mode, void* stream) {
+    if (int rc = strided_args(outer, k_len, inner, block_size)) return rc;
+    if (int rc = check_mxfp_fmt(exp_bits, frac_bits, round_mode, 0, block_size)) return rc;
+    if (int rc = check_dtype(x_dtype, "input")) return rc;
+    if (outer == 0 || k_len == 0 || inner == 0) return OK;
+    if (!x || !scales || !elements) return fail(ERR_INVALID, "null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool el16 = aligned(elements, 16);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        unsigned grid; bool ok;
+        if constexpr (decltype(f)::kStatic) {
+            if (x_dtype == BF16 && inner % 2 == 0 && aligned(x, 4)) {
+                const StridedGeom g = strided_geom(outer, k_len, inner, 2, grid, ok);
+                if (!ok) return fail(ERR_UNSUPPORTED, "tensor too large for one launch");
+                hipLaunchKernelGGL((mxfp_strided_bf16_kernel<decltype(f), 0>), dim3(grid), dim3(kThreads), 0, s,
+                                   static_cast<const uint16_t*>(x), scales, elements, nullptr, g, el16, f);
+                return check_launch("extract_mxfp_strided");
+            }
+        }
+        const StridedGeom g = strided_geom(outer, k_len, inner, 1, grid, ok);
+        if (!ok) return fail(ERR_UNSUPPORTED, "tensor too large for one launch");
+        return dispatch_dtype(x_dtype, [&](auto dt) {
+            hipLaunchKernelGGL((mxfp_strided_kernel<decltype(dt)::value, F32, decltype(f), 0>), dim3(grid), dim3(kThreads), 0, s, x,
+                               scales, elements, nullptr, g, el16, f);
+            return check_launch("extract_mxfp_strided");
+        });
+    });
+}
+
+int mase_hip_qdq_mxfp_strided(const void* x, int x_dtype, void* out, int out_dtype, int64_t outer, int64_t k_len,
+                              int64_t inner, int block_size, int exp_bits, int frac_bits, int is_finite, int round_mode,
+                              void* stream) {
+    if (int rc = strided_args(outer, k_len, inner, block_size)) return rc;
+    if (int rc = check_mxfp_fmt(exp_bits, frac_bits, round_mode, 0, block_size)) return rc;
+    if (int rc = check_dtype(x_dtype, "input")) return rc;
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (outer == 0 || k_len == 0 || inner == 0) return OK;
+    if (!x || !out) return fail(ERR_INVALID, "null pointer");
+    if (x == out && dtype_size(x_dtype) != dtype_size(out_dtype)) return fail(ERR_INVALID, "in-place use needs equal element sizes");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
+        unsigned grid; bool ok;
+        if constexpr (decltype(f)::kStatic) {
+            if (x_dtype == BF16 && out_dtype == BF16 && inner % 2 == 0 && aligned(x, 4) && aligned(out, 4)) {
+                const StridedGeom g = strided_geom(outer, k_len, inner, 2, grid, ok);
+                if (!ok) return fail(ERR_UNSUPPORTED, "tensor too large for one launch");
+                hipLaunchKernelGGL((mxfp_strided_bf16_kernel<decltype(f), 1>), dim3(grid), dim3(kThreads), 0, s,
+                                   static_cast<const uint16_t*>(x), nullptr, nullptr, static_cast<uint16_t*>(out), g, false, f);
+                return check_launch("qdq_mxfp_strided");
+            }
+        }
+        const StridedGeom g = strided_geom(outer, k_len, inner, 1, grid, ok);
+        if (!ok) return fail(ERR_UNSUPPORTED, "tensor too large for one launch");
+        return dispatch_dtype(x_dtype, [&](auto di) {
+            return dispatch_dtype(out_dtype, [&](auto dout) {
+                hipLaunchKernelGGL((mxfp_strided_kernel<decltype(di)::value, decltype(dout)::value, decltype(f), 1>), dim3(grid),
+                                   dim3(kThreads), 0, s, x, nullptr, nullptr, out, g, false, f);
+                return check_launch("qdq_mxfp_strided");
+            });
+        });
+    });
+}
+
 
 }  // extern "C"

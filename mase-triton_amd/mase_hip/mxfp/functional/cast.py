@@ -22,7 +22,11 @@ def extract_mxfp_components(tensor: Tensor, block_dim: int, mxfp_meta: MXFPMeta)
     tensor_meta = MXFPTensorMeta(
         device=device_str(tensor.device), dtype=dtype_str(tensor.dtype), shape=shape_tuple(tensor.shape),
         block_dim=block_dim, meta=mxfp_meta)
-    scales, elements = kernels.extract_mxfp_components(flatten_for_quantize(tensor, block_dim), mxfp_meta=mxfp_meta)
+    if tensor.device.type == "cuda" and kernels.strided_blocks_supported(tensor_meta.shape, block_dim, mxfp_meta):
+        # blocks along an inner axis are read in place: same outputs as the permuted copy below
+        scales, elements = kernels.extract_mxfp_components_strided(tensor, block_dim, mxfp_meta)
+    else:
+        scales, elements = kernels.extract_mxfp_components(flatten_for_quantize(tensor, block_dim), mxfp_meta=mxfp_meta)
     return scales, elements, tensor_meta
 
 
@@ -48,5 +52,9 @@ def quantize_dequantize(tensor: Tensor, block_dim: int, mxfp_meta: MXFPMeta,
     assert -ndim <= block_dim < ndim
     if output_dtype is None:
         output_dtype = tensor.dtype
+    if tensor.device.type == "cuda" and kernels.strided_blocks_supported(shape_tuple(tensor.shape), block_dim, mxfp_meta):
+        # contiguous result in the tensor's own layout (the permuted-copy route returns the same
+        # values as a transposed view)
+        return kernels.quantize_dequantize_strided(tensor, block_dim, mxfp_meta, output_dtype)
     flat = kernels.quantize_dequantize(flatten_for_quantize(tensor, block_dim), mxfp_meta, output_dtype)
     return permute_for_dequantize(flat, ori_shape=shape_tuple(tensor.shape), block_dim=block_dim)

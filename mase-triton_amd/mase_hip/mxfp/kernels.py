@@ -3,7 +3,8 @@
 ``extract_mxfp_components`` / ``compose_mxfp_tensor`` have the names and signatures of the
 reference's Triton wrappers (src/mase_triton/mxfp/kernels/cast.py:126-160, 237-272); results are
 bit-identical to the reference's PyTorch "fake" implementation (src/mase_triton/mxfp/fake.py).
-``quantize_dequantize`` and ``mxfp_gemm`` have no counterpart there (fused paths).
+``quantize_dequantize``, the ``*_strided`` casts and ``mxfp_gemm`` have no counterpart there
+(fused paths; blocks along a non-last axis without the permuted copy).
 """
 from __future__ import annotations
 
@@ -67,6 +68,56 @@ def quantize_dequantize(x: Tensor, mxfp_meta: MXFPMeta, output_dtype: torch.dtyp
     return out
 
 
+def strided_blocks_supported(shape: tuple[int, ...], block_dim: int, mxfp_meta: MXFPMeta) -> bool:
+    """Can blocks along ``block_dim`` be taken in place (no permuted copy)?  The axis must not be
+    the last one (those blocks are contiguous already) and must hold whole blocks of 32."""
+    ndim = len(shape)
+    block_dim %= ndim
+    return block_dim != ndim - 1 and mxfp_meta.block_size == 32 and shape[block_dim] % 32 == 0
+
+
+def _strided_extents(shape, block_dim: int) -> tuple[int, int, int]:
+    block_dim %= len(shape)
+    outer = inner = 1
+    for d in shape[:block_dim]:
+        outer *= d
+    for d in shape[block_dim + 1:]:
+        inner *= d
+    return outer, shape[block_dim], inner
+
+
+def extract_mxfp_components_strided(x: Tensor, block_dim: int, mxfp_meta: MXFPMeta) -> tuple[Tensor, Tensor]:
+    """N-D float tensor, blocks along ``block_dim`` -> (scales uint8 [n/32, 1], elements uint8
+    [n/32, 32]) in the order of the tensor with ``block_dim`` rotated last; no permuted copy."""
+    assert strided_blocks_supported(tuple(x.shape), block_dim, mxfp_meta)
+    _lib.require_gpu(x, "input tensor")
+    x = _lib.dense(_lib.as_float_input(x))
+    outer, k_len, inner = _strided_extents(x.shape, block_dim)
+    n = x.numel()
+    scales = torch.empty((n // 32, 1), dtype=torch.uint8, device=x.device)
+    elements = torch.empty((n // 32, 32), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().mase_hip_extract_mxfp_strided(
+            x.data_ptr(), _lib.dtype_code(x.dtype), scales.data_ptr(), elements.data_ptr(), outer, k_len, inner, 32,
+            *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
+    return scales, elements
+
+
+def quantize_dequantize_strided(x: Tensor, block_dim: int, mxfp_meta: MXFPMeta, output_dtype: torch.dtype) -> Tensor:
+    """compose(extract(x)) with blocks along ``block_dim`` in one pass; the result is contiguous
+    in x's own shape."""
+    assert strided_blocks_supported(tuple(x.shape), block_dim, mxfp_meta)
+    _lib.require_gpu(x, "input tensor")
+    x = _lib.dense(_lib.as_float_input(x))
+    outer, k_len, inner = _strided_extents(x.shape, block_dim)
+    out = torch.empty(x.shape, dtype=output_dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.load().mase_hip_qdq_mxfp_strided(
+            x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(output_dtype), outer, k_len, inner, 32,
+            *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
+    return out
+
+
 def mxfp_gemm(
     a: Tensor | None,
     a_scales: Tensor | None,
@@ -80,11 +131,13 @@ def mxfp_gemm(
     N: int,
     K: int,
     output_dtype: torch.dtype,
+    out: Tensor | None = None,
 ) -> Tensor:
     """y[M,N] = A[M,K] @ W[N,K]^T (+ bias) on bf16 MFMA with fp32 accumulation.
 
     A is either a dense [M,K] tensor (``a``; used as is) or MXFP components blocked along K.
     W is MXFP components of the row-major [N,K] weight, blocked along K.
+    ``out``: optional contiguous [M,N] tensor of ``output_dtype`` to write into.
     """
     dev = w_elements.device
     _lib.require_gpu(w_elements, "w_elements")
@@ -110,7 +163,11 @@ def mxfp_gemm(
         bias = _lib.dense(bias)
         assert bias.numel() == N
         b_ptr, b_dt = bias.data_ptr(), _lib.dtype_code(bias.dtype)
-    y = torch.empty((M, N), dtype=output_dtype, device=dev)
+    if out is None:
+        y = torch.empty((M, N), dtype=output_dtype, device=dev)
+    else:
+        assert out.is_contiguous() and out.dtype == output_dtype and out.numel() == M * N and out.device == dev
+        y = out
     with torch.cuda.device(dev):
         _lib.check(_lib.load().mase_hip_mxfp_gemm(
             a_ptr, a_dt, a_sc_ptr, a_el_ptr, a_e, a_m, w_scales.data_ptr(), w_elements.data_ptr(),

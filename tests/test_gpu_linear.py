@@ -334,3 +334,31 @@ def test_mxfp_matmul(mh, func_type, backend):
         b_q = b.cpu()
     y_chk = torch.matmul(a_q.float(), b_q.float()).to(torch.bfloat16)
     assert rel_fro(y, y_chk) <= REL_FRO_TOL
+
+
+@pytest.mark.parametrize("a_shape,b_shape,dtype", [
+    ((3, 40, 256), (256, 192), torch.bfloat16),          # matrix `other`: one GEMM over all rows
+    ((2, 600, 128), (2, 128, 320), torch.bfloat16),      # a launch per batch, 256 x 256 tiles
+    ((40, 16, 64), (40, 64, 96), torch.bfloat16),        # many batches: one batched dense GEMM
+    ((2, 4, 24, 96), (4, 96, 64), torch.bfloat16),       # broadcast batch axes: dense GEMM
+    ((2, 50, 128), (2, 128, 72), torch.float32),         # fp32 in and out
+    ((4, 48), (48, 40), torch.bfloat16),                 # contraction axis not a multiple of 32
+])
+def test_mxfp_matmul_fused_routes(mh, a_shape, b_shape, dtype):
+    """Every route of the fused backend against the checker's quantisation of the same operands
+    (`other` quantised down its second-to-last axis)."""
+    g = torch.Generator().manual_seed(sum(a_shape))
+    a = (torch.randn(*a_shape, generator=g) * 5).to(dtype)
+    b = (torch.randn(*b_shape, generator=g) * 3).to(dtype)
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    a_q = oracle.qdq_mxfp(a, 32, 4, 3)
+    bt = b.transpose(-1, -2).contiguous()
+    b_q = oracle.qdq_mxfp(bt.flatten(), 32, 4, 3).view(bt.shape).transpose(-1, -2)
+    for func_type in ("XqWq", "XWq"):
+        y = mh.F.mxfp_matmul(a.to(DEV), b.to(DEV), fmt if func_type == "XqWq" else None, fmt, func_type, "fused")
+        y_chk = torch.matmul((a_q if func_type == "XqWq" else a).double(), b_q.double()).to(dtype)
+        assert y.shape == y_chk.shape and y.dtype == dtype
+        tol = REL_FRO_TOL if dtype == torch.bfloat16 else 1e-5
+        assert rel_fro(y, y_chk) <= tol, func_type
+        y_sep = mh.F.mxfp_matmul(a.to(DEV), b.to(DEV), fmt if func_type == "XqWq" else None, fmt, func_type, "separate")
+        assert rel_fro(y, y_sep) <= tol, func_type
