@@ -140,6 +140,18 @@ int mase_hip_qdq_mxfp_strided(const void* x, int x_dtype, void* out, int out_dty
                               int frac_bits, int is_finite, int round_mode, void* stream);
 
 /*
+ * Storage form of element codes: n codes of `bits` (4 or 6) significant bits, one per byte in `elements`, as a
+ * little-endian bit stream in `packed` (code i at bits [bits*i, bits*i + bits); n*bits/8 bytes).  n % 16 == 0;
+ * `elements` 16-byte and `packed` 8-byte aligned.  unpack restores exactly the bytes pack read (with the bits above
+ * `bits` cleared).
+ * No counterpart in the reference, which keeps one byte per code in memory and in state_dict
+ * (src/mase_triton/mxfp/layers.py:69-80, src/mase_triton/mxfp/fake.py:71-79); these serve a packed on-disk /
+ * at-rest form of a quantised layer.
+ */
+int mase_hip_pack_codes(const uint8_t* elements, uint8_t* packed, int64_t n, int bits, void* stream);
+int mase_hip_unpack_codes(const uint8_t* packed, uint8_t* elements, int64_t n, int bits, void* stream);
+
+/*
  * y[M,N] (out_dtype) = A[M,K] * W[N,K]^T (+ bias[N]), fp32 accumulation on bf16 MFMA.
  *
  *   A: either dense (a_dense != NULL, dtype a_dtype, row-major [M,K], NOT yet quantised: it is

@@ -24,6 +24,8 @@ SIGNATURES = {
     "mase_hip_qdq_mxfp": (_i32, [_vp, _i32, _vp, _i32, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
     "mase_hip_extract_mxfp_strided": (_i32, [_vp, _i32, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
     "mase_hip_qdq_mxfp_strided": (_i32, [_vp, _i32, _vp, _i32, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "mase_hip_pack_codes": (_i32, [_vp, _vp, _i64, _i32, _vp]),
+    "mase_hip_unpack_codes": (_i32, [_vp, _vp, _i64, _i32, _vp]),
     "mase_hip_mxfp_gemm": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
                                   _vp, _i32, _i64, _i64, _i64, _i32, _vp]),
 }

@@ -127,6 +127,41 @@ class MXFPLinearPTQ(nn.Module):
                        x_mxfp_meta=x_mxfp_meta, w_mxfp_meta=w_mxfp_meta, b_mxfp_meta=b_mxfp_meta,
                        layer_type=layer_type, backend=backend)
 
+    def export_quantized(self) -> dict:
+        """Everything needed to rebuild the layer, as tensors, strings and integers only (safe to
+        ``torch.save`` and to load with ``weights_only=True``): element codes bit-packed, tensor
+        metas as plain dicts.  Quantised-weight layer types only."""
+        from . import packing
+
+        assert self.w_scales is not None, "export_quantized needs a quantised weight (Wq layer types)"
+        d = {"format": "mase_hip.mxfp.linear/1", "layer_type": self.layer_type,
+             "x_mxfp_meta": None if self.x_mxfp_meta is None else packing.meta_to_dict(self.x_mxfp_meta),
+             "w": packing.export_components(self.w_scales, self.w_elements, self.w_tensor_meta),
+             "b": None, "bias": None if self.bias is None else self.bias.detach().clone()}
+        if self.b_scales is not None:
+            d["b"] = {"scales": self.b_scales.detach().reshape(-1).clone(), "elements": self.b_elements.detach().clone(),
+                      "tensor_meta": packing.tensor_meta_to_dict(self.b_tensor_meta)}
+        return d
+
+    @classmethod
+    def from_exported(cls, d: dict, backend: Literal["separate", "fused"] = "fused", device=None):
+        """Inverse of :meth:`export_quantized`."""
+        from . import packing
+
+        assert d.get("format") == "mase_hip.mxfp.linear/1", "not an exported MXFP linear layer"
+        w_scales, w_elements, w_tm = packing.import_components(d["w"], device=device)
+        b_scales = b_elements = b_tm = None
+        if d["b"] is not None:
+            b_tm = packing.tensor_meta_from_dict(d["b"]["tensor_meta"], device=device)
+            b_scales, b_elements = d["b"]["scales"].view(-1, 1), d["b"]["elements"]
+            if device is not None:
+                b_scales, b_elements = b_scales.to(device), b_elements.to(device)
+        bias = d["bias"]
+        if bias is not None and device is not None:
+            bias = bias.to(device)
+        x_meta = None if d["x_mxfp_meta"] is None else packing.meta_from_dict(d["x_mxfp_meta"])
+        return cls.from_quantized(w_scales, w_elements, w_tm, bias, b_scales, b_elements, b_tm, x_meta, d["layer_type"], backend)
+
     @classmethod
     def from_quantized(cls, w_scales: Tensor | None, w_elements: Tensor | None, w_tensor_meta: MXFPTensorMeta | None,
                        bias: Tensor | None, b_scales: Tensor | None, b_elements: Tensor | None,

@@ -301,3 +301,39 @@ def test_config_c3_hashes():
     yb = bits_of(oracle.compose_mxfp(sc, el, 32, 2, 1, True, torch.bfloat16)).copy()
     yb[(yb & 0x7FFF) > 0x7F80] = 0x7FC0
     assert _sha(yb) == want[("c3", "dq_bf16_nan_canonical")]
+
+
+# ----------------------------------------------------------------------------- packed storage form of codes
+def test_packed_codes_hand_computed_vectors():
+    """Bit stream, least significant bit first: worked out by hand, not by the checker's formula."""
+    from oracle import packing
+
+    # 4-bit: codes 0x1, 0xF, 0x8, 0x3 -> bytes 0xF1, 0x38
+    assert packing.pack_codes(np.array([0x1, 0xF, 0x8, 0x3], np.uint8), 4).tolist() == [0xF1, 0x38]
+    # 6-bit: codes 1, 0, 0, 0 -> bit 0 set; codes 0, 1, 0, 0 -> bit 6; 0, 0, 1, 0 -> bit 12 (byte 1 bit 4); 0, 0, 0, 1 -> bit 18 (byte 2 bit 2)
+    assert packing.pack_codes(np.array([1, 0, 0, 0], np.uint8), 6).tolist() == [0x01, 0x00, 0x00]
+    assert packing.pack_codes(np.array([0, 1, 0, 0], np.uint8), 6).tolist() == [0x40, 0x00, 0x00]
+    assert packing.pack_codes(np.array([0, 0, 1, 0], np.uint8), 6).tolist() == [0x00, 0x10, 0x00]
+    assert packing.pack_codes(np.array([0, 0, 0, 1], np.uint8), 6).tolist() == [0x00, 0x00, 0x04]
+    # 6-bit: 0x3F, 0x00, 0x3F, 0x00 -> bits 0-5 and 12-17: 0x3F, 0xF0, 0x03
+    assert packing.pack_codes(np.array([0x3F, 0, 0x3F, 0], np.uint8), 6).tolist() == [0x3F, 0xF0, 0x03]
+    # 6-bit: 0x2A (101010), 0x15 (010101), 0x2A, 0x15 -> 0b01101010, 0b10100101, 0b01010110 read LSB first
+    assert packing.pack_codes(np.array([0x2A, 0x15, 0x2A, 0x15], np.uint8), 6).tolist() == [0x6A, 0xA5, 0x56]
+    # bits above the code width are dropped
+    assert packing.pack_codes(np.array([0xF1, 0x2F], np.uint8), 4).tolist() == [0xF1]
+
+
+@pytest.mark.parametrize("bits", [4, 6])
+def test_packed_codes_round_trip(bits):
+    from oracle import packing
+
+    rng = np.random.default_rng(bits)
+    codes = rng.integers(0, 1 << bits, size=4096, dtype=np.uint8)
+    packed = packing.pack_codes(codes, bits)
+    assert packed.size == codes.size * bits // 8
+    assert np.array_equal(packing.unpack_codes(packed, bits, codes.size), codes)
+    # every code value at every position of a group
+    every = np.tile(np.arange(1 << bits, dtype=np.uint8), 4)
+    for shift in range(4):
+        c = np.roll(every, shift)
+        assert np.array_equal(packing.unpack_codes(packing.pack_codes(c, bits), bits, c.size), c)
