@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--counter-probe", action="store_true",
                     help="profiling aid for rocprofv3 --pmc: a plain 256 MiB device copy (calibration), then 3 launches "
                          "each of the GEMM and of the C3 extract / compose kernels; prints nothing to time")
+    ap.add_argument("--shape-sweep", action="store_true",
+                    help="context run, not the metric: mxfp_linear fused vs separate over M at N=14336, K=4096, and the "
+                         "in-place casts along a non-last axis against the permuted-copy route; prints its own JSON line")
     return ap.parse_args()
 
 
@@ -289,6 +292,48 @@ def cpu_baseline(torch):
                       f"path (quantise x, dequantise x and W, F.linear), {dt:.1f} s"}
 
 
+def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
+    """Host-timed (launch overhead included) context figures; every shape takes a different GEMM kernel."""
+    from mase_hip.mxfp.helpers import flatten_for_quantize
+
+    dev = "cuda:0"
+    N, K = 14336, 4096
+    gen = torch.Generator(device=dev).manual_seed(5)
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e6 / steps
+
+    w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
+    w_sc, w_el, w_tm = MXFP_F.extract_mxfp_components(w, block_dim=1, mxfp_meta=fmt)
+    rows = []
+    for M in (16, 64, 128, 256, 384, 512, 1024, 2048, 4096):
+        x = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
+        call = dict(x=x, x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
+                    b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
+        f_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="fused"))
+        s_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="separate"))
+        rows.append({"M": M, "fused_us": round(f_us, 1), "separate_us": round(s_us, 1),
+                     "fused_TFLOPs": round(2.0 * M * N * K / f_us / 1e6, 1)})
+    n = w.numel()
+    cast = {
+        "shape": [N, K], "block_axis": 0,
+        "extract_in_place_us": round(timed(lambda: mxk.extract_mxfp_components_strided(w, 0, fmt)), 1),
+        "extract_permuted_copy_us": round(timed(lambda: mxk.extract_mxfp_components(flatten_for_quantize(w, 0), fmt)), 1),
+        "qdq_in_place_us": round(timed(lambda: mxk.quantize_dequantize_strided(w, 0, fmt, torch.bfloat16)), 1),
+        "qdq_permuted_copy_us": round(timed(lambda: mxk.quantize_dequantize(flatten_for_quantize(w, 0), fmt, torch.bfloat16)), 1),
+    }
+    cast["extract_in_place_GBps"] = round(n * (3 + 1 / 32) / cast["extract_in_place_us"] / 1e3, 0)
+    cast["qdq_in_place_GBps"] = round(n * 4 / cast["qdq_in_place_us"] / 1e3, 0)
+    return {"linear_N14336_K4096": rows, "casts_along_axis0": cast}
+
+
 def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
     """Few launches of each kernel next to a copy of known size, for hardware-counter runs."""
     dev = "cuda:0"
@@ -331,6 +376,9 @@ def main():
     torch.cuda.set_device(0)
     if args.counter_probe:
         counter_probe(torch, MXFP_F, mxk, MXFP8_E4M3_fn, MXFPMeta(32, 8, 2, 1, True, "rn"))
+        return
+    if args.shape_sweep:
+        print(json.dumps({"shape_sweep": shape_sweep(torch, MXFP_F, mxk, MXFP8_E4M3_fn)}))
         return
     lin = bench_linear(args, torch, MXFP_F, mxk, MXFP8_E4M3_fn)
     M, N, K = lin["shape"]
