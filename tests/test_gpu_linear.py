@@ -416,3 +416,30 @@ def test_mxfp_matmul_fused_routes(mh, a_shape, b_shape, dtype):
         assert rel_fro(y, y_chk) <= tol, func_type
         y_sep = mh.F.mxfp_matmul(a.to(DEV), b.to(DEV), fmt if func_type == "XqWq" else None, fmt, func_type, "separate")
         assert rel_fro(y, y_sep) <= tol, func_type
+
+
+def test_gemm_dispatch_boundaries(mh):
+    """Shapes on both sides of every kernel-selection threshold (rows 128 / 129, 511 / 512 / 513; N and K that do
+    or do not divide by the tile sizes; few and many tiles), each against fp32 dequantize-then-matmul on the GPU."""
+    g = torch.Generator().manual_seed(99)
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    shapes = []
+    for M in (1, 127, 128, 129, 255, 256, 257, 383, 511, 512, 513, 640, 1023, 1025):
+        for N, K in ((128, 128), (96, 128), (160, 160), (256, 384), (384, 96)):
+            shapes.append((M, N, K))
+    shapes += [(129, 12288, 128), (511, 12288, 128), (512, 12288, 128), (513, 12288, 256), (640, 12416, 128), (130, 4160, 256)]
+    worst = 0.0
+    for M, N, K in shapes:
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        w = (0.05 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+        x_dq = oracle.qdq_mxfp(x.flatten(), 32, 4, 3).view(M, K).to(DEV)
+        w_sc, w_el = oracle.extract_mxfp(w, 32, 4, 3)
+        w_dq = oracle.compose_mxfp(w_sc, w_el, 32, 4, 3, True, torch.bfloat16).view(N, K).to(DEV)
+        b = torch.randn(N, generator=g).to(torch.bfloat16).to(DEV)
+        for odt in (torch.bfloat16, torch.float32):
+            y = mh.mxk.mxfp_gemm(x_dq, None, None, None, w_sc.to(DEV), w_el.to(DEV), fmt, b, M, N, K, odt)
+            y_ref = (x_dq.float() @ w_dq.float().T + b.float()).to(odt)
+            err = rel_fro(y, y_ref)
+            worst = max(worst, err)
+            assert err <= (REL_FRO_TOL if odt == torch.bfloat16 else 1e-5), (M, N, K, odt, err)
+    assert worst > 0.0  # summation orders differ: exact equality everywhere would mean the kernels did not run
