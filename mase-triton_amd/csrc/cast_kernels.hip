@@ -596,6 +596,64 @@ __global__ __launch_bounds__(kThreads) void mxfp_strided_kernel(const void* x, u
 // bfloat16 in (and out), compile-time format: two positions of the inner axis per lane (one
 // 32-bit load per row), packed 16-bit arithmetic as in mxfp_bf16_b32_kernel with one scale per
 // 16-bit half.  Needs inner % 2 == 0 and 4-byte aligned x / out.
+// One block of 32 rows for the lane's two columns, read at x + first (+ j * inner).  res[j]: MODE 0 the two codes
+// of row j (low byte of each 16-bit half), MODE 1 the two bf16 results; scale[t]: the scale byte of column t.
+template <class F, int MODE>
+__device__ inline void strided_bf16_block(const uint16_t* x, int64_t first, int64_t inner, const F& f, uint32_t (&res)[32],
+                                          uint32_t (&scale)[2]) {
+    uint32_t h[32];
+    u16x2 m = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        h[j] = *reinterpret_cast<const uint32_t*>(x + first + j * inner);
+        m = __builtin_elementwise_max(m, as_u16x2(h[j] & 0x7FFF7FFFu));
+    }
+    uint32_t amax[2];
+    bool hard = false;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        amax[c] = m[c];
+        const int scale_n = max((int)(amax[c] >> 7) - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
+        hard |= amax[c] >= 0x7F80u || scale_n >= 151 || (MODE == 1 && amax[c] != 0u && scale_n <= fmt_bias(f));
+        scale[c] = (uint32_t)scale_n;
+    }
+    if (__builtin_amdgcn_ballot_w64(hard) == 0) {
+        const uint32_t lo = (uint32_t)(((int)scale[0] - fmt_bias(f)) << 7) & 0xFFFFu;
+        const uint32_t hi = (uint32_t)(((int)scale[1] - fmt_bias(f)) << 7) & 0xFFFFu;
+        const uint32_t ssb2 = lo | (hi << 16);
+#pragma unroll
+        for (int j = 0; j < 32; ++j) res[j] = MODE == 0 ? PackedBf16<F>::codes(h[j], ssb2) : PackedBf16<F>::qdq(h[j], ssb2);
+    } else {
+        // exact per-element routine
+        int se[2];
+        float sc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint32_t amax32 = amax[t] << 16;
+            se[t] = shared_exponent<F, true>(amax32, f);
+            scale[t] = amax32 < 0x00800000u ? 0u : (uint32_t)(se[t] + 127);
+            sc[t] = scale_f32(scale[t]);
+        }
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const uint32_t c0 = encode_mxfp_element(h[j] << 16, se[0], f);
+            const uint32_t c1 = encode_mxfp_element(h[j] & 0xFFFF0000u, se[1], f);
+            res[j] = MODE == 0 ? (c0 | (c1 << 16)) : pack_bf16(mxfp_value(c0, sc[0], f), mxfp_value(c1, sc[1], f));
+        }
+    }
+}
+
+// bytes 0 / 2 of res[j] are the codes of the lane's first / second column in row j -> 32 code bytes per column
+__device__ inline void gather_column_codes(const uint32_t (&res)[32], uint32_t (&cd)[2][8]) {
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        const uint32_t t01 = __builtin_amdgcn_perm(res[4 * w + 1], res[4 * w], 0x06020400u);
+        const uint32_t t23 = __builtin_amdgcn_perm(res[4 * w + 3], res[4 * w + 2], 0x06020400u);
+        cd[0][w] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+        cd[1][w] = __builtin_amdgcn_perm(t23, t01, 0x07060302u);
+    }
+}
+
 template <class F, int MODE>
 __global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_kernel(const uint16_t* x, uint8_t* __restrict__ scales,
                                                                       uint8_t* __restrict__ elements, uint16_t* out,
@@ -606,58 +664,11 @@ __global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_kernel(const uint1
         const int64_t kb = kb0 + q;
         if (kb >= g.nkb) break;
         const int64_t first = (o * g.K + kb * 32) * g.inner + i0;
-        uint32_t h[32];
-        u16x2 m = {0, 0};
-#pragma unroll
-        for (int j = 0; j < 32; ++j) {
-            h[j] = *reinterpret_cast<const uint32_t*>(x + first + j * g.inner);
-            m = __builtin_elementwise_max(m, as_u16x2(h[j] & 0x7FFF7FFFu));
-        }
-        uint32_t amax[2], scale[2];
-        bool hard = false;
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            amax[c] = m[c];
-            const int scale_n = max((int)(amax[c] >> 7) - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
-            hard |= amax[c] >= 0x7F80u || scale_n >= 151 || (MODE == 1 && amax[c] != 0u && scale_n <= fmt_bias(f));
-            scale[c] = (uint32_t)scale_n;
-        }
-        // res[j]: MODE 0 two codes (low byte of each half), MODE 1 two bf16 results
-        uint32_t res[32];
-        if (__builtin_amdgcn_ballot_w64(hard) == 0) {
-            const uint32_t lo = (uint32_t)(((int)scale[0] - fmt_bias(f)) << 7) & 0xFFFFu;
-            const uint32_t hi = (uint32_t)(((int)scale[1] - fmt_bias(f)) << 7) & 0xFFFFu;
-            const uint32_t ssb2 = lo | (hi << 16);
-#pragma unroll
-            for (int j = 0; j < 32; ++j) res[j] = MODE == 0 ? PackedBf16<F>::codes(h[j], ssb2) : PackedBf16<F>::qdq(h[j], ssb2);
-        } else {
-            // exact per-element routine
-            int se[2];
-            float sc[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const uint32_t amax32 = amax[t] << 16;
-                se[t] = shared_exponent<F, true>(amax32, f);
-                scale[t] = amax32 < 0x00800000u ? 0u : (uint32_t)(se[t] + 127);
-                sc[t] = scale_f32(scale[t]);
-            }
-#pragma unroll
-            for (int j = 0; j < 32; ++j) {
-                const uint32_t c0 = encode_mxfp_element(h[j] << 16, se[0], f);
-                const uint32_t c1 = encode_mxfp_element(h[j] & 0xFFFF0000u, se[1], f);
-                res[j] = MODE == 0 ? (c0 | (c1 << 16)) : pack_bf16(mxfp_value(c0, sc[0], f), mxfp_value(c1, sc[1], f));
-            }
-        }
+        uint32_t res[32], scale[2];
+        strided_bf16_block<F, MODE>(x, first, g.inner, f, res, scale);
         if (MODE == 0) {
-            // bytes 0 / 2 of res[j] are the codes of the lane's first / second column in row j
             uint32_t cd[2][8];
-#pragma unroll
-            for (int w = 0; w < 8; ++w) {
-                const uint32_t t01 = __builtin_amdgcn_perm(res[4 * w + 1], res[4 * w], 0x06020400u);
-                const uint32_t t23 = __builtin_amdgcn_perm(res[4 * w + 3], res[4 * w + 2], 0x06020400u);
-                cd[0][w] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
-                cd[1][w] = __builtin_amdgcn_perm(t23, t01, 0x07060302u);
-            }
+            gather_column_codes(res, cd);
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const int64_t col = o * g.inner + i0 + t;
@@ -675,6 +686,57 @@ __global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_kernel(const uint1
 #pragma unroll
             for (int j = 0; j < 32; ++j) *reinterpret_cast<uint32_t*>(out + first + j * g.inner) = res[j];
         }
+    }
+}
+
+// Extract with whole-line stores: a workgroup takes 128 adjacent columns and four consecutive k-blocks (one per
+// wavefront), i.e. one 128-byte line of codes per column.  The lanes' 32-byte pieces meet in LDS ([column][128 B],
+// row of column c = 64 (c & 1) + (c >> 1), 16-byte chunk k of a row at position k ^ ((row >> 1) & 7): conflict-free
+// for the lane-per-column writes and for the 8-lanes-per-line reads), and every store instruction then writes 8
+// whole lines instead of 64 quarter lines; the four scale bytes of a column leave as one dword.
+// Needs inner % 128 == 0, K % 128 == 0, 16-byte aligned elements and 4-byte aligned scales.
+constexpr int kStridedTCols = 128;
+template <class F>
+__global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_lines_kernel(const uint16_t* x, uint8_t* __restrict__ scales,
+                                                                            uint8_t* __restrict__ elements, int64_t K, int64_t inner,
+                                                                            int64_t nkb, F f) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[kStridedTCols * 128];
+    __shared__ __attribute__((aligned(4))) uint8_t sc_tile[kStridedTCols * 4];
+    const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+    // workgroup -> (outer, group of 4 k-blocks, chunk of 128 columns), column chunk fastest
+    const int64_t col_chunks = inner / kStridedTCols, kgroups = nkb / 4;
+    int64_t bid = blockIdx.x;
+    const int64_t cc = bid % col_chunks;
+    bid /= col_chunks;
+    const int64_t kg = bid % kgroups, o = bid / kgroups;
+    const int64_t iw = cc * kStridedTCols, kb0 = kg * 4;
+    {
+        const int64_t first = (o * K + (kb0 + q) * 32) * inner + iw + 2 * lane;
+        uint32_t res[32], scale[2], cd[2][8];
+        strided_bf16_block<F, 0>(x, first, inner, f, res, scale);
+        gather_column_codes(res, cd);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int row = 64 * t + lane;
+            uint8_t* const r = tile + row * 128;
+            const int sw = (row >> 1) & 7;
+            *reinterpret_cast<uint4*>(r + (((2 * q) ^ sw) * 16)) = make_uint4(cd[t][0], cd[t][1], cd[t][2], cd[t][3]);
+            *reinterpret_cast<uint4*>(r + (((2 * q + 1) ^ sw) * 16)) = make_uint4(cd[t][4], cd[t][5], cd[t][6], cd[t][7]);
+            sc_tile[(2 * lane + t) * 4 + q] = (uint8_t)scale[t];
+        }
+    }
+    __syncthreads();
+    const int64_t col0 = o * inner + iw;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int row = 8 * (4 * q + p) + (lane >> 3), k = lane & 7;
+        const int col = 2 * (row & 63) + (row >> 6);
+        const uint4 v = *reinterpret_cast<const uint4*>(tile + row * 128 + ((k ^ ((row >> 1) & 7)) * 16));
+        st128<false>(elements + (col0 + col) * K + kb0 * 32 + k * 16, v);
+    }
+    if (lane < 32) {
+        const int col = 32 * q + lane;
+        *reinterpret_cast<uint32_t*>(scales + (col0 + col) * nkb + kb0) = *reinterpret_cast<const uint32_t*>(sc_tile + col * 4);
     }
 }
 
@@ -904,6 +966,13 @@ int mase_hip_extract_mxfp_strided(const void* x, int x_dtype, uint8_t* scales, u
         unsigned grid; bool ok;
         if constexpr (decltype(f)::kStatic) {
             if (x_dtype == BF16 && inner % 2 == 0 && aligned(x, 4)) {
+                if (inner % kStridedTCols == 0 && k_len % 128 == 0 && el16 && aligned(scales, 4)) {
+                    const int64_t blocks = outer * (k_len / 128) * (inner / kStridedTCols);
+                    if (blocks > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "tensor too large for one launch");
+                    hipLaunchKernelGGL((mxfp_strided_bf16_lines_kernel<decltype(f)>), dim3((unsigned)blocks), dim3(kThreads), 0, s,
+                                       static_cast<const uint16_t*>(x), scales, elements, k_len, inner, k_len / 32, f);
+                    return check_launch("extract_mxfp_strided");
+                }
                 const StridedGeom g = strided_geom(outer, k_len, inner, 2, grid, ok);
                 if (!ok) return fail(ERR_UNSUPPORTED, "tensor too large for one launch");
                 hipLaunchKernelGGL((mxfp_strided_bf16_kernel<decltype(f), 0>), dim3(grid), dim3(kThreads), 0, s,

@@ -85,7 +85,7 @@ def test_reference_vectors_laid_out_down_the_rows(mh, dt, blocks_per_column):
 @pytest.mark.parametrize("dt", ["bfloat16", "float16", "float32"])
 @pytest.mark.parametrize("shape,block_dim", [
     ((64, 8), 0), ((32, 1), 0), ((96, 1028), 0), ((160, 1030), -2), ((3, 64, 20), 1), ((2, 3, 128, 36), -2),
-    ((2, 32, 3, 5), 1), ((256, 4096), 0), ((5, 32, 4), -2),
+    ((2, 32, 3, 5), 1), ((256, 4096), 0), ((5, 32, 4), -2), ((3, 128, 256), 1), ((2, 256, 2, 64), 1), ((384, 128), 0),
 ])
 def test_strided_vs_checker_on_the_rotated_copy(mh, dt, shape, block_dim):
     g = torch.Generator().manual_seed(sum(shape) + block_dim)
@@ -104,11 +104,12 @@ def test_strided_vs_checker_on_the_rotated_copy(mh, dt, shape, block_dim):
         assert_bits_equal(mh.mxk.quantize_dequantize_strided(xd, block_dim, meta, x.dtype), want, dt, f"qdq {dt} {tag}")
 
 
-def test_strided_special_blocks_and_scales(mh):
-    """bf16 matrix whose columns hold inf / NaN, all-zero blocks, blocks of subnormals, very large
+@pytest.mark.parametrize("inner", [64, 128])
+def test_strided_special_blocks_and_scales(mh, inner):
+    """(inner = 128 with K = 128 takes the whole-line-store extract kernel.)  bf16 matrix whose columns hold inf / NaN, all-zero blocks, blocks of subnormals, very large
     and very small magnitudes (scales near 0 and 254): the packed fast path must hand these to
     the exact routine."""
-    K, inner = 128, 64
+    K = 128
     g = torch.Generator().manual_seed(21)
     x = torch.randn(K, inner, generator=g)
     x[:, 1] *= 2.0 ** 120
