@@ -413,6 +413,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 #include "gemm_tall.h"
 #include "gemm_skinny.h"
 #include "gemm_mid.h"
+#include "gemm_wide.h"
 
 // ---------------------------------------------------------------------------------------------
 // Small-shape kernel: 128 x 128 x 32 tiles, single LDS buffer.  Used when the problem cannot
@@ -543,9 +544,12 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             return launch_gemm_skinny<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
     }
     if constexpr (A_MODE == 0) {
-        // more rows than that, fewer than a 512-row tile: 128 x 128 tiles, eight wavefronts each
-        if (fits32 && M > 128 && M < UM && N % MD_N == 0 && K % MD_MAC == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
-            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0)
+        // a few hundred rows: 256 x 128 tiles for 256 < M <= 512, 128 x 128 tiles for 128 < M <= 256
+        const bool mid_ok = fits32 && N % MD_N == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
+                            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0;
+        if (mid_ok && M > WD_M && M <= 2 * WD_M && K % WD_K == 0)
+            return launch_gemm_wide<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+        if (mid_ok && M > 128 && M <= WD_M && K % MD_MAC == 0)
             return launch_gemm_mid<FW, DT_OUT, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
     }
     if constexpr (A_MODE == 0 && DT_OUT != F32) {

@@ -268,10 +268,15 @@ def test_gemm_few_rows_special_values(mh):
     ((511, 1024, 1664), "MXFP8_E5M2_fn", torch.float16, False),    # four m-tiles, 13 macro steps, generic decode of E5M2
     ((384, 2048, 2048), "OCP_MXFP6_E2M3", torch.bfloat16, False),  # 48 tiles, K rotation wraps (16 n-tiles = 16 macro steps)
     ((300, 4352, 512), "MXFP8_E4M3_fn", torch.bfloat16, True),     # 34 n-tiles, more than the 4 macro steps: rotation modulo
+    ((257, 128, 64), "MXFP8_E4M3_fn", torch.bfloat16, False),      # 256 x 128 tiles: two m-tiles (one row in the second), one step
+    ((512, 256, 320), "OCP_MXFP6_E3M2", torch.float32, True),      # 5 steps of 64 k (K not a multiple of 128), fp32 output
+    ((400, 640, 832), "OCP_MXFP4_E2M1", torch.float16, True),      # 13 steps: the 6-step unrolled loop wraps twice
+    ((250, 1024, 1152), "MXFP8_E5M2_fn", torch.bfloat16, True),    # 128 x 128 tiles, 9 macro steps
 ])
 def test_gemm_mid_rows(mh, MNK, w_tag, odt, with_bias):
-    """128 < M < 512 with N % 128 == 0 and K % 128 == 0 takes the 128 x 128 tile kernel (eight wavefronts, K halves
-    added through LDS, loads and compose placed between the MFMAs)."""
+    """128 < M <= 256 with N % 128 == 0 and K % 128 == 0 takes the 128 x 128 tile kernel (eight wavefronts, K halves
+    added through LDS, loads and compose placed between the MFMAs); 256 < M <= 512 with K % 64 == 0 the 256 x 128 tile
+    kernel (eight wavefronts of 64 x 64, 64-k steps)."""
     M, N, K = MNK
     g = torch.Generator().manual_seed(M * 3 + N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -296,10 +301,11 @@ def test_gemm_mid_rows(mh, MNK, w_tag, odt, with_bias):
     assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref.to(odt)) <= (1e-5 if odt == torch.float32 else REL_FRO_TOL)
 
 
-def test_gemm_mid_rows_special_values(mh):
-    """Scale 255 (a block that held an inf or NaN) on the 128 x 128 tile kernel: those output columns are NaN, the
-    rest finite."""
-    M, N, K = 300, 512, 640
+@pytest.mark.parametrize("M", [200, 300])
+def test_gemm_mid_rows_special_values(mh, M):
+    """Scale 255 (a block that held an inf or NaN) on the 128 x 128 (M = 200) and 256 x 128 (M = 300) tile kernels:
+    those output columns are NaN, the rest finite."""
+    N, K = 512, 640
     g = torch.Generator().manual_seed(17)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = torch.randn(N, K, generator=g).to(torch.bfloat16)
