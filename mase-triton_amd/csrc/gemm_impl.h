@@ -552,8 +552,8 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         if (mid_ok && M > 128 && M <= WD_M && K % MD_MAC == 0)
             return launch_gemm_mid<FW, DT_OUT, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
     }
-    if constexpr (A_MODE == 0 && DT_OUT != F32) {
-        // tall tiles: dense A, 16-bit output, whole tiles only, enough of them to occupy the chip
+    if constexpr (A_MODE == 0) {
+        // tall tiles: dense A, whole tiles only, enough of them to occupy the chip
         const int tall_tiles_m = (M + UM - 1) / UM;
         const int64_t tall_tiles = (int64_t)tall_tiles_m * (N / UN);
         if (fits32 && M >= UM && N % UN == 0 && K % UMAC == 0 && tall_tiles >= TALL_MIN_TILES &&

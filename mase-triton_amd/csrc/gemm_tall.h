@@ -456,6 +456,43 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
                 bv[0] = load_bias(bias, bias_dtype, cur.n0 + (int)ol);
                 bv[1] = load_bias(bias, bias_dtype, cur.n0 + 64 + (int)ol);
             }
+            if constexpr (DT_OUT == F32) {
+                // fp32 output: 16 passes of 32 rows x 32 columns (128 bytes per row again); a lane writes the 16 bytes of
+                // its four consecutive columns as chunk 2 g + (l >> 5) of row l & 31
+                uint8_t* const y_wave32 = static_cast<uint8_t*>(y) + ((size_t)(cur.m0 + wave * 128) * N + cur.n0) * 4;
+                const uint32_t o_st_voff32 = ((ol >> 3) * (uint32_t)N + (ol & 7u) * 4u) * 4u;
+                static_for<4>([&](auto i_c) {
+                    static_for<4>([&](auto j_c) {
+                        constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
+                        static_for<4>([&](auto g_c) {
+                            constexpr int g = decltype(g_c)::value;
+                            float r[4];
+                            static_for<4>([&](auto t_c) {
+                                constexpr int t = decltype(t_c)::value, col = 32 * j + 8 * g + t;  // + 4 for the upper half-wave
+                                r[t] = acc_read(acc[j][i][4 * g + t]);
+                                if (HAS_BIAS) {
+                                    const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv[col >> 6]), col & 63));
+                                    const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bv[col >> 6]), (col + 4) & 63));
+                                    r[t] += o_half ? hi : lo;
+                                }
+                            });
+                            const uint32_t chunk = ((uint32_t)(2 * g) + o_half) ^ (o_row & 7u);
+                            *reinterpret_cast<uint4*>(lds_out + o_row * 128u + chunk * 16u) =
+                                make_uint4(f32_bits(r[0]), f32_bits(r[1]), f32_bits(r[2]), f32_bits(r[3]));
+                        });
+                        u32x4 v[4];
+                        static_for<4>([&](auto t_c) {
+                            constexpr int t = decltype(t_c)::value;
+                            v[t] = *reinterpret_cast<const u32x4*>(lds_out + o_rd_off + t * 1024);
+                        });
+                        static_for<4>([&](auto t_c) {
+                            constexpr int t = decltype(t_c)::value;
+                            async_store16(o_st_voff32, y_wave32 + ((size_t)(i * 32 + 8 * t) * N + j * 32) * 4, v[t]);
+                        });
+                        __builtin_amdgcn_sched_barrier(0);  // one pass at a time
+                    });
+                });
+            } else
             static_for<4>([&](auto i_c) {
                 static_for<2>([&](auto jh_c) {
                     constexpr int i = decltype(i_c)::value, jh = decltype(jh_c)::value;

@@ -148,9 +148,11 @@ def test_mxfp_linear_vs_cpu_reference_path(mh):
     ((16384, 1024, 512), "OCP_MXFP6_E2M3", torch.bfloat16),  # tall problem: 32 x 8 tiles
     ((1000, 8192, 256), "MXFP8_E4M3_fn", torch.bfloat16),    # M not a multiple of 512: the last tile row is shifted up
     ((3001, 2048, 384), "OCP_MXFP6_E3M2", torch.float16),    # 6 tile rows, the last one overlapping by 71 rows
+    ((2048, 8320, 384), "MXFP8_E4M3_fn", torch.float32),     # fp32 output: 16 staging passes per tile, several tiles per workgroup
+    ((1000, 12288, 128), "OCP_MXFP4_E2M1", torch.float32),   # fp32 output, shifted last tile row
 ])
 def test_gemm_large_tile_shapes(mh, MNK, w_tag, odt):
-    """Shapes that take the 512 x 128 tile kernel (dense A, 16-bit output, no bias, whole tiles): the whole output
+    """Shapes that take the 512 x 128 tile kernel (dense A, no bias, whole tiles): the whole output
     against an fp32 dequantize-then-matmul on the GPU, and a sample of it against float64 accumulation."""
     M, N, K = MNK
     g = torch.Generator().manual_seed(M + N + K)
@@ -162,12 +164,13 @@ def test_gemm_large_tile_shapes(mh, MNK, w_tag, odt):
     w_dq = oracle.compose_mxfp(w_sc, w_el, 32, we, wm, True, torch.bfloat16).view(N, K)
     y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, w_tag), None, M, N, K, odt)
     assert y.shape == (M, N) and y.dtype == odt
+    tol = 1e-5 if odt == torch.float32 else REL_FRO_TOL
     y_gpu = (x_dq.to(DEV).float() @ w_dq.to(DEV).float().T).to(odt)
-    assert rel_fro(y, y_gpu) <= REL_FRO_TOL
+    assert rel_fro(y, y_gpu) <= tol
     rows = torch.arange(0, M, 61)
     cols = torch.arange(0, N, 37)
     y_ref = oracle.matmul_nt(x_dq[rows], w_dq[cols]).to(odt)
-    assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref) <= REL_FRO_TOL
+    assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref) <= tol
 
 
 @pytest.mark.parametrize("bdt", [torch.float32, torch.bfloat16, torch.float16])
@@ -193,6 +196,13 @@ def test_gemm_large_tile_bias(mh, bdt):
                           M, N, K, torch.bfloat16)
     col_shift = (y.float() - y0.float()).mean(dim=0).cpu()
     assert torch.allclose(col_shift, b.float(), atol=0.02, rtol=0.02)
+    # fp32 output: the bias lands exactly
+    y32 = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), b.to(DEV),
+                           M, N, K, torch.float32)
+    y32_0 = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), None,
+                             M, N, K, torch.float32)
+    assert rel_fro(y32, x_dq.to(DEV).float() @ w_dq.to(DEV).float().T + b.to(DEV).float()) <= 1e-5
+    assert torch.allclose((y32 - y32_0).cpu(), b.float().expand(M, N), atol=1e-5, rtol=1e-5)
 
 
 def test_gemm_large_tile_special_values(mh):
