@@ -515,9 +515,6 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
         }
 }
 
-#ifndef TALL_MIN_TILES
-#define TALL_MIN_TILES 96
-#endif
 inline int device_cu_count() {
     static int n_cus = 0;
     if (n_cus == 0) {
@@ -544,21 +541,32 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             return launch_gemm_skinny<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
     }
     if constexpr (A_MODE == 0) {
-        // a few hundred rows: 256 x 128 tiles for 256 < M <= 512, 128 x 128 tiles for 128 < M <= 256
-        const bool mid_ok = fits32 && N % MD_N == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
-                            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0;
-        if (mid_ok && M > WD_M && M <= 2 * WD_M && K % WD_K == 0)
-            return launch_gemm_wide<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
-        if (mid_ok && M > 128 && M <= WD_M && K % MD_MAC == 0)
-            return launch_gemm_mid<FW, DT_OUT, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
-    }
-    if constexpr (A_MODE == 0) {
-        // tall tiles: dense A, whole tiles only, enough of them to occupy the chip
-        const int tall_tiles_m = (M + UM - 1) / UM;
-        const int64_t tall_tiles = (int64_t)tall_tiles_m * (N / UN);
-        if (fits32 && M >= UM && N % UN == 0 && K % UMAC == 0 && tall_tiles >= TALL_MIN_TILES &&
-            (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
-            (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0) {
+        // More rows: three tile shapes.  The larger the tile the fewer instructions per MFMA (a composed W row serves more
+        // rows of A), but the fewer tiles there are to spread over the CUs.  Pick the shape with the least estimated time:
+        // (rounds of one tile per CU) x (time of one tile, relative, measured at K = 4096: 48 / 67 / 98 us for
+        // 128 x 128 / 256 x 128 / 512 x 128); ties go to the larger tile.
+        const bool al = (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0;
+        const bool mid_ok = fits32 && al && M > 128 && N % MD_N == 0 && K % MD_MAC == 0;
+        const bool wide_ok = fits32 && al && M > 128 && N % WD_N == 0 && K % WD_K == 0;
+        const bool tall_ok = fits32 && al && M >= UM && N % UN == 0 && K % UMAC == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
+                             (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0;
+        if (mid_ok || wide_ok || tall_ok) {
+            const int cus = device_cu_count();
+            if (cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
+            const int64_t n128 = N / 128;
+            auto cost = [&](int tile_rows, double tile_time) {
+                const int64_t tiles = (int64_t)((M + tile_rows - 1) / tile_rows) * n128;
+                return tile_time * (double)((tiles + cus - 1) / cus);
+            };
+            int pick = -1;
+            double best = 0.0;
+            if (mid_ok) { pick = 0; best = cost(MD_M, 1.0); }
+            if (wide_ok) { const double c = cost(WD_M, 1.4); if (pick < 0 || c <= best) { pick = 1; best = c; } }
+            if (tall_ok) { const double c = cost(UM, 2.05); if (pick < 0 || c <= best) { pick = 2; best = c; } }
+            if (pick == 0) return launch_gemm_mid<FW, DT_OUT, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+            if (pick == 1) return launch_gemm_wide<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+            const int tall_tiles_m = (M + UM - 1) / UM;
+            const int64_t tall_tiles = (int64_t)tall_tiles_m * (N / UN);
             auto kern = mxfp_gemm_tall_kernel<FW, DT_OUT>;
             static bool attr_done = false;
             if (!attr_done) {
@@ -566,8 +574,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
                 if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
                 attr_done = true;
             }
-            const int cus = device_cu_count();
-            if (cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
+            // one persistent workgroup per CU (a multiple of the 8 XCDs), never more than tiles
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
             hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
                                w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN);

@@ -141,18 +141,19 @@ def test_mxfp_linear_vs_cpu_reference_path(mh):
 
 
 @pytest.mark.parametrize("MNK,w_tag,odt", [
-    ((4096, 2048, 128), "MXFP8_E4M3_fn", torch.bfloat16),    # 128 tiles, a single 128-k macro step per tile
+    ((4096, 4096, 128), "MXFP8_E4M3_fn", torch.bfloat16),    # 256 tiles, a single 128-k macro step per tile
     ((2048, 8320, 384), "OCP_MXFP6_E3M2", torch.bfloat16),   # 260 tiles: some workgroups take two, one XCD is short
     ((8192, 2048, 1024), "OCP_MXFP4_E2M1", torch.float16),   # one tile per workgroup, fp16 output
     ((1536, 16384, 256), "MXFP8_E5M2_fn", torch.bfloat16),   # 3 tile rows: the last group of tile rows is a single row
     ((16384, 1024, 512), "OCP_MXFP6_E2M3", torch.bfloat16),  # tall problem: 32 x 8 tiles
-    ((1000, 8192, 256), "MXFP8_E4M3_fn", torch.bfloat16),    # M not a multiple of 512: the last tile row is shifted up
-    ((3001, 2048, 384), "OCP_MXFP6_E3M2", torch.float16),    # 6 tile rows, the last one overlapping by 71 rows
+    ((1000, 14336, 256), "MXFP8_E4M3_fn", torch.bfloat16),   # M not a multiple of 512: the last tile row is shifted up
+    ((3001, 5376, 384), "OCP_MXFP6_E3M2", torch.float16),    # 6 tile rows, the last one overlapping by 71 rows
     ((2048, 8320, 384), "MXFP8_E4M3_fn", torch.float32),     # fp32 output: 16 staging passes per tile, several tiles per workgroup
     ((1000, 12288, 128), "OCP_MXFP4_E2M1", torch.float32),   # fp32 output, shifted last tile row
 ])
 def test_gemm_large_tile_shapes(mh, MNK, w_tag, odt):
-    """Shapes that take the 512 x 128 tile kernel (dense A, no bias, whole tiles): the whole output
+    """Shapes for which the launcher picks the 512 x 128 tile kernel (its tiles fill the CUs in whole rounds; dense A, no
+    bias): the whole output
     against an fp32 dequantize-then-matmul on the GPU, and a sample of it against float64 accumulation."""
     M, N, K = MNK
     g = torch.Generator().manual_seed(M + N + K)
@@ -176,7 +177,7 @@ def test_gemm_large_tile_shapes(mh, MNK, w_tag, odt):
 @pytest.mark.parametrize("bdt", [torch.float32, torch.bfloat16, torch.float16])
 def test_gemm_large_tile_bias(mh, bdt):
     """Bias on the 512 x 128 tile kernel (added to the fp32 accumulators before the output rounding)."""
-    M, N, K = 4096, 2048, 256
+    M, N, K = 4096, 4096, 256
     g = torch.Generator().manual_seed(5)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
@@ -207,7 +208,7 @@ def test_gemm_large_tile_bias(mh, bdt):
 
 def test_gemm_large_tile_special_values(mh):
     """Scale 255 (a block that held an inf) on the 512 x 128 tile kernel: that output column is NaN, the rest finite."""
-    M, N, K = 4096, 2048, 256
+    M, N, K = 4096, 4096, 256
     g = torch.Generator().manual_seed(11)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = torch.randn(N, K, generator=g).to(torch.bfloat16)
@@ -282,11 +283,14 @@ def test_gemm_few_rows_special_values(mh):
     ((512, 256, 320), "OCP_MXFP6_E3M2", torch.float32, True),      # 5 steps of 64 k (K not a multiple of 128), fp32 output
     ((400, 640, 832), "OCP_MXFP4_E2M1", torch.float16, True),      # 13 steps: the 6-step unrolled loop wraps twice
     ((250, 1024, 1152), "MXFP8_E5M2_fn", torch.bfloat16, True),    # 128 x 128 tiles, 9 macro steps
+    ((384, 14336, 256), "MXFP8_E4M3_fn", torch.bfloat16, False),   # 256 x 128 tiles by tile count: 224 of them against 336 of 128 x 128
+    ((1100, 4096, 384), "OCP_MXFP6_E2M3", torch.float16, True),    # 256 x 128 tiles for many rows: 160 tiles in one round, ragged M
+    ((1024, 4096, 256), "MXFP8_E4M3_fn", torch.bfloat16, True),    # 128 x 128 tiles for many rows: 256 tiles, exactly one per CU
 ])
 def test_gemm_mid_rows(mh, MNK, w_tag, odt, with_bias):
-    """128 < M <= 256 with N % 128 == 0 and K % 128 == 0 takes the 128 x 128 tile kernel (eight wavefronts, K halves
-    added through LDS, loads and compose placed between the MFMAs); 256 < M <= 512 with K % 64 == 0 the 256 x 128 tile
-    kernel (eight wavefronts of 64 x 64, 64-k steps)."""
+    """M > 128 with N % 128 == 0: the 128 x 128 tile kernel (K % 128 == 0; eight wavefronts, K halves added through LDS,
+    loads and compose placed between the MFMAs) or the 256 x 128 tile kernel (K % 64 == 0; eight wavefronts of 64 x 64,
+    64-k steps), whichever the launcher estimates faster from the tile counts."""
     M, N, K = MNK
     g = torch.Generator().manual_seed(M * 3 + N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -313,14 +317,14 @@ def test_gemm_mid_rows(mh, MNK, w_tag, odt, with_bias):
 
 @pytest.mark.parametrize("M", [200, 300])
 def test_gemm_mid_rows_special_values(mh, M):
-    """Scale 255 (a block that held an inf or NaN) on the 128 x 128 (M = 200) and 256 x 128 (M = 300) tile kernels:
-    those output columns are NaN, the rest finite."""
-    N, K = 512, 640
+    """Scale 255 (a block that held an inf or NaN) on the 128 x 128 (M = 200, K = 640) and 256 x 128 (M = 300, K = 576,
+    not a multiple of 128) tile kernels: those output columns are NaN, the rest finite."""
+    N, K = 512, (640 if M == 200 else 576)
     g = torch.Generator().manual_seed(17)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = torch.randn(N, K, generator=g).to(torch.bfloat16)
     w[77, 300] = float("inf")
-    w[400, 639] = float("nan")
+    w[400, K - 1] = float("nan")
     w_sc, w_el = oracle.extract_mxfp(w, 32, 4, 3)
     x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
     y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), None,
