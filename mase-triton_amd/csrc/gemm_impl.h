@@ -412,6 +412,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 
 #include "gemm_tall.h"
 #include "gemm_skinny.h"
+#include "gemm_rows16.h"
 #include "gemm_mid.h"
 #include "gemm_wide.h"
 
@@ -535,8 +536,19 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     const bool fits32 = (int64_t)M * K * 2 < ((int64_t)1 << 32) && (int64_t)N * K < ((int64_t)1 << 32);  // 32-bit operand offsets
     const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
     if constexpr (A_MODE == 0) {
+        // fewest rows of A and not many rows of W: one workgroup per 16 rows of W, so that there are enough workgroups
+        // (the 32-row kernel below has N / 32; measured better up to N = 12288 for M <= 16 and up to N = 8192 for M <= 64)
+        if (M <= 64 && N % R16_N == 0 && N <= (M <= 16 ? 12288 : 8192) && K % 128 == 0 && K <= (1 << 24) &&
+            (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 7) == 0) {
+            if (M <= 16) return launch_gemm_rows16<FW, DT_OUT, 1, 8>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+            if (M <= 32) return launch_gemm_rows16<FW, DT_OUT, 2, 4>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+            return launch_gemm_rows16<FW, DT_OUT, 4, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+        }
+    }
+    if constexpr (A_MODE == 0) {
         // few rows of A: bound by streaming W; one workgroup per 32 rows of W
-        if (M <= 128 && N % SK_N == 0 && K % SK_MAC == 0 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
+        // (K bound: both kernels address a row of A or W with a 32-bit byte offset from a per-workgroup base)
+        if (M <= 128 && N % SK_N == 0 && K % SK_MAC == 0 && K <= (1 << 24) && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
             (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0)
             return launch_gemm_skinny<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
     }

@@ -202,148 +202,10 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
     }
 }
 
-// ---------------------------------------------------------------------------------------------
-// M <= 64: the same product with no workgroup barrier in the K loop.  Wavefront w of a workgroup owns the k
-// range [32 w, 32 w + 32) of every 128-k macro step, for all 32 rows of W and all rows of A:
-//   * a lane (g = l >> 5, r = l & 31) loads the 16 codes of W row r at k 16 g .. 16 g + 15 of that range, composes
-//     them in registers, and uses codes 0..7 / 8..15 directly as its MFMA operand of the range's first / second
-//     16-k step: an MFMA may pair the k values of a step in any order as long as both operands use the same one,
-//     so the A fragment of lane (g, r') is read from k 16 g + 8 e .. + 7 as well;
-//   * the matching 64-byte pieces of the A rows come by DMA into a ring of LDS slots private to the wavefront.
-// Every wavefront is its own stream with loads D macro steps ahead; the partial sums meet once at the end.
-template <class FW, int DT_OUT, int MT, int R>
-__global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_stream_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K) {
-    constexpr int D = R - 1;                      // look-ahead in macro steps
-    constexpr int OPS = 2 + 2 * MT;               // vector-memory operations per wavefront and macro step
-    constexpr int SLOT = 32 * MT * 64;            // one macro step's A piece of a wavefront: 32 MT rows x 64 B
-    static_assert(D * OPS < 64, "vmcnt is a 6-bit counter");
-    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n0 = blockIdx.x * SK_N;
-    const int kblocks = K / 32, nmac = K / SK_MAC;
-    uint8_t* const ring = lds + wave * (R * SLOT);                                  // [R][32 MT rows][64 B]
-    const uint32_t ring_addr = (uint32_t)(uintptr_t)lds + (uint32_t)wave * (R * SLOT);
-
-    // A DMA: instruction j (of 2 MT) covers rows 16 j .. 16 j + 15; lane l fills position l & 3 of row 16 j + (l >> 2),
-    // which must hold chunk (l & 3) ^ ((row >> 2) & 3).  Rows past M re-read row M - 1.
-    uint32_t a_voff[2 * MT];
-#pragma unroll
-    for (int j = 0; j < 2 * MT; ++j) {
-        const int row = 16 * j + (lane >> 2);
-        a_voff[j] = (uint32_t)min(row, M - 1) * (uint32_t)K * 2u + (uint32_t)(((lane & 3) ^ ((row >> 2) & 3)) * 16);
-    }
-    const uint8_t* const a_base = reinterpret_cast<const uint8_t*>(a_dense) + wave * 64;       // k = 32 w
-    const uint8_t* const w_base = w_elements + (size_t)n0 * K + wave * 32;
-    const uint8_t* const ws_base = w_scales + (size_t)n0 * kblocks + wave;
-    const uint32_t w_voff = (uint32_t)(lane & 31) * (uint32_t)K + (uint32_t)(lane >> 5) * 16u;
-    const uint32_t ws_voff = (uint32_t)(lane & 31) * (uint32_t)kblocks;
-    // A fragment of 16-k step e: chunk 2 g + e of row 32 t + r
-    uint32_t f_off[2];
-#pragma unroll
-    for (int e = 0; e < 2; ++e)
-        f_off[e] = (uint32_t)(lane & 31) * 64u + (uint32_t)(((2 * (lane >> 5) + e) ^ ((lane >> 2) & 3)) * 16);
-
-    floatx16 acc[MT];
-#pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[t][v] = 0.0f;
-
-    u32x4 w_raw[R];
-    uint32_t w_scale[R];
-    // past the end the last macro step is read again (unused): the number of operations per step stays the same
-    auto issue_loads = [&](int mac, auto slot_c) {
-        constexpr int slot = decltype(slot_c)::value;
-        const int mc = min(mac, nmac - 1);
-        async_load16(w_raw[slot], w_voff, w_base + (size_t)mc * SK_MAC);
-        async_load_u8(w_scale[slot], ws_voff, ws_base + mc * (SK_MAC / 32));
-        const uint8_t* const a_src = a_base + (size_t)mc * (SK_MAC * 2);
-#pragma unroll
-        for (int j = 0; j < 2 * MT; ++j) dma_1kb(ring_addr + (uint32_t)slot * SLOT + j * 1024, a_voff[j], a_src);
-    };
-
-    static_for<D>([&](auto d_c) { issue_loads(decltype(d_c)::value, d_c); });
-    for (int base = 0; base < nmac; base += R) {
-        static_for<R>([&](auto r_c) {
-            constexpr int r = decltype(r_c)::value;
-            const int mac = base + r;
-            if (mac < nmac) {
-                issue_loads(mac + D, IntC<(r + D) % R>{});            // into the slot consumed one step ago
-                wait_vmcnt<D * OPS>(w_raw[r], w_scale[r]);             // this step's loads have arrived
-                uint4 lo, hi;
-                Composer<FW>::template compose16<true>(make_uint4(w_raw[r].x, w_raw[r].y, w_raw[r].z, w_raw[r].w), w_scale[r], lo, hi);
-                const bf16x8 wf0 = __builtin_bit_cast(bf16x8, lo), wf1 = __builtin_bit_cast(bf16x8, hi);
-                const uint8_t* const pa = ring + r * SLOT;
-#pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    const bf16x8 af0 = *reinterpret_cast<const bf16x8*>(pa + t * 2048 + f_off[0]);
-                    const bf16x8 af1 = *reinterpret_cast<const bf16x8*>(pa + t * 2048 + f_off[1]);
-                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf0, af0, acc[t], 0, 0, 0);
-                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf1, af1, acc[t], 0, 0, 0);
-                }
-                // the slot is handed back to the DMA engine in the next step: its reads must have returned
-                __builtin_amdgcn_s_waitcnt(0xC07F);
-            }
-        });
-    }
-    wait_vmcnt<0>(w_raw[0], w_scale[0]);  // the look-ahead loads still target LDS and registers
-
-    // ---- add the four wavefronts' partial sums: wavefronts 1..3 park theirs in LDS ([w-1][t][v][lane]), 0 adds
-    __syncthreads();
-    float* const red = reinterpret_cast<float*>(lds);
-    if (wave != 0) {
-#pragma unroll
-        for (int t = 0; t < MT; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) red[(((wave - 1) * MT + t) * 16 + v) * 64 + lane] = acc[t][v];
-    }
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll 1
-    for (int w = 0; w < 3; ++w)
-#pragma unroll
-        for (int t = 0; t < MT; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[t][v] += red[((w * MT + t) * 16 + v) * 64 + lane];
-    const bool vec_ok = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const int n = n0 + 8 * g + 4 * (lane >> 5);
-        float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (bias)
-            for (int t = 0; t < 4; ++t) b[t] = load_bias(bias, bias_dtype, n + t);
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const int m = 32 * t + (lane & 31);
-            if (m < M) {
-                const float r[4] = {acc[t][4 * g] + b[0], acc[t][4 * g + 1] + b[1], acc[t][4 * g + 2] + b[2], acc[t][4 * g + 3] + b[3]};
-                store_out4<DT_OUT>(y, (int64_t)m * N + n, r, vec_ok, 4);
-            }
-        }
-    }
-}
-
 template <class FW, int DT_OUT>
 int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
                        void* y, int M, int N, int K, hipStream_t s) {
     const dim3 grid((unsigned)(N / SK_N));
-    auto go_stream = [&](auto mt_c, auto r_c) {
-        constexpr int MT = decltype(mt_c)::value, R = decltype(r_c)::value;
-        constexpr int lds_bytes = 4 * R * 32 * MT * 64;   // >= the 12 MT KB the final reduction needs
-        auto kern = mxfp_gemm_stream_kernel<FW, DT_OUT, MT, R>;
-        static bool attr_done = false;
-        if (!attr_done) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
-            attr_done = true;
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
-                           bias, bias_dtype, y, M, N, K);
-        return check_launch("mxfp_gemm");
-    };
     auto go = [&](auto mt_c) {
         constexpr int MT = decltype(mt_c)::value;
         // look-ahead D (macro steps) and lines per row L: the A stages must leave LDS for two workgroups per CU
@@ -360,9 +222,6 @@ int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8
                            bias, bias_dtype, y, M, N, K);
         return check_launch("mxfp_gemm");
     };
-    // few workgroups (at most one per two CUs): the barrier-free kernel, whose weakness is address-unit load per CU
-    if (M <= 32 && N / SK_N <= 128) return go_stream(IntC<1>{}, IntC<6>{});
-    if (M <= 64 && N / SK_N <= 128) return go_stream(IntC<2>{}, IntC<4>{});
     if (M <= 16) {  // 16-row A stages leave LDS for a look-ahead of 8 macro steps
         constexpr int D = 8, L = 1, AR = 16;
         constexpr int lds_bytes = (D + 1) * AR * 256 * L + 2 * SK_N * 256 * L;

@@ -225,19 +225,28 @@ def test_gemm_large_tile_special_values(mh):
 
 
 @pytest.mark.parametrize("MNK,w_tag,odt,with_bias", [
+    # one workgroup per 16 rows of W (M <= 64 and N up to 8192, 12288 for M <= 16)
     ((1, 1024, 128), "MXFP8_E4M3_fn", torch.bfloat16, False),     # one row, a single macro step
-    ((16, 2048, 640), "OCP_MXFP4_E2M1", torch.float32, True),     # 5 macro steps: the look-ahead ring wraps once
-    ((33, 512, 1024), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # two m-tiles, the second almost empty
-    ((64, 96, 256), "MXFP8_E5M2_fn", torch.float16, False),       # three workgroups
+    ((16, 2048, 640), "OCP_MXFP4_E2M1", torch.float32, True),     # 5 macro steps, look-ahead 8: all loads in the prologue
+    ((8, 8192, 1408), "MXFP8_E4M3_fn", torch.bfloat16, False),    # 11 macro steps: the 9-slot ring wraps
+    ((12, 12288, 256), "OCP_MXFP6_E2M3", torch.float16, True),    # the largest N this kernel takes
+    ((24, 6144, 896), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # two 16-row tiles of A, look-ahead 4; 7 macro steps
+    ((33, 512, 1024), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # four tiles of A, the third holds one row
+    ((64, 8192, 512), "OCP_MXFP4_E2M1", torch.float16, False),    # four full tiles, look-ahead 2
+    ((64, 80, 256), "MXFP8_E5M2_fn", torch.float32, False),       # five workgroups; N not a multiple of 32
+    # one workgroup per 32 rows of W
+    ((8, 14336, 256), "MXFP8_E4M3_fn", torch.bfloat16, True),     # M <= 16: 16-row A stages, look-ahead 8
+    ((16, 12320, 1280), "OCP_MXFP4_E2M1", torch.float32, False),  # 10 macro steps: that ring wraps
+    ((24, 9216, 896), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # 16 < M <= 32; 7 macro steps
+    ((64, 8224, 512), "OCP_MXFP4_E2M1", torch.float16, False),    # two m-tiles
     ((100, 1024, 2048), "OCP_MXFP6_E2M3", torch.bfloat16, False), # four m-tiles, ragged
     ((128, 4096, 1536), "MXFP8_E4M3_fn", torch.float32, True),
-    ((8, 8192, 1024), "MXFP8_E4M3_fn", torch.bfloat16, False),    # many workgroups, M <= 16: 16-row A stages, look-ahead 8
-    ((24, 6144, 896), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # many workgroups, 16 < M <= 32; 7 macro steps
-    ((64, 8192, 512), "OCP_MXFP4_E2M1", torch.float16, False),    # many workgroups, two m-tiles
+    ((65, 96, 256), "MXFP8_E5M2_fn", torch.float16, False),       # three workgroups
 ])
 def test_gemm_few_rows(mh, MNK, w_tag, odt, with_bias):
-    """M <= 128 with N % 32 == 0 and K % 128 == 0 takes the kernel that streams W once (one workgroup per 32 rows of W,
-    K split over its wavefronts, partial sums added through LDS)."""
+    """M <= 128 with K % 128 == 0 takes a kernel that streams W once: one workgroup per 16 rows of W (16x16x32 MFMA) for
+    M <= 64 and moderate N, else one per 32 rows (32x32x16 MFMA, N % 32 == 0); in both K is split over the wavefronts
+    and the partial sums are added through LDS."""
     M, N, K = MNK
     g = torch.Generator().manual_seed(M * 7 + N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -256,8 +265,9 @@ def test_gemm_few_rows(mh, MNK, w_tag, odt, with_bias):
     assert rel_fro(y, y_ref.to(odt)) <= (1e-5 if odt == torch.float32 else REL_FRO_TOL)
 
 
-def test_gemm_few_rows_special_values(mh):
-    M, N, K = 8, 256, 384
+@pytest.mark.parametrize("M", [8, 40, 100])  # 16-row kernel with one / four tiles of A, 32-row kernel
+def test_gemm_few_rows_special_values(mh, M):
+    N, K = 256, 384
     g = torch.Generator().manual_seed(13)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = torch.randn(N, K, generator=g).to(torch.bfloat16)
@@ -439,15 +449,16 @@ def test_mxfp_matmul_fused_routes(mh, a_shape, b_shape, dtype):
 
 
 def test_gemm_dispatch_boundaries(mh):
-    """Shapes on both sides of every kernel-selection threshold (rows 128 / 129, 511 / 512 / 513; N and K that do
+    """Shapes on both sides of every kernel-selection threshold (rows 16 / 17, 64 / 65, 128 / 129, 511 / 512 / 513; N and K that do
     or do not divide by the tile sizes; few and many tiles), each against fp32 dequantize-then-matmul on the GPU."""
     g = torch.Generator().manual_seed(99)
     fmt = preset(mh, "MXFP8_E4M3_fn")
     shapes = []
-    for M in (1, 127, 128, 129, 255, 256, 257, 383, 511, 512, 513, 640, 1023, 1025):
-        for N, K in ((128, 128), (96, 128), (160, 160), (256, 384), (384, 96)):
+    for M in (1, 16, 17, 32, 33, 64, 65, 127, 128, 129, 255, 256, 257, 383, 511, 512, 513, 640, 1023, 1025):
+        for N, K in ((128, 128), (96, 128), (160, 160), (256, 384), (384, 96), (48, 256)):
             shapes.append((M, N, K))
-    shapes += [(129, 12288, 128), (511, 12288, 128), (512, 12288, 128), (513, 12288, 256), (640, 12416, 128), (130, 4160, 256)]
+    shapes += [(16, 12288, 128), (16, 12304, 128), (17, 8192, 128), (17, 12288, 128), (64, 8208, 128), (64, 8224, 128),
+               (129, 12288, 128), (511, 12288, 128), (512, 12288, 128), (513, 12288, 256), (640, 12416, 128), (130, 4160, 256)]
     worst = 0.0
     for M, N, K in shapes:
         x = torch.randn(M, K, generator=g).to(torch.bfloat16)
