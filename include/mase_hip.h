@@ -8,9 +8,11 @@
  * checkout) and takes what that function takes, flattened to plain pointers and sizes.
  *
  * Conventions
- *   - All pointers are DEVICE pointers on the current HIP device.  The library never
- *     allocates, frees or synchronises; work is enqueued on `stream` (a hipStream_t, NULL for
- *     the default stream) and the call returns immediately.
+ *   - All pointers are DEVICE pointers on the current HIP device, and `stream` (a hipStream_t,
+ *     NULL for the default stream) belongs to it: make the device current (hipSetDevice) before
+ *     the call.  The library never allocates, frees or synchronises; work is enqueued on
+ *     `stream` and the call returns immediately.  Calls may come from several host threads and
+ *     for several devices of one process.
  *   - dtype codes:      0 = float32, 1 = float16, 2 = bfloat16   (MASE_F32/F16/BF16)
  *   - round_mode codes: 0 = rn (nearest even), 1 = ru, 2 = rd, 3 = rz
  *   - is_finite != 0: the all-ones exponent is an ordinary binade (the reference's "_fn"

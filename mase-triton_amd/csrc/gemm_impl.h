@@ -516,17 +516,6 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
         }
 }
 
-inline int device_cu_count() {
-    static int n_cus = 0;
-    if (n_cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
-        n_cus = prop.multiProcessorCount > 8 ? prop.multiProcessorCount : 8;
-    }
-    return n_cus;
-}
-
 template <int A_MODE, class FA, class FW, int DT_OUT>
 int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_elements, const uint8_t* w_scales,
                 const uint8_t* w_elements, const void* bias, int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
@@ -564,7 +553,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
                              (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0;
         if (mid_ok || wide_ok || tall_ok) {
             const int cus = device_cu_count();
-            if (cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
+            if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
             const int64_t n128 = N / 128;
             auto cost = [&](int tile_rows, double tile_time) {
                 const int64_t tiles = (int64_t)((M + tile_rows - 1) / tile_rows) * n128;
@@ -580,12 +569,8 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             const int tall_tiles_m = (M + UM - 1) / UM;
             const int64_t tall_tiles = (int64_t)tall_tiles_m * (N / UN);
             auto kern = mxfp_gemm_tall_kernel<FW, DT_OUT>;
-            static bool attr_done = false;
-            if (!attr_done) {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, U_LDS_BYTES);
-                if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
-                attr_done = true;
-            }
+            static std::atomic<uint64_t> lds_allowed{0};
+            if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed)) return rc;
             // one persistent workgroup per CU (a multiple of the 8 XCDs), never more than tiles
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
             hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
@@ -597,14 +582,10 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         const bool guard_k = K % TK != 0;
         auto kern = guard_k ? mxfp_gemm_kernel<A_MODE, FA, FW, DT_OUT, true> : mxfp_gemm_kernel<A_MODE, FA, FW, DT_OUT, false>;
         constexpr int lds_bytes = 4 * SLAB_BYTES;
-        static bool attr_set[2] = {false, false};
-        if (!attr_set[guard_k]) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
-            attr_set[guard_k] = true;
-        }
+        static std::atomic<uint64_t> lds_allowed[2];
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed[guard_k])) return rc;
         const int n_cus = device_cu_count();
-        if (n_cus <= 0) return fail(ERR_RUNTIME, "hipGetDeviceProperties failed");
+        if (n_cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
         // one persistent workgroup per CU (rounded down to a multiple of 8 XCD slots), never more than tiles
         const int64_t want = big_tiles < n_cus ? ((big_tiles + 7) / 8) * 8 : (n_cus / 8) * 8;
         const unsigned grid = (unsigned)want;

@@ -270,12 +270,8 @@ template <class FW, int DT_OUT, int KS>
 int launch_gemm_mid(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
                     void* y, int M, int N, int K, hipStream_t s) {
     auto kern = mxfp_gemm_mid_kernel<FW, DT_OUT, KS>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, MD_LDS_BYTES);
-        if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), MD_LDS_BYTES, lds_allowed)) return rc;
     const int tiles_m = (M + MD_M - 1) / MD_M;
     const int64_t tiles = (int64_t)tiles_m * (N / MD_N);
     if (tiles > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "too many tiles for one launch");

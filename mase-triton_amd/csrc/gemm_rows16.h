@@ -187,12 +187,8 @@ int launch_gemm_rows16(const void* a_dense, const uint8_t* w_scales, const uint8
                        void* y, int M, int N, int K, hipStream_t s) {
     constexpr int lds_bytes = (D + 1) * 16 * MT * 256 + 2 * R16_N * 256;  // >= the 3 MT KB the final reduction needs
     auto kern = mxfp_gemm_rows16_kernel<FW, DT_OUT, MT, D>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed)) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)(N / R16_N)), dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales,
                        w_elements, bias, bias_dtype, y, M, N, K);
     return check_launch("mxfp_gemm");

@@ -212,12 +212,8 @@ int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8
         constexpr int D = MT == 1 ? 4 : MT == 2 ? 2 : 1, L = 1, AR = 32;
         constexpr int lds_bytes = (D + 1) * AR * MT * 256 * L + 2 * SK_N * 256 * L;
         auto kern = mxfp_gemm_skinny_kernel<FW, DT_OUT, MT, D, L, AR>;
-        static bool attr_done = false;
-        if (!attr_done) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
-            attr_done = true;
-        }
+        static std::atomic<uint64_t> lds_allowed{0};
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed)) return rc;
         hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
                            bias, bias_dtype, y, M, N, K);
         return check_launch("mxfp_gemm");
@@ -226,12 +222,8 @@ int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8
         constexpr int D = 8, L = 1, AR = 16;
         constexpr int lds_bytes = (D + 1) * AR * 256 * L + 2 * SK_N * 256 * L;
         auto kern = mxfp_gemm_skinny_kernel<FW, DT_OUT, 1, D, L, AR>;
-        static bool attr16_done = false;
-        if (!attr16_done) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-            if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
-            attr16_done = true;
-        }
+        static std::atomic<uint64_t> lds_allowed{0};
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed)) return rc;
         hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
                            bias, bias_dtype, y, M, N, K);
         return check_launch("mxfp_gemm");

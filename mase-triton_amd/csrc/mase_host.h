@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <string>
 
 #include "mase_device.h"
@@ -23,6 +24,36 @@ inline int check_launch(const char* what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(ERR_RUNTIME, std::string(what) + ": " + hipGetErrorString(e));
     return OK;
+}
+
+// A kernel that uses more than 64 KB of dynamic LDS has to be given the limit once on every device it runs on (the
+// attribute belongs to the function as loaded on the current device).  `done` is the call site's record: bit d = set on
+// device d; devices past 63 set it on every launch.  Safe from several threads (setting it twice is harmless).
+inline int allow_dynamic_lds(const void* kern, int bytes, std::atomic<uint64_t>& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipGetDevice: ") + hipGetErrorString(e));
+    const uint64_t bit = dev >= 0 && dev < 64 ? uint64_t(1) << dev : 0;
+    if (bit && (done.load(std::memory_order_relaxed) & bit)) return OK;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipFuncSetAttribute: ") + hipGetErrorString(e));
+    done.fetch_or(bit, std::memory_order_relaxed);
+    return OK;
+}
+
+// compute units of the current device (at least 8), or -1
+inline int device_cu_count() {
+    static std::atomic<int> cus[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return -1;
+    const bool cached = dev >= 0 && dev < 64;
+    int n = cached ? cus[dev].load(std::memory_order_relaxed) : 0;
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
+        n = n > 8 ? n : 8;
+        if (cached) cus[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
 }
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
