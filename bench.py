@@ -310,17 +310,23 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e6 / steps
 
+    def linear_rows(n_out, k_in, Ms):
+        wt = (0.02 * torch.randn(n_out, k_in, generator=gen, device=dev)).to(torch.bfloat16)
+        sc, el, tm = MXFP_F.extract_mxfp_components(wt, block_dim=1, mxfp_meta=fmt)
+        out = []
+        for M in Ms:
+            x = torch.randn(M, k_in, generator=gen, device=dev).to(torch.bfloat16)
+            call = dict(x=x, x_meta=fmt, w=None, w_scales=sc, w_elements=el, w_tensor_meta=tm, b=None, b_scales=None,
+                        b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
+            f_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="fused"))
+            s_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="separate"))
+            out.append({"M": M, "fused_us": round(f_us, 1), "separate_us": round(s_us, 1),
+                        "fused_TFLOPs": round(2.0 * M * n_out * k_in / f_us / 1e6, 1)})
+        return out
+
+    rows = linear_rows(N, K, (16, 64, 128, 256, 384, 512, 1024, 2048, 4096))
+    rows_down = linear_rows(K, N, (16, 64, 256, 1024, 4096))  # the transposed layer shape: few W rows, long K
     w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
-    w_sc, w_el, w_tm = MXFP_F.extract_mxfp_components(w, block_dim=1, mxfp_meta=fmt)
-    rows = []
-    for M in (16, 64, 128, 256, 384, 512, 1024, 2048, 4096):
-        x = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
-        call = dict(x=x, x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
-                    b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
-        f_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="fused"))
-        s_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="separate"))
-        rows.append({"M": M, "fused_us": round(f_us, 1), "separate_us": round(s_us, 1),
-                     "fused_TFLOPs": round(2.0 * M * N * K / f_us / 1e6, 1)})
     n = w.numel()
     cast = {
         "shape": [N, K], "block_axis": 0,
@@ -331,7 +337,7 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
     }
     cast["extract_in_place_GBps"] = round(n * (3 + 1 / 32) / cast["extract_in_place_us"] / 1e3, 0)
     cast["qdq_in_place_GBps"] = round(n * 4 / cast["qdq_in_place_us"] / 1e3, 0)
-    return {"linear_N14336_K4096": rows, "casts_along_axis0": cast}
+    return {"linear_N14336_K4096": rows, "linear_N4096_K14336": rows_down, "casts_along_axis0": cast}
 
 
 def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):

@@ -175,6 +175,35 @@ int mase_hip_mxfp_gemm(const void* a_dense, int a_dtype, const uint8_t* a_scales
                        int w_frac_bits, const void* bias, int bias_dtype, void* y, int out_dtype,
                        int64_t M, int64_t N, int64_t K, int block_size, void* stream);
 
+/*
+ * The same product with room for partial sums.  A product with few output tiles and a long K
+ * (say a [256, 4096] output over K = 14336: 64 tiles of 128 x 128 for 256 compute units) runs
+ * several times faster when K is split over several workgroups per tile; the splits leave fp32
+ * partial sums in `workspace` and a second kernel on the same stream adds them, adds the bias
+ * and rounds to out_dtype.  The library allocates nothing, so the caller brings the memory:
+ *
+ *   mase_hip_mxfp_gemm_workspace_bytes(a_is_dense, M, N, K)
+ *       bytes with which this shape would be split on the current device, 0 if it would not
+ *       (MXFP A, enough tiles, short K, sizes the split kernel does not take).
+ *   mase_hip_mxfp_gemm_ws(..., workspace, workspace_bytes, stream)
+ *       `workspace`: 16-byte aligned device memory of at least that many bytes, or NULL.  With
+ *       NULL, or fewer bytes than the shape asks for, the call is mase_hip_mxfp_gemm.  The
+ *       contents before the call do not matter and are undefined after it; calls that share
+ *       a workspace must be ordered on one stream.
+ *
+ * The result differs from mase_hip_mxfp_gemm's only in the order of the fp32 additions.
+ * Same reference counterpart as mase_hip_mxfp_gemm (src/mase_triton/mxfp/functional/linear.py:
+ * 31-32,50-64); the reference has no workspace argument because its GEMM is torch's, which
+ * allocates its own.
+ */
+int64_t mase_hip_mxfp_gemm_workspace_bytes(int a_is_dense, int64_t M, int64_t N, int64_t K);
+int mase_hip_mxfp_gemm_ws(const void* a_dense, int a_dtype, const uint8_t* a_scales,
+                          const uint8_t* a_elements, int a_exp_bits, int a_frac_bits,
+                          const uint8_t* w_scales, const uint8_t* w_elements, int w_exp_bits,
+                          int w_frac_bits, const void* bias, int bias_dtype, void* y,
+                          int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

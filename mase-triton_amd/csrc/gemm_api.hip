@@ -4,10 +4,10 @@
 
 using namespace mase;
 
-extern "C" int mase_hip_mxfp_gemm(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements,
-                                  int a_exp_bits, int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements,
-                                  int w_exp_bits, int w_frac_bits, const void* bias, int bias_dtype, void* y, int out_dtype,
-                                  int64_t M, int64_t N, int64_t K, int block_size, void* stream) {
+static int gemm_entry(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements, int a_exp_bits,
+                      int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements, int w_exp_bits, int w_frac_bits,
+                      const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
+                      void* workspace, int64_t workspace_bytes, void* stream) {
     if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(ERR_INVALID, "M, N, K must fit in 31 bits");
     if (block_size != 32) return fail(ERR_UNSUPPORTED, "the GEMM supports block_size 32 only");
@@ -24,12 +24,37 @@ extern "C" int mase_hip_mxfp_gemm(const void* a_dense, int a_dtype, const uint8_
         if (!aligned(a_elements, 16)) return fail(ERR_INVALID, "a_elements must be 16-byte aligned");
     }
     if (!aligned(w_elements, 16)) return fail(ERR_INVALID, "w_elements must be 16-byte aligned");
+    if (workspace_bytes < 0) return fail(ERR_INVALID, "workspace_bytes must not be negative");
+    if (workspace && !aligned(workspace, 16)) return fail(ERR_INVALID, "workspace must be 16-byte aligned");
+    if (!workspace) workspace_bytes = 0;
     const GemmArgs g{a_dense, a_scales, a_elements, a_is_dense ? 0 : a_exp_bits, a_frac_bits, w_scales, w_elements, bias, bias_dtype,
-                     y, out_dtype, (int)M, (int)N, (int)K, static_cast<hipStream_t>(stream)};
+                     y, out_dtype, (int)M, (int)N, (int)K, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
     if (w_exp_bits == 4 && w_frac_bits == 3) return gemm_w_e4m3(g);
     if (w_exp_bits == 5 && w_frac_bits == 2) return gemm_w_e5m2(g);
     if (w_exp_bits == 2 && w_frac_bits == 3) return gemm_w_e2m3(g);
     if (w_exp_bits == 3 && w_frac_bits == 2) return gemm_w_e3m2(g);
     if (w_exp_bits == 2 && w_frac_bits == 1) return gemm_w_e2m1(g);
     return fail(ERR_INVALID, "MXFP element (exp_bits, frac_bits) must be one of (4,3) (5,2) (2,3) (3,2) (2,1)");
+}
+
+extern "C" int mase_hip_mxfp_gemm(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements,
+                                  int a_exp_bits, int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements,
+                                  int w_exp_bits, int w_frac_bits, const void* bias, int bias_dtype, void* y, int out_dtype,
+                                  int64_t M, int64_t N, int64_t K, int block_size, void* stream) {
+    return gemm_entry(a_dense, a_dtype, a_scales, a_elements, a_exp_bits, a_frac_bits, w_scales, w_elements, w_exp_bits, w_frac_bits,
+                      bias, bias_dtype, y, out_dtype, M, N, K, block_size, nullptr, 0, stream);
+}
+
+extern "C" int mase_hip_mxfp_gemm_ws(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements,
+                                     int a_exp_bits, int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements,
+                                     int w_exp_bits, int w_frac_bits, const void* bias, int bias_dtype, void* y, int out_dtype,
+                                     int64_t M, int64_t N, int64_t K, int block_size, void* workspace, int64_t workspace_bytes,
+                                     void* stream) {
+    return gemm_entry(a_dense, a_dtype, a_scales, a_elements, a_exp_bits, a_frac_bits, w_scales, w_elements, w_exp_bits, w_frac_bits,
+                      bias, bias_dtype, y, out_dtype, M, N, K, block_size, workspace, workspace_bytes, stream);
+}
+
+extern "C" int64_t mase_hip_mxfp_gemm_workspace_bytes(int a_is_dense, int64_t M, int64_t N, int64_t K) {
+    if (!a_is_dense || M < 1 || N < 1 || K < 1 || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return 0;
+    return plan_split_k((int)M, (int)N, (int)K, device_cu_count()).workspace_bytes((int)M, (int)N);
 }

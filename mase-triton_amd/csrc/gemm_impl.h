@@ -518,12 +518,21 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
 
 template <int A_MODE, class FA, class FW, int DT_OUT>
 int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_elements, const uint8_t* w_scales,
-                const uint8_t* w_elements, const void* bias, int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
+                const uint8_t* w_elements, const void* bias, int bias_dtype, void* y, int M, int N, int K, void* workspace,
+                int64_t workspace_bytes, hipStream_t s) {
     const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
     const int64_t big_tiles = (int64_t)tiles_m * tiles_n;
     // 256 x 256 tiles need enough of them to occupy the 256 CUs; smaller problems use 128 x 128
     const bool fits32 = (int64_t)M * K * 2 < ((int64_t)1 << 32) && (int64_t)N * K < ((int64_t)1 << 32);  // 32-bit operand offsets
     const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
+    if constexpr (A_MODE == 0) {
+        // few tiles and a long K: with a workspace, K is split over several workgroups per tile
+        if (workspace && fits32 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
+            const SplitPlan plan = plan_split_k(M, N, K, device_cu_count());
+            if (plan.splits > 1 && workspace_bytes >= plan.workspace_bytes(M, N))
+                return launch_gemm_mid_split_k<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, plan, workspace, s);
+        }
+    }
     if constexpr (A_MODE == 0) {
         // fewest rows of A and not many rows of W: one workgroup per 16 rows of W, so that there are enough workgroups
         // (the 32-row kernel below has N / 32; measured better up to N = 12288 for M <= 16 and up to N = 8192 for M <= 64)
@@ -607,7 +616,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
 struct GemmArgs {
     const void* a_dense; const uint8_t* a_scales; const uint8_t* a_elements; int a_exp_bits, a_frac_bits;
     const uint8_t* w_scales; const uint8_t* w_elements; const void* bias; int bias_dtype; void* y; int out_dtype;
-    int M, N, K; hipStream_t stream;
+    int M, N, K; void* workspace; int64_t workspace_bytes; hipStream_t stream;
 };
 int gemm_w_e4m3(const GemmArgs& g);
 int gemm_w_e5m2(const GemmArgs& g);
@@ -621,12 +630,12 @@ int gemm_for_weight_format(const GemmArgs& g) {
         constexpr int DO = decltype(dout)::value;
         if (g.a_dense)
             return launch_gemm<0, SFmt<4, 3>, FW, DO>(g.a_dense, nullptr, nullptr, g.w_scales, g.w_elements, g.bias, g.bias_dtype, g.y,
-                                                      g.M, g.N, g.K, g.stream);
+                                                      g.M, g.N, g.K, g.workspace, g.workspace_bytes, g.stream);
         const int E = g.a_exp_bits, M = g.a_frac_bits;
 #define MASE_A_FMT(e, m)                                                                                                       \
         if (E == e && M == m)                                                                                                  \
             return launch_gemm<1, SFmt<e, m>, FW, DO>(nullptr, g.a_scales, g.a_elements, g.w_scales, g.w_elements, g.bias,     \
-                                                      g.bias_dtype, g.y, g.M, g.N, g.K, g.stream);
+                                                      g.bias_dtype, g.y, g.M, g.N, g.K, nullptr, 0, g.stream);
         MASE_A_FMT(4, 3) MASE_A_FMT(5, 2) MASE_A_FMT(2, 3) MASE_A_FMT(3, 2) MASE_A_FMT(2, 1)
 #undef MASE_A_FMT
         return fail(ERR_INVALID, "MXFP element (exp_bits, frac_bits) must be one of (4,3) (5,2) (2,3) (3,2) (2,1)");

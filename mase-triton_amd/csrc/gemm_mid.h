@@ -32,7 +32,8 @@ constexpr int MD_LDS_BYTES = MD_A_STAGES * MD_A_STAGE + 2 * MD_W_STAGE;  // 160 
 template <class FW, int DT_OUT, int KS>
 __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
     const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m) {
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y_all, int M, int N, int K, int tiles_m, int k_len,
+    int64_t y_split_bytes) {
     constexpr int WAVES = 4 * KS, QW = 8 / KS;             // 16-k steps per wavefront and macro step
     constexpr int A_DMAS = MD_A_STAGE / 1024 / WAVES;      // per wavefront and macro step
     constexpr int W_LOADS = MD_N * MD_MAC / 16 / (64 * WAVES);  // code loads (and as many scale loads) per lane
@@ -48,7 +49,12 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
     // m-tile fastest: the workgroups that share 128 rows of W run next to each other in time
     const int tile_m = (int)(blockIdx.x % (unsigned)tiles_m), tile_n = (int)(blockIdx.x / (unsigned)tiles_m);
     const int m0 = tile_m * MD_M, n0 = tile_n * MD_N;
-    const int kblocks = K / 32, nmac = K / MD_MAC;
+    // blockIdx.y = split of K: this workgroup multiplies k in [k_begin, k_begin + k_len) (the last split may be shorter)
+    // and writes its sums to its own [M, N] array, y_split_bytes apart.  One split: k_len = K.
+    const int k_begin = (int)blockIdx.y * k_len;
+    const int kblocks = K / 32, nmac = min(k_len, K - k_begin) / MD_MAC;
+    a_dense += k_begin;
+    void* const y = static_cast<uint8_t*>(y_all) + (size_t)blockIdx.y * (size_t)y_split_bytes;
 
     // A DMA: an instruction moves 1 KB = 4 rows; lane l fills position l % 16 of row 4 (8 w + j) + l / 16, which must
     // hold chunk (l % 16) ^ (row & 15).  Rows past M re-read row M - 1 (their products are never stored).
@@ -60,8 +66,8 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
     }
     // W: the wavefront loads 8 W_LOADS rows as whole lines: lane = 16 codes (16 k) of its row 8 h + (l >> 3)
     const int w_chunk = lane & 7;
-    const uint8_t* const w_base = w_elements + (size_t)(n0 + wave * (8 * W_LOADS)) * K;          // wave-uniform
-    const uint8_t* const ws_base = w_scales + (size_t)(n0 + wave * (8 * W_LOADS)) * kblocks;
+    const uint8_t* const w_base = w_elements + (size_t)(n0 + wave * (8 * W_LOADS)) * K + k_begin;          // wave-uniform
+    const uint8_t* const ws_base = w_scales + (size_t)(n0 + wave * (8 * W_LOADS)) * kblocks + k_begin / 32;
     uint32_t w_voff[W_LOADS], ws_voff[W_LOADS], w_lds_off[W_LOADS][2];
 #pragma unroll
     for (int h = 0; h < W_LOADS; ++h) {
@@ -89,7 +95,7 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
     uint32_t w_scale[3][W_LOADS];
     // workgroups start at different macro steps of K (and wrap around), so that at any moment they read different
     // columns of W and A: addresses that spread over the memory channels
-    const int rot = (int)((unsigned)tile_n % (unsigned)nmac);
+    const int rot = (int)((unsigned)(tile_n + blockIdx.y) % (unsigned)nmac);
     // past the end the last macro step is read again (unused), which keeps the operation count per step, and with
     // it the wait counts, the same
     auto k_of = [&](int mac) __attribute__((always_inline)) {
@@ -276,6 +282,73 @@ int launch_gemm_mid(const void* a_dense, const uint8_t* w_scales, const uint8_t*
     const int64_t tiles = (int64_t)tiles_m * (N / MD_N);
     if (tiles > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "too many tiles for one launch");
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256 * KS), MD_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                       w_elements, bias, bias_dtype, y, M, N, K, tiles_m);
+                       w_elements, bias, bias_dtype, y, M, N, K, tiles_m, K, (int64_t)0);
+    return check_launch("mxfp_gemm");
+}
+
+// ---------------------------------------------------------------------------------------------
+// K split over several workgroups per tile, for products with few tiles and a long K (a [256, 4096] output has 64 tiles
+// for 256 CUs): split z multiplies its share of K into the fp32 array partial[z][M][N] of a caller-provided workspace,
+// and a second kernel adds the arrays, the bias, and rounds to the output type.
+
+struct SplitPlan {
+    int splits;  // 1: do not split
+    int k_len;   // k per split, a multiple of the macro step
+    int64_t workspace_bytes(int M, int N) const { return splits > 1 ? (int64_t)splits * M * N * 4 : 0; }
+};
+
+// The same plan for the size query and the launch: it depends on the shape and the CU count only.
+inline SplitPlan plan_split_k(int M, int N, int K, int cus) {
+    SplitPlan p{1, K};
+    // up to 64 rows the weight-streaming kernels are as fast or faster (64 x 4096 x 4096: 14.5 us against 20.4 us split)
+    if (M <= 64 || N % MD_N != 0 || K % MD_MAC != 0 || cus <= 0) return p;
+    const int64_t tiles = (int64_t)((M + MD_M - 1) / MD_M) * (N / MD_N);
+    const int nmac = K / MD_MAC;
+    if (tiles * 2 > cus) return p;                                 // a second workgroup per tile would not find a free CU
+    int want = (int)(cus / tiles);
+    if (want > nmac / 4) want = nmac / 4;                          // at least four macro steps per split
+    if (want > 16) want = 16;
+    if (want < 2) return p;
+    const int mac_per = (nmac + want - 1) / want;
+    p.k_len = mac_per * MD_MAC;
+    p.splits = (nmac + mac_per - 1) / mac_per;                     // no empty split
+    return p;
+}
+
+template <int DT_OUT>
+__global__ __launch_bounds__(256) void split_k_reduce_kernel(const float* __restrict__ partial, int splits, int64_t mn, int N,
+                                                             const void* __restrict__ bias, int bias_dtype, void* __restrict__ y) {
+    // a lane adds four consecutive outputs of every split (N % 4 == 0: they share a row)
+    const int64_t o = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (o >= mn) return;
+    float4 acc = *reinterpret_cast<const float4*>(partial + o);
+    for (int z = 1; z < splits; ++z) {
+        const float4 v = *reinterpret_cast<const float4*>(partial + (size_t)z * mn + o);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    float r[4] = {acc.x, acc.y, acc.z, acc.w};
+    if (bias) {
+        const int n = (int)(o % N);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) r[t] += load_bias(bias, bias_dtype, n + t);
+    }
+    store_out4<DT_OUT>(y, o, r, (reinterpret_cast<uintptr_t>(y) & 15) == 0, 4);
+}
+
+template <class FW, int DT_OUT>
+int launch_gemm_mid_split_k(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
+                            void* y, int M, int N, int K, const SplitPlan& plan, void* workspace, hipStream_t s) {
+    auto kern = mxfp_gemm_mid_kernel<FW, F32, 2>;
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), MD_LDS_BYTES, lds_allowed)) return rc;
+    const int tiles_m = (M + MD_M - 1) / MD_M;
+    const int64_t tiles = (int64_t)tiles_m * (N / MD_N);
+    const int64_t mn = (int64_t)M * N;
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)plan.splits), dim3(512), MD_LDS_BYTES, s,
+                       static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace, M, N, K,
+                       tiles_m, plan.k_len, mn * 4);
+    if (int rc = check_launch("mxfp_gemm")) return rc;
+    hipLaunchKernelGGL(split_k_reduce_kernel<DT_OUT>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const float*>(workspace), plan.splits, mn, N, bias, bias_dtype, y);
     return check_launch("mxfp_gemm");
 }

@@ -28,6 +28,9 @@ SIGNATURES = {
     "mase_hip_unpack_codes": (_i32, [_vp, _vp, _i64, _i32, _vp]),
     "mase_hip_mxfp_gemm": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
                                   _vp, _i32, _i64, _i64, _i64, _i32, _vp]),
+    "mase_hip_mxfp_gemm_ws": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
+                                     _vp, _i32, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
+    "mase_hip_mxfp_gemm_workspace_bytes": (_i64, [_i32, _i64, _i64, _i64]),
 }
 
 

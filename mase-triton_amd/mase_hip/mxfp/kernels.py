@@ -132,12 +132,15 @@ def mxfp_gemm(
     K: int,
     output_dtype: torch.dtype,
     out: Tensor | None = None,
+    split_k: bool = True,
 ) -> Tensor:
     """y[M,N] = A[M,K] @ W[N,K]^T (+ bias) on bf16 MFMA with fp32 accumulation.
 
     A is either a dense [M,K] tensor (``a``; used as is) or MXFP components blocked along K.
     W is MXFP components of the row-major [N,K] weight, blocked along K.
     ``out``: optional contiguous [M,N] tensor of ``output_dtype`` to write into.
+    ``split_k``: allow a temporary for partial sums (a few M*N*4 bytes) where the library asks for one;
+    False keeps the call free of allocations other than the output.
     """
     dev = w_elements.device
     _lib.require_gpu(w_elements, "w_elements")
@@ -168,9 +171,13 @@ def mxfp_gemm(
     else:
         assert out.is_contiguous() and out.dtype == output_dtype and out.numel() == M * N and out.device == dev
         y = out
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        _lib.check(_lib.load().mase_hip_mxfp_gemm(
+        # few output tiles and a long K: the library splits K over more workgroups if it is given room for the partial sums
+        ws_bytes = lib.mase_hip_mxfp_gemm_workspace_bytes(int(a is not None), M, N, K) if split_k else 0
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
+        _lib.check(lib.mase_hip_mxfp_gemm_ws(
             a_ptr, a_dt, a_sc_ptr, a_el_ptr, a_e, a_m, w_scales.data_ptr(), w_elements.data_ptr(),
             w_meta.element_exp_bits, w_meta.element_frac_bits, b_ptr, b_dt, y.data_ptr(),
-            _lib.dtype_code(output_dtype), M, N, K, 32, _lib.stream_ptr(dev)))
+            _lib.dtype_code(output_dtype), M, N, K, 32, None if ws is None else ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
     return y

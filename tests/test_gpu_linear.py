@@ -239,8 +239,9 @@ def test_gemm_large_tile_special_values(mh):
     ((16, 12320, 1280), "OCP_MXFP4_E2M1", torch.float32, False),  # 10 macro steps: that ring wraps
     ((24, 9216, 896), "OCP_MXFP6_E3M2", torch.bfloat16, True),    # 16 < M <= 32; 7 macro steps
     ((64, 8224, 512), "OCP_MXFP4_E2M1", torch.float16, False),    # two m-tiles
-    ((100, 1024, 2048), "OCP_MXFP6_E2M3", torch.bfloat16, False), # four m-tiles, ragged
-    ((128, 4096, 1536), "MXFP8_E4M3_fn", torch.float32, True),
+    ((100, 1024, 896), "OCP_MXFP6_E2M3", torch.bfloat16, False),  # four m-tiles, ragged; fewer workgroups than CUs: look-ahead 3
+    ((128, 16512, 256), "MXFP8_E4M3_fn", torch.float32, True),    # four m-tiles, 516 workgroups: look-ahead 1
+    ((128, 4096, 1536), "MXFP8_E4M3_fn", torch.float32, True),    # (K long enough to be split over workgroups instead)
     ((65, 96, 256), "MXFP8_E5M2_fn", torch.float16, False),       # three workgroups
 ])
 def test_gemm_few_rows(mh, MNK, w_tag, odt, with_bias):
@@ -323,6 +324,97 @@ def test_gemm_mid_rows(mh, MNK, w_tag, odt, with_bias):
     if b is not None:
         y_ref = y_ref + b[cols]
     assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref.to(odt)) <= (1e-5 if odt == torch.float32 else REL_FRO_TOL)
+
+
+@pytest.mark.parametrize("MNK,splits,w_tag,odt,with_bias", [
+    ((256, 512, 2048), 4, "MXFP8_E4M3_fn", torch.bfloat16, True),      # 8 tiles, 16 macro steps of K: 4 splits of 4
+    ((511, 1024, 1664), 3, "OCP_MXFP6_E3M2", torch.float32, False),    # 13 macro steps as 5 + 5 + 3, ragged M
+    ((250, 1024, 1152), 2, "OCP_MXFP4_E2M1", torch.bfloat16, True),    # 9 macro steps as 5 + 4
+    ((100, 1024, 2048), 4, "OCP_MXFP6_E2M3", torch.float16, True),     # one row of tiles, most of its rows past M
+    ((65, 128, 8192), 16, "MXFP8_E5M2_fn", torch.bfloat16, False),     # a single tile, 16 splits (the most)
+    ((384, 4096, 1024), 2, "MXFP8_E4M3_fn", torch.bfloat16, False),    # 96 tiles: a second workgroup per tile still fits
+])
+def test_gemm_split_k(mh, MNK, splits, w_tag, odt, with_bias):
+    """Few 128 x 128 output tiles and a long K: given a workspace the library splits K over several workgroups per tile
+    (fp32 partial sums, then a kernel that adds them and the bias).  Checked against the CPU checker and against the
+    same call without a workspace."""
+    from mase_hip import _lib
+
+    M, N, K = MNK
+    assert _lib.load().mase_hip_mxfp_gemm_workspace_bytes(1, M, N, K) == splits * M * N * 4
+    assert _lib.load().mase_hip_mxfp_gemm_workspace_bytes(0, M, N, K) == 0   # MXFP A is not split
+    g = torch.Generator().manual_seed(M + 5 * N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.float32) if with_bias else None
+    we, wm = PRESETS[w_tag]
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    w_sc, w_el = oracle.extract_mxfp(w, 32, we, wm)
+    w_dq = oracle.compose_mxfp(w_sc, w_el, 32, we, wm, True, torch.bfloat16).view(N, K)
+    args = (x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, w_tag), None if b is None else b.to(DEV),
+            M, N, K, odt)
+    y = mh.mxk.mxfp_gemm(*args)
+    assert y.shape == (M, N) and y.dtype == odt
+    y_ref = oracle.matmul_nt(x_dq, w_dq)
+    if b is not None:
+        y_ref = y_ref + b.float()
+    tol = 1e-5 if odt == torch.float32 else REL_FRO_TOL
+    assert rel_fro(y, y_ref.to(odt)) <= tol
+    y_plain = mh.mxk.mxfp_gemm(*args, split_k=False)
+    assert rel_fro(y, y_plain) <= tol
+    if odt == torch.float32:
+        assert not torch.equal(y, y_plain)  # another order of additions: equality would mean K was not split
+
+
+def test_gemm_split_k_special_values(mh):
+    M, N, K = 200, 256, 2048
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    w[77, 300] = float("inf")      # first split
+    w[130, 1999] = float("nan")    # last split
+    w_sc, w_el = oracle.extract_mxfp(w, 32, 4, 3)
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    y = mh.mxk.mxfp_gemm(x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), None,
+                         M, N, K, torch.bfloat16).cpu()
+    bad = torch.zeros(N, dtype=torch.bool)
+    bad[77] = bad[130] = True
+    assert y[:, bad].isnan().all()
+    assert y[:, ~bad].isfinite().all()
+
+
+def test_gemm_workspace_too_small_or_absent(mh):
+    """The C entry point with a workspace falls back to the unsplit product when the workspace is missing or short."""
+    from mase_hip import _lib
+
+    lib = _lib.load()
+    M, N, K = 256, 512, 2048
+    g = torch.Generator(device=DEV).manual_seed(8)
+    a = mh.mxk.quantize_dequantize(torch.randn(M * K, generator=g, device=DEV).to(torch.bfloat16), preset(mh, "MXFP8_E4M3_fn"),
+                                   torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g, device=DEV)).to(torch.bfloat16)
+    w_sc, w_el = mh.mxk.extract_mxfp_components(w.view(-1), preset(mh, "MXFP8_E4M3_fn"))
+    need = lib.mase_hip_mxfp_gemm_workspace_bytes(1, M, N, K)
+    assert need == 4 * M * N * 4
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+
+    def run(ws_ptr, ws_bytes):
+        y = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+        rc = lib.mase_hip_mxfp_gemm_ws(a.data_ptr(), 2, None, None, 0, 0, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, None, 0,
+                                       y.data_ptr(), 0, M, N, K, 32, ws_ptr, ws_bytes, _lib.stream_ptr(torch.device(DEV)))
+        assert rc == 0, lib.mase_hip_last_error()
+        torch.cuda.synchronize()
+        return y
+
+    y_plain = mh.mxk.mxfp_gemm(a.view(M, K), None, None, None, w_sc, w_el, preset(mh, "MXFP8_E4M3_fn"), None, M, N, K,
+                               torch.float32, split_k=False)
+    y_split = run(ws.data_ptr(), need)
+    assert rel_fro(y_split, y_plain) <= 1e-5 and not torch.equal(y_split, y_plain)
+    assert torch.equal(run(None, need), y_plain)                 # no workspace
+    assert torch.equal(run(ws.data_ptr(), need - 1), y_plain)    # one byte short
+    assert lib.mase_hip_mxfp_gemm_ws(a.data_ptr(), 2, None, None, 0, 0, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, None, 0,
+                                     y_plain.data_ptr(), 0, M, N, K, 32, ws.data_ptr() + 4, need - 4,
+                                     _lib.stream_ptr(torch.device(DEV))) == -1   # misaligned workspace
 
 
 @pytest.mark.parametrize("M", [200, 300])
