@@ -9,14 +9,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("M", [8, 200, 1024])
-def test_fused_layer_replays_from_a_graph(M):
+@pytest.mark.parametrize("M,K,N", [(8, 512, 12288), (200, 512, 12288), (1024, 512, 12288),
+                                   (200, 4096, 512)])  # the last: K split over workgroups, workspace from torch's allocator
+def test_fused_layer_replays_from_a_graph(M, K, N):
     from mase_hip import _lib
     from mase_hip.mxfp.layers import MXFPLinearPTQ
     from mase_hip.mxfp.meta import MXFP8_E4M3_fn, OCP_MXFP6_E3M2
 
     _lib.load()
-    K, N = 512, 12288
     lin = torch.nn.Linear(K, N, bias=True, dtype=torch.bfloat16, device=DEV)
     layer = MXFPLinearPTQ.from_linear(lin, MXFP8_E4M3_fn, OCP_MXFP6_E3M2, None, "XqWqB", "fused")
     g = torch.Generator(device=DEV).manual_seed(M)
