@@ -99,10 +99,10 @@ def test_random_gemm_shapes_vs_dequantize_then_matmul():
 
     rng = random.Random(3)
     g = torch.Generator().manual_seed(3)
-    for _ in range(80):
+    for _ in range(100):
         M = rng.choice([1, 5, 16, 31, 64, 100, 128, 129, 200, 256, 257, 300, 384, 500, 512, 513, 700, 1024, 1500])
         N = rng.choice([32, 64, 96, 128, 256, 384, 640, 1024, 2048, 12288])
-        K = rng.choice([32, 64, 96, 128, 192, 256, 384, 512, 1024])
+        K = rng.choice([32, 64, 96, 128, 192, 256, 384, 512, 1024, 1536, 2048, 4224])  # the longer ones get K split over workgroups
         e, m = rng.choice(PRESETS)
         odt = rng.choice([torch.bfloat16, torch.float16, torch.float32])
         x = torch.randn(M, K, generator=g).to(torch.bfloat16)
