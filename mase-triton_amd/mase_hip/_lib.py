@@ -1,6 +1,7 @@
 """ctypes binding of lib/libmase_hip.so (declarations: include/mase_hip.h at the repo root)."""
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 
@@ -90,8 +91,24 @@ def round_code(mode: str) -> int:
         raise ValueError(f"Unknown rounding mode: {mode}") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device: torch.device) -> int:
+    """hipStream_t of torch's current stream on ``device`` (the raw getter costs a fraction of building a Stream object)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
+
+
+_NO_SWITCH = contextlib.nullcontext()
+
+
+def on_device(device: torch.device):
+    """Context in which ``device`` is the current HIP device; nothing to do (and nothing paid) when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def dense(t: torch.Tensor) -> torch.Tensor:

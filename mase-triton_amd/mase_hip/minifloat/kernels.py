@@ -23,7 +23,7 @@ def extract_minifloat_component(x: Tensor, minifloat_meta: MinifloatMeta) -> Ten
     _lib.require_gpu(x, "input tensor")
     x = _lib.dense(_lib.as_float_input(x))
     codes = torch.empty(x.shape, dtype=torch.uint16, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_extract_minifloat(
             x.data_ptr(), _lib.dtype_code(x.dtype), codes.data_ptr(), x.numel(), *_fmt(minifloat_meta),
             _lib.round_code(minifloat_meta.round_mode), _lib.stream_ptr(x.device)))
@@ -36,7 +36,7 @@ def compose_minifloat_component(elements: Tensor, minifloat_meta: MinifloatMeta,
     _lib.require_gpu(elements, "elements")
     elements = _lib.dense(elements)
     out = torch.empty(elements.shape, dtype=output_dtype, device=elements.device)
-    with torch.cuda.device(elements.device):
+    with _lib.on_device(elements.device):
         _lib.check(_lib.load().mase_hip_compose_minifloat(
             elements.data_ptr(), out.data_ptr(), _lib.dtype_code(output_dtype), elements.numel(),
             *_fmt(minifloat_meta), _lib.stream_ptr(elements.device)))
@@ -48,7 +48,7 @@ def quantize_dequantize(x: Tensor, minifloat_meta: MinifloatMeta, output_dtype: 
     _lib.require_gpu(x, "input tensor")
     x = _lib.dense(_lib.as_float_input(x))
     out = torch.empty(x.shape, dtype=output_dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_qdq_minifloat(
             x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(output_dtype), x.numel(),
             *_fmt(minifloat_meta), _lib.round_code(minifloat_meta.round_mode), _lib.stream_ptr(x.device)))

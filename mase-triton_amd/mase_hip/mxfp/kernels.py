@@ -29,7 +29,7 @@ def extract_mxfp_components(x: Tensor, mxfp_meta: MXFPMeta) -> tuple[Tensor, Ten
     assert n % B == 0
     scales = torch.empty((n // B, 1), dtype=torch.uint8, device=x.device)
     elements = torch.empty((n // B, B), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_extract_mxfp(
             x.data_ptr(), _lib.dtype_code(x.dtype), scales.data_ptr(), elements.data_ptr(), n, B,
             *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
@@ -46,7 +46,7 @@ def compose_mxfp_tensor(scales: Tensor, elements: Tensor, mxfp_meta: MXFPMeta, o
     n, B = elements.numel(), mxfp_meta.block_size
     assert n % B == 0 and scales.numel() == n // B
     out = torch.empty((n,), dtype=output_dtype, device=elements.device)
-    with torch.cuda.device(elements.device):
+    with _lib.on_device(elements.device):
         _lib.check(_lib.load().mase_hip_compose_mxfp(
             scales.data_ptr(), elements.data_ptr(), out.data_ptr(), _lib.dtype_code(output_dtype), n, B,
             *_fmt(mxfp_meta), _lib.stream_ptr(elements.device)))
@@ -61,7 +61,7 @@ def quantize_dequantize(x: Tensor, mxfp_meta: MXFPMeta, output_dtype: torch.dtyp
     n, B = x.numel(), mxfp_meta.block_size
     assert n % B == 0
     out = torch.empty((n,), dtype=output_dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_qdq_mxfp(
             x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(output_dtype), n, B,
             *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
@@ -96,7 +96,7 @@ def extract_mxfp_components_strided(x: Tensor, block_dim: int, mxfp_meta: MXFPMe
     n = x.numel()
     scales = torch.empty((n // 32, 1), dtype=torch.uint8, device=x.device)
     elements = torch.empty((n // 32, 32), dtype=torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_extract_mxfp_strided(
             x.data_ptr(), _lib.dtype_code(x.dtype), scales.data_ptr(), elements.data_ptr(), outer, k_len, inner, 32,
             *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
@@ -111,11 +111,23 @@ def quantize_dequantize_strided(x: Tensor, block_dim: int, mxfp_meta: MXFPMeta, 
     x = _lib.dense(_lib.as_float_input(x))
     outer, k_len, inner = _strided_extents(x.shape, block_dim)
     out = torch.empty(x.shape, dtype=output_dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_qdq_mxfp_strided(
             x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(output_dtype), outer, k_len, inner, 32,
             *_fmt(mxfp_meta), _lib.round_code(mxfp_meta.round_mode), _lib.stream_ptr(x.device)))
     return out
+
+
+_WS_BYTES: dict[tuple, int] = {}
+
+
+def _workspace_bytes(lib, dev_index, a_is_dense: bool, M: int, N: int, K: int) -> int:
+    """The library's answer depends on the shape and the device only: ask once."""
+    key = (dev_index, a_is_dense, M, N, K)
+    n = _WS_BYTES.get(key)
+    if n is None:
+        n = _WS_BYTES[key] = lib.mase_hip_mxfp_gemm_workspace_bytes(int(a_is_dense), M, N, K)
+    return n
 
 
 def mxfp_gemm(
@@ -172,9 +184,9 @@ def mxfp_gemm(
         assert out.is_contiguous() and out.dtype == output_dtype and out.numel() == M * N and out.device == dev
         y = out
     lib = _lib.load()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         # few output tiles and a long K: the library splits K over more workgroups if it is given room for the partial sums
-        ws_bytes = lib.mase_hip_mxfp_gemm_workspace_bytes(int(a is not None), M, N, K) if split_k else 0
+        ws_bytes = _workspace_bytes(lib, dev.index, a is not None, M, N, K) if split_k else 0
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
         _lib.check(lib.mase_hip_mxfp_gemm_ws(
             a_ptr, a_dt, a_sc_ptr, a_el_ptr, a_e, a_m, w_scales.data_ptr(), w_elements.data_ptr(),

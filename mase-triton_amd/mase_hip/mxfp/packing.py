@@ -38,7 +38,7 @@ def pack_elements(elements: Tensor, mxfp_meta: MXFPMeta) -> Tensor:
     n = flat.numel()
     assert n % 16 == 0, "element count must be a multiple of 16"
     packed = torch.empty(n * bits // 8, dtype=torch.uint8, device=flat.device)
-    with torch.cuda.device(flat.device):
+    with _lib.on_device(flat.device):
         _lib.check(_lib.load().mase_hip_pack_codes(flat.data_ptr(), packed.data_ptr(), n, bits, _lib.stream_ptr(flat.device)))
     return packed
 
@@ -55,7 +55,7 @@ def unpack_elements(packed: Tensor, mxfp_meta: MXFPMeta, n_elements: int) -> Ten
     packed = _lib.dense(packed)
     assert n_elements % 16 == 0
     elements = torch.empty(n_elements, dtype=torch.uint8, device=packed.device)
-    with torch.cuda.device(packed.device):
+    with _lib.on_device(packed.device):
         _lib.check(_lib.load().mase_hip_unpack_codes(packed.data_ptr(), elements.data_ptr(), n_elements, bits,
                                                      _lib.stream_ptr(packed.device)))
     return elements.view(n_elements // B, B)
