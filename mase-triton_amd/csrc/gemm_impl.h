@@ -527,7 +527,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
     if constexpr (A_MODE == 0) {
         // few tiles and a long K: with a workspace, K is split over several workgroups per tile
-        if (workspace && fits32 && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
+        if (workspace && K <= (1 << 23) && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
             const SplitPlan plan = plan_split_k(M, N, K, device_cu_count());
             if (plan.splits > 1 && workspace_bytes >= plan.workspace_bytes(M, N))
                 return launch_gemm_mid_split_k<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, plan, workspace, s);
@@ -556,10 +556,13 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         // (rounds of one tile per CU) x (time of one tile, relative, measured at K = 4096: 48 / 67 / 98 us for
         // 128 x 128 / 256 x 128 / 512 x 128); ties go to the larger tile.
         const bool al = (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0;
-        const bool mid_ok = fits32 && al && M > 128 && N % MD_N == 0 && K % MD_MAC == 0;
-        const bool wide_ok = fits32 && al && M > 128 && N % WD_N == 0 && K % WD_K == 0;
-        const bool tall_ok = fits32 && al && M >= UM && N % UN == 0 && K % UMAC == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
-                             (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0;
+        // (these kernels address with a 64-bit base per tile and 32-bit offsets within the tile's rows: operands of any
+        // size, as long as 256 rows of A, or a few rows of y, stay below 4 GiB)
+        const bool reach = K <= (1 << 23) && N <= (1 << 26);
+        const bool mid_ok = reach && al && M > 128 && N % MD_N == 0 && K % MD_MAC == 0;
+        const bool wide_ok = reach && al && M > 128 && N % WD_N == 0 && K % WD_K == 0;
+        const bool tall_ok = reach && al && M >= UM && N % UN == 0 && K % UMAC == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
+                             (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0 && (int64_t)((M + UM - 1) / UM) * (N / UN) < (1 << 30);
         if (mid_ok || wide_ok || tall_ok) {
             const int cus = device_cu_count();
             if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");

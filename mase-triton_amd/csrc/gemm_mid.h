@@ -53,7 +53,8 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
     // and writes its sums to its own [M, N] array, y_split_bytes apart.  One split: k_len = K.
     const int k_begin = (int)blockIdx.y * k_len;
     const int kblocks = K / 32, nmac = min(k_len, K - k_begin) / MD_MAC;
-    a_dense += k_begin;
+    // 64-bit base of the tile's first row (and the split's first k): the per-lane offsets below stay within the tile's rows
+    const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)m0 * K + k_begin) * 2;
     void* const y = static_cast<uint8_t*>(y_all) + (size_t)blockIdx.y * (size_t)y_split_bytes;
 
     // A DMA: an instruction moves 1 KB = 4 rows; lane l fills position l % 16 of row 4 (8 w + j) + l / 16, which must
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
 #pragma unroll
     for (int j = 0; j < A_DMAS; ++j) {
         const int row = (wave * A_DMAS + j) * 4 + (lane >> 4);
-        a_voff[j] = (uint32_t)min(m0 + row, M - 1) * (uint32_t)K * 2u + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
+        a_voff[j] = (uint32_t)(min(m0 + row, M - 1) - m0) * (uint32_t)K * 2u + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
     }
     // W: the wavefront loads 8 W_LOADS rows as whole lines: lane = 16 codes (16 k) of its row 8 h + (l >> 3)
     const int w_chunk = lane & 7;
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
     // do not expect)
     auto issue_a = [&](int mac, auto stage_c) __attribute__((always_inline)) {
         constexpr int stage = decltype(stage_c)::value;
-        const uint8_t* const a_src = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)k_of(mac) * (MD_MAC * 2);
+        const uint8_t* const a_src = a_tile + (size_t)k_of(mac) * (MD_MAC * 2);
         const uint32_t dst = lds_a_addr + (uint32_t)stage * MD_A_STAGE + (uint32_t)wave * (A_DMAS * 1024);
         static_for<A_DMAS>([&](auto j_c) __attribute__((always_inline)) {
             constexpr int j = decltype(j_c)::value;
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
                 // instructions issue in order, so work placed behind a run of MFMAs would wait for the whole run
                 constexpr int ns = r % 3, cs = (r + 1) % 3, a_stage = (r + 2) % 3, w_stage = (r + 1) % 2;
                 const int mc_a = k_of(mac + 2), mc_w = k_of(mac + 3);
-                const uint8_t* const a_src = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)mc_a * (MD_MAC * 2);
+                const uint8_t* const a_src = a_tile + (size_t)mc_a * (MD_MAC * 2);
                 const uint32_t a_dst = lds_a_addr + (uint32_t)a_stage * MD_A_STAGE + (uint32_t)wave * (A_DMAS * 1024);
                 const uint8_t* const w_src = w_base + (size_t)mc_w * MD_MAC;
                 const uint8_t* const ws_src = ws_base + mc_w * (MD_MAC / 32);

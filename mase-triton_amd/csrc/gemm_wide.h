@@ -39,6 +39,8 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     const int tile_m = (int)(blockIdx.x % (unsigned)tiles_m), tile_n = (int)(blockIdx.x / (unsigned)tiles_m);
     const int m0 = tile_m * WD_M, n0 = tile_n * WD_N;
     const int kblocks = K / 32, nsteps = K / WD_K;
+    // 64-bit base of the tile's first row: the per-lane offsets below stay within the tile's rows
+    const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)m0 * K * 2;
 
     // A DMA: an instruction moves 1 KB = 8 rows; lane l fills position l & 7 of row 8 (4 w + j) + (l >> 3), which must
     // hold chunk (l & 7) ^ ((row >> 1) & 7).  Rows past M re-read row M - 1 (their products are never stored).
@@ -46,7 +48,7 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
 #pragma unroll
     for (int j = 0; j < A_DMAS; ++j) {
         const int row = (wave * A_DMAS + j) * 8 + (lane >> 3);
-        a_voff[j] = (uint32_t)min(m0 + row, M - 1) * (uint32_t)K * 2u + (uint32_t)(((lane & 7) ^ ((row >> 1) & 7)) * 16);
+        a_voff[j] = (uint32_t)(min(m0 + row, M - 1) - m0) * (uint32_t)K * 2u + (uint32_t)(((lane & 7) ^ ((row >> 1) & 7)) * 16);
     }
     // W: thread t loads the 16 codes at k 16 (t & 3) .. + 15 of row t >> 2
     const int w_row = tid >> 2, w_piece = tid & 3;
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     // do not expect)
     auto issue_a = [&](int s, auto stage_c) __attribute__((always_inline)) {
         constexpr int stage = decltype(stage_c)::value;
-        const uint8_t* const a_src = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)k_of(s) * (WD_K * 2);
+        const uint8_t* const a_src = a_tile + (size_t)k_of(s) * (WD_K * 2);
         const uint32_t dst = lds_a_addr + (uint32_t)stage * WD_A_STAGE + (uint32_t)wave * (A_DMAS * 1024);
         static_for<A_DMAS>([&](auto j_c) __attribute__((always_inline)) {
             constexpr int j = decltype(j_c)::value;
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
                 // this step's loads (A(s + 2) into the stage read last step, W(s + 3) into the ring slot composed last
                 // step) and the compose of W(s + 1) are spread over the step's 16 MFMAs: instructions issue in order, so
                 // work placed behind a run of MFMAs would wait for the whole run
-                const uint8_t* const a_src = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)k_of(s + 2) * (WD_K * 2);
+                const uint8_t* const a_src = a_tile + (size_t)k_of(s + 2) * (WD_K * 2);
                 const uint32_t a_dst = lds_a_addr + (uint32_t)a_stage * WD_A_STAGE + (uint32_t)wave * (A_DMAS * 1024);
                 const int kw = k_of(s + 3);
                 const uint8_t* const w_src = w_base + (size_t)kw * WD_K;
