@@ -35,8 +35,11 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave >> 1, wave_n = wave & 1;
-    // m-tile fastest: the workgroups that share 128 rows of W run next to each other in time
-    const int tile_m = (int)(blockIdx.x % (unsigned)tiles_m), tile_n = (int)(blockIdx.x / (unsigned)tiles_m);
+    // m-tile fastest: the workgroups that share 128 rows of W run next to each other in time, and, workgroups being dealt
+    // to the 8 XCDs in turn, on the same XCD (one L2): XCD x takes the x-th eighth of the tiles
+    const unsigned n_wg = gridDim.x, per_xcd = n_wg >> 3;
+    const unsigned tile = (n_wg & 7u) == 0 ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
+    const int tile_m = (int)(tile % (unsigned)tiles_m), tile_n = (int)(tile / (unsigned)tiles_m);
     const int m0 = tile_m * WD_M, n0 = tile_n * WD_N;
     const int kblocks = K / 32, nsteps = K / WD_K;
     // 64-bit base of the tile's first row: the per-lane offsets below stay within the tile's rows
