@@ -312,7 +312,7 @@ inline SplitPlan plan_split_k(int M, int N, int K, int cus) {
     int most = (int)(cus / tiles);
     if (most > nmac / 4) most = nmac / 4;                          // at least four macro steps per split
     if (most > 16) most = 16;
-    // Splitting pays when the macro steps a workgroup no longer walks (0.7 us each or more, measured) outweigh the second
+    // Splitting pays when the macro steps a workgroup no longer walks (0.8 us each or more, measured) outweigh the second
     // launch (4 us) and the traffic of the partial sums (written and read once per split, at 4.7 TB/s measured):
     // K = 1024 in two splits of a [512, 4096] output was 24 us against 16 us unsplit.
     const double mn_mb = (double)M * N * 4.0 / 1e6;
@@ -320,7 +320,7 @@ inline SplitPlan plan_split_k(int M, int N, int K, int cus) {
     for (int want = 2; want <= most; ++want) {
         const int mac_per = (nmac + want - 1) / want;
         const int splits = (nmac + mac_per - 1) / mac_per;         // no empty split
-        const double gain = (nmac - mac_per) * 0.7 - (4.0 + (2.0 * splits + 0.5) * mn_mb * 0.21);
+        const double gain = (nmac - mac_per) * 0.8 - (4.0 + (2.0 * splits + 0.5) * mn_mb * 0.21);
         if (gain > best) {
             best = gain;
             p.splits = splits;
