@@ -415,6 +415,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 #include "gemm_rows16.h"
 #include "gemm_mid.h"
 #include "gemm_wide.h"
+#include "gemm_split_k.h"
 
 // ---------------------------------------------------------------------------------------------
 // Small-shape kernel: 128 x 128 x 32 tiles, single LDS buffer.  Used when the problem cannot
@@ -530,7 +531,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         if (workspace && K <= (1 << 23) && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
             const SplitPlan plan = plan_split_k(M, N, K, device_cu_count());
             if (plan.splits > 1 && workspace_bytes >= plan.workspace_bytes(M, N))
-                return launch_gemm_mid_split_k<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, plan, workspace, s);
+                return launch_gemm_split_k<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, plan, workspace, s);
         }
     }
     if constexpr (A_MODE == 0) {

@@ -289,81 +289,3 @@ int launch_gemm_mid(const void* a_dense, const uint8_t* w_scales, const uint8_t*
                        w_elements, bias, bias_dtype, y, M, N, K, tiles_m, K, (int64_t)0);
     return check_launch("mxfp_gemm");
 }
-
-// ---------------------------------------------------------------------------------------------
-// K split over several workgroups per tile, for products with few tiles and a long K (a [256, 4096] output has 64 tiles
-// for 256 CUs): split z multiplies its share of K into the fp32 array partial[z][M][N] of a caller-provided workspace,
-// and a second kernel adds the arrays, the bias, and rounds to the output type.
-
-struct SplitPlan {
-    int splits;  // 1: do not split
-    int k_len;   // k per split, a multiple of the macro step
-    int64_t workspace_bytes(int M, int N) const { return splits > 1 ? (int64_t)splits * M * N * 4 : 0; }
-};
-
-// The same plan for the size query and the launch: it depends on the shape and the CU count only.
-inline SplitPlan plan_split_k(int M, int N, int K, int cus) {
-    SplitPlan p{1, K};
-    // up to 64 rows the weight-streaming kernels are as fast or faster (64 x 4096 x 4096: 14.5 us against 20.4 us split)
-    if (M <= 64 || N % MD_N != 0 || K % MD_MAC != 0 || cus <= 0) return p;
-    const int64_t tiles = (int64_t)((M + MD_M - 1) / MD_M) * (N / MD_N);
-    const int nmac = K / MD_MAC;
-    if (tiles * 2 > cus) return p;                                 // a second workgroup per tile would not find a free CU
-    int most = (int)(cus / tiles);
-    if (most > nmac / 4) most = nmac / 4;                          // at least four macro steps per split
-    if (most > 16) most = 16;
-    // Splitting pays when the macro steps a workgroup no longer walks (0.8 us each or more, measured) outweigh the second
-    // launch (4 us) and the traffic of the partial sums (written and read once per split, at 4.7 TB/s measured):
-    // K = 1024 in two splits of a [512, 4096] output was 24 us against 16 us unsplit.
-    const double mn_mb = (double)M * N * 4.0 / 1e6;
-    double best = 0.0;
-    for (int want = 2; want <= most; ++want) {
-        const int mac_per = (nmac + want - 1) / want;
-        const int splits = (nmac + mac_per - 1) / mac_per;         // no empty split
-        const double gain = (nmac - mac_per) * 0.8 - (4.0 + (2.0 * splits + 0.5) * mn_mb * 0.21);
-        if (gain > best) {
-            best = gain;
-            p.splits = splits;
-            p.k_len = mac_per * MD_MAC;
-        }
-    }
-    return p;
-}
-
-template <int DT_OUT>
-__global__ __launch_bounds__(256) void split_k_reduce_kernel(const float* __restrict__ partial, int splits, int64_t mn, int N,
-                                                             const void* __restrict__ bias, int bias_dtype, void* __restrict__ y) {
-    // a lane adds four consecutive outputs of every split (N % 4 == 0: they share a row)
-    const int64_t o = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (o >= mn) return;
-    float4 acc = *reinterpret_cast<const float4*>(partial + o);
-    for (int z = 1; z < splits; ++z) {
-        const float4 v = *reinterpret_cast<const float4*>(partial + (size_t)z * mn + o);
-        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
-    }
-    float r[4] = {acc.x, acc.y, acc.z, acc.w};
-    if (bias) {
-        const int n = (int)(o % N);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) r[t] += load_bias(bias, bias_dtype, n + t);
-    }
-    store_out4<DT_OUT>(y, o, r, (reinterpret_cast<uintptr_t>(y) & 15) == 0, 4);
-}
-
-template <class FW, int DT_OUT>
-int launch_gemm_mid_split_k(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
-                            void* y, int M, int N, int K, const SplitPlan& plan, void* workspace, hipStream_t s) {
-    auto kern = mxfp_gemm_mid_kernel<FW, F32, 2>;
-    static std::atomic<uint64_t> lds_allowed{0};
-    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), MD_LDS_BYTES, lds_allowed)) return rc;
-    const int tiles_m = (M + MD_M - 1) / MD_M;
-    const int64_t tiles = (int64_t)tiles_m * (N / MD_N);
-    const int64_t mn = (int64_t)M * N;
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)plan.splits), dim3(512), MD_LDS_BYTES, s,
-                       static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace, M, N, K,
-                       tiles_m, plan.k_len, mn * 4);
-    if (int rc = check_launch("mxfp_gemm")) return rc;
-    hipLaunchKernelGGL(split_k_reduce_kernel<DT_OUT>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s,
-                       static_cast<const float*>(workspace), plan.splits, mn, N, bias, bias_dtype, y);
-    return check_launch("mxfp_gemm");
-}

@@ -24,7 +24,7 @@ constexpr int WD_THREADS = 512;
 template <class FW, int DT_OUT>
 __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m) {
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y_all, int M, int N, int K, int tiles_m, int k_len, int64_t y_split_bytes) {
     constexpr int A_DMAS = WD_A_STAGE / 1024 / 8;          // 4 per wavefront and step
     constexpr int OPS = A_DMAS + 2;                        // vector-memory operations per wavefront and step
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -41,9 +41,13 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     const unsigned tile = (n_wg & 7u) == 0 ? (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3) : blockIdx.x;
     const int tile_m = (int)(tile % (unsigned)tiles_m), tile_n = (int)(tile / (unsigned)tiles_m);
     const int m0 = tile_m * WD_M, n0 = tile_n * WD_N;
-    const int kblocks = K / 32, nsteps = K / WD_K;
-    // 64-bit base of the tile's first row: the per-lane offsets below stay within the tile's rows
-    const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(a_dense) + (size_t)m0 * K * 2;
+    // blockIdx.y = split of K: this workgroup multiplies k in [k_begin, k_begin + k_len) (the last split may be shorter)
+    // and writes its sums to its own [M, N] array, y_split_bytes apart.  One split: k_len = K.
+    const int k_begin = (int)blockIdx.y * k_len;
+    const int kblocks = K / 32, nsteps = min(k_len, K - k_begin) / WD_K;
+    void* const y = static_cast<uint8_t*>(y_all) + (size_t)blockIdx.y * (size_t)y_split_bytes;
+    // 64-bit base of the tile's first row (and the split's first k): the per-lane offsets below stay within the tile's rows
+    const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)m0 * K + k_begin) * 2;
 
     // A DMA: an instruction moves 1 KB = 8 rows; lane l fills position l & 7 of row 8 (4 w + j) + (l >> 3), which must
     // hold chunk (l & 7) ^ ((row >> 1) & 7).  Rows past M re-read row M - 1 (their products are never stored).
@@ -55,8 +59,8 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     }
     // W: thread t loads the 16 codes at k 16 (t & 3) .. + 15 of row t >> 2
     const int w_row = tid >> 2, w_piece = tid & 3;
-    const uint8_t* const w_base = w_elements + (size_t)n0 * K;
-    const uint8_t* const ws_base = w_scales + (size_t)n0 * kblocks;
+    const uint8_t* const w_base = w_elements + (size_t)n0 * K + k_begin;
+    const uint8_t* const ws_base = w_scales + (size_t)n0 * kblocks + k_begin / 32;
     const uint32_t w_voff = (uint32_t)w_row * (uint32_t)K + (uint32_t)w_piece * 16u;
     const uint32_t ws_voff = (uint32_t)w_row * (uint32_t)kblocks + (uint32_t)(w_piece >> 1);
     uint32_t w_lds_off[2];
@@ -79,7 +83,7 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     uint32_t w_scale[3];
     // workgroups start at different steps of K (and wrap around), so that at any moment they read different columns
     // of W and A: addresses that spread over the memory channels
-    const int rot = (int)((unsigned)tile_n % (unsigned)nsteps);
+    const int rot = (int)((unsigned)(tile_n + blockIdx.y) % (unsigned)nsteps);
     // past the end the last step is read again (unused), which keeps the operation count per step, and with it the
     // wait counts, the same
     auto k_of = [&](int s) __attribute__((always_inline)) {
@@ -224,6 +228,6 @@ int launch_gemm_wide(const void* a_dense, const uint8_t* w_scales, const uint8_t
     const int64_t tiles = (int64_t)tiles_m * (N / WD_N);
     if (tiles > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "too many tiles for one launch");
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(WD_THREADS), WD_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                       w_elements, bias, bias_dtype, y, M, N, K, tiles_m);
+                       w_elements, bias, bias_dtype, y, M, N, K, tiles_m, K, (int64_t)0);
     return check_launch("mxfp_gemm");
 }

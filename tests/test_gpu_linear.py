@@ -369,6 +369,44 @@ def test_gemm_split_k(mh, MNK, splits, w_tag, odt, with_bias):
         assert torch.equal(y, y_plain)
 
 
+@pytest.mark.parametrize("MNK,odt,with_bias", [
+    ((300, 4096, 12288), torch.bfloat16, True),    # 2 x 32 tiles of 256 x 128, the second tile row mostly past M; 4 splits of 24
+    ((384, 4096, 12416), torch.float32, False),    # 97 macro steps as 25 + 25 + 25 + 22
+])
+def test_gemm_split_k_wide_tiles(mh, MNK, odt, with_bias):
+    """Long K and an output too large for more than two splits of its 128 x 128 tiles: the split runs on 256 x 128 tiles
+    (here four splits; 96 tiles of 128 x 128 would allow two).  The whole output against an fp32 dequantize-then-matmul
+    on the GPU, a sample of it against float64 accumulation, and the unsplit call."""
+    from mase_hip import _lib
+
+    M, N, K = MNK
+    assert _lib.load().mase_hip_mxfp_gemm_workspace_bytes(1, M, N, K) == 4 * M * N * 4
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16) if with_bias else None
+    x_dq = oracle.qdq_mxfp(x, 32, 4, 3)
+    w_sc, w_el = oracle.extract_mxfp(w, 32, 4, 3)
+    w_dq = oracle.compose_mxfp(w_sc, w_el, 32, 4, 3, True, torch.bfloat16).view(N, K)
+    args = (x_dq.to(DEV), None, None, None, w_sc.to(DEV), w_el.to(DEV), preset(mh, "MXFP8_E4M3_fn"), None if b is None else b.to(DEV),
+            M, N, K, odt)
+    y = mh.mxk.mxfp_gemm(*args)
+    tol = 1e-5 if odt == torch.float32 else REL_FRO_TOL
+    y_gpu = x_dq.to(DEV).float() @ w_dq.to(DEV).float().T
+    if b is not None:
+        y_gpu = y_gpu + b.to(DEV).float()
+    assert rel_fro(y, y_gpu.to(odt)) <= tol
+    rows, cols = torch.arange(0, M, 7), torch.arange(0, N, 53)
+    y_ref = oracle.matmul_nt(x_dq[rows], w_dq[cols])
+    if b is not None:
+        y_ref = y_ref + b[cols].float()
+    assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref.to(odt)) <= tol
+    y_plain = mh.mxk.mxfp_gemm(*args, split_k=False)
+    assert rel_fro(y, y_plain) <= tol
+    if odt == torch.float32:
+        assert not torch.equal(y, y_plain)
+
+
 def test_gemm_split_k_special_values(mh):
     M, N, K = 200, 256, 2048
     g = torch.Generator().manual_seed(21)
