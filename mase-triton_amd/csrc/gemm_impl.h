@@ -529,7 +529,8 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     if constexpr (A_MODE == 0) {
         // few tiles and a long K: with a workspace, K is split over several workgroups per tile
         if (workspace && K <= (1 << 23) && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
-            const SplitPlan plan = plan_split_k(M, N, K, device_cu_count());
+            // (the 512 x 128 kernel reads four scale bytes at a time)
+            const SplitPlan plan = plan_split_k(M, N, K, device_cu_count(), (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0);
             if (plan.splits > 1 && workspace_bytes >= plan.workspace_bytes(M, N))
                 return launch_gemm_split_k<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, plan, workspace, s);
         }
@@ -587,7 +588,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             // one persistent workgroup per CU (a multiple of the 8 XCDs), never more than tiles
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
             hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                               w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN);
+                               w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN, 1, (int64_t)0);
             return check_launch("mxfp_gemm");
         }
     }

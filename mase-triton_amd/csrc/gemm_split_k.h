@@ -1,13 +1,13 @@
 // K split over several workgroups per tile, for products with few tiles and a long K (a [256, 4096] output has 64 tiles
 // of 128 x 128 for 256 CUs): split z multiplies its share of K into the fp32 array partial[z][M][N] of a caller-provided
-// workspace, on the 128 x 128 or the 256 x 128 tile kernel, and a second kernel adds the arrays, the bias, and rounds to
+// workspace, on the 128 x 128, 256 x 128 or 512 x 128 tile kernel, and a second kernel adds the arrays, the bias, and rounds to
 // the output type.
 // (included from gemm_impl.h, inside namespace mase, after gemm_mid.h and gemm_wide.h)
 
 struct SplitPlan {
     int splits;  // 1: do not split
     int k_len;   // k per split, a multiple of 128
-    int kind;    // 0: 128 x 128 tiles, 1: 256 x 128 tiles
+    int kind;    // 0: 128 x 128 tiles, 1: 256 x 128 tiles, 2: 512 x 128 tiles
     int64_t workspace_bytes(int M, int N) const { return splits > 1 ? (int64_t)splits * M * N * 4 : 0; }
 };
 
@@ -25,7 +25,7 @@ inline double split_step_us(int64_t wgs, int cus) {
 // 512-row tiles), plus, when split, 4 us for the second launch and the partial sums written and read once at 4.7 TB/s
 // (K = 1024 in two splits of a [512, 4096] output was 24 us against 16 us unsplit); the cheapest wins, and if that is
 // an unsplit one the plan says so.
-inline SplitPlan plan_split_k(int M, int N, int K, int cus) {
+inline SplitPlan plan_split_k(int M, int N, int K, int cus, bool allow_tall = true) {
     SplitPlan p{1, K, 0};
     // up to 64 rows the weight-streaming kernels are as fast or faster (64 x 4096 x 4096: 14.5 us against 20.4 us split)
     if (M <= 64 || N % 128 != 0 || K % 128 != 0 || cus <= 0) return p;
@@ -40,21 +40,25 @@ inline SplitPlan plan_split_k(int M, int N, int K, int cus) {
     double best = price(128, 1.0, nmac, 1);
     if (M > 128) best = std::min(best, price(256, 1.4, nmac, 1));
     if (M >= 512) best = std::min(best, price(512, 2.05, nmac, 1));
-    for (int kind = 0; kind < 2; ++kind) {
-        if (kind == 1 && M <= 256) break;                          // a 256-row tile would be mostly empty rows
-        const int rows = kind == 0 ? 128 : 256;
+    for (int kind = 0; kind < 3; ++kind) {
+        if (kind == 1 && M <= 256) continue;                       // a 256-row tile would be mostly empty rows
+        if (kind == 2 && (M < 512 || !allow_tall)) continue;
+        const int rows = 128 << kind;
+        const double rel = kind == 0 ? 1.0 : kind == 1 ? 1.4 : 2.05;
         const int64_t tiles = (int64_t)((M + rows - 1) / rows) * n128;
         if (tiles * 2 > cus) continue;                             // a second workgroup per tile would not find a free CU
         int most = (int)(cus / tiles);
-        // macro steps per split at least: 4, and 24 on the 256 x 128 tiles, whose longer prologue and larger fp32 tile only
-        // pay over a long run (512 x 4096 x 4096: 38 us in four splits of 8 against 34 us on 128 x 128 tiles in two of 16)
+        // macro steps per split at least: 4, and 24 on the larger tiles, whose longer prologue and larger fp32 tile only pay
+        // over a long run (512 x 4096 x 4096: 38 us on 256 x 128 tiles in four splits of 8 against 34 us on 128 x 128 tiles
+        // in two of 16)
         const int least = kind == 0 ? 4 : 24;
         if (most > nmac / least) most = nmac / least;
         if (most > 16) most = 16;
         for (int want = 2; want <= most; ++want) {
+            if (kind == 2 && nmac % want != 0) continue;           // the 512 x 128 kernel walks equal shares only
             const int mac_per = (nmac + want - 1) / want;
             const int splits = (nmac + mac_per - 1) / mac_per;     // no empty split
-            const double t = price(rows, kind == 0 ? 1.0 : 1.4, mac_per, splits);
+            const double t = price(rows, rel, mac_per, splits);
             if (t < best) {
                 best = t;
                 p.splits = splits;
@@ -98,7 +102,7 @@ int launch_gemm_split_k(const void* a_dense, const uint8_t* w_scales, const uint
         hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * (N / MD_N)), (unsigned)plan.splits), dim3(512), MD_LDS_BYTES, s,
                            static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
                            M, N, K, tiles_m, plan.k_len, mn * 4);
-    } else {
+    } else if (plan.kind == 1) {
         auto kern = mxfp_gemm_wide_kernel<FW, F32>;
         static std::atomic<uint64_t> lds_allowed{0};
         if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), WD_LDS_BYTES, lds_allowed)) return rc;
@@ -106,6 +110,15 @@ int launch_gemm_split_k(const void* a_dense, const uint8_t* w_scales, const uint
         hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * (N / WD_N)), (unsigned)plan.splits), dim3(WD_THREADS), WD_LDS_BYTES, s,
                            static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
                            M, N, K, tiles_m, plan.k_len, mn * 4);
+    } else {
+        auto kern = mxfp_gemm_tall_kernel<FW, F32>;
+        static std::atomic<uint64_t> lds_allowed{0};
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed)) return rc;
+        const int tiles_m = (M + UM - 1) / UM;
+        const int walks = tiles_m * (N / UN) * plan.splits;          // at most one per CU (the plan splits only then)
+        hipLaunchKernelGGL(kern, dim3((unsigned)((walks + 7) / 8 * 8)), dim3(kGemmThreads), U_LDS_BYTES, s,
+                           static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
+                           M, N, K, tiles_m, N / UN, plan.splits, mn * 4);
     }
     if (int rc = check_launch("mxfp_gemm")) return rc;
     hipLaunchKernelGGL(split_k_reduce_kernel<DT_OUT>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s,

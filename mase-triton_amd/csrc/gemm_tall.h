@@ -112,17 +112,20 @@ struct TallTile {
     const uint8_t* a;   // this wave's first A row
     const uint8_t* w;   // first W row (codes)
     const uint8_t* ws;  // first W row (scales)
+    size_t y_off;       // byte offset of this tile's output array (K split: one [M, N] array per split)
     int m0, n0;
 };
 
 template <class FW, int DT_OUT>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_tall_kernel(
     const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, int splits, int64_t y_split_bytes) {
+    // splits > 1: every tile is walked `splits` times, each time over K / splits of k and into its own [M, N] output array
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kblocks = K / 32, nmac = K / UMAC;  // the launcher guarantees K % 128 == 0
+    const int k_len = K / splits;                 // the launcher guarantees K % (128 splits) == 0
+    const int kblocks = K / 32, nmac = k_len / UMAC;
     const uint32_t lds_aw = (uint32_t)(uintptr_t)lds + (uint32_t)wave * U_A_WAVE_BYTES;  // this wave's rows of stage 0
     uint8_t* const lds_a_ptr = lds + wave * U_A_WAVE_BYTES;
     uint8_t* const lds_w_ptr = lds + U_A_STAGES * U_A_STAGE_BYTES;
@@ -156,12 +159,13 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
             w_lds_off[pp][e] = (uint32_t)w_row * 128u + (uint32_t)(((4 * pp + 2 * w_half + e) ^ ((w_row >> 1) & 7)) * 16);
     // W fragment reads use the same offsets as A's (same row length and swizzle)
 
-    const int n_tiles = tiles_m * tiles_n;
+    const int n_tiles = tiles_m * tiles_n * splits;
     const int per_xcd = (n_tiles + 7) >> 3;
     const int slots = gridDim.x >> 3;
     auto has_tile = [&](int local) { return local < per_xcd && (int)(blockIdx.x & 7) * per_xcd + local < n_tiles; };
     auto tile_at = [&](int local) {
-        const int pos = (blockIdx.x & 7) * per_xcd + local;
+        const int walk = (blockIdx.x & 7) * per_xcd + local;
+        const int pos = walk / splits, z = walk - pos * splits;      // the splits of a tile run next to each other
         // groups of 2 tile-rows, rows fastest: the 32 tiles an XCD runs at once form a 2 x 16 patch
         constexpr int GROUP = 2;
         const int in_group = GROUP * tiles_n;
@@ -173,9 +177,11 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         // its neighbour are computed twice, identically
         t.m0 = min((first_m + rr % rows) * UM, M - UM);
         t.n0 = (rr / rows) * UN;
-        t.a = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)(t.m0 + wave * 128) * K) * 2;
-        t.w = w_elements + (size_t)t.n0 * K;
-        t.ws = w_scales + (size_t)t.n0 * kblocks;
+        const size_t k0 = (size_t)z * k_len;
+        t.a = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)(t.m0 + wave * 128) * K + k0) * 2;
+        t.w = w_elements + (size_t)t.n0 * K + k0;
+        t.ws = w_scales + (size_t)t.n0 * kblocks + k0 / 32;
+        t.y_off = (size_t)z * (size_t)y_split_bytes;
         return t;
     };
 
@@ -438,7 +444,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         //      m = m0 + wave*128 + i*32 + lane%32,  n = n0 + j*32 + 8*g + 4*(lane/32).
         //      Staged through LDS in 8 passes of 32 rows x 64 columns so that every store instruction
         //      writes 8 whole 128-byte lines.
-        uint8_t* const y_wave = static_cast<uint8_t*>(y) + ((size_t)(cur.m0 + wave * 128) * N + cur.n0) * 2;
+        uint8_t* const y_wave = static_cast<uint8_t*>(y) + cur.y_off + ((size_t)(cur.m0 + wave * 128) * N + cur.n0) * 2;
         // output staging (per wave, 32 rows of 128 bytes, 16-byte chunk c of row r at position c ^ (r & 7)):
         // a lane writes 8 bytes of row l & 31 and reads 16 bytes of row 8 t + (l >> 3).  The lane number goes
         // through an asm so that these addresses are recomputed here instead of living in registers
@@ -459,7 +465,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
             if constexpr (DT_OUT == F32) {
                 // fp32 output: 16 passes of 32 rows x 32 columns (128 bytes per row again); a lane writes the 16 bytes of
                 // its four consecutive columns as chunk 2 g + (l >> 5) of row l & 31
-                uint8_t* const y_wave32 = static_cast<uint8_t*>(y) + ((size_t)(cur.m0 + wave * 128) * N + cur.n0) * 4;
+                uint8_t* const y_wave32 = static_cast<uint8_t*>(y) + cur.y_off + ((size_t)(cur.m0 + wave * 128) * N + cur.n0) * 4;
                 const uint32_t o_st_voff32 = ((ol >> 3) * (uint32_t)N + (ol & 7u) * 4u) * 4u;
                 static_for<4>([&](auto i_c) {
                     static_for<4>([&](auto j_c) {

@@ -372,11 +372,13 @@ def test_gemm_split_k(mh, MNK, splits, w_tag, odt, with_bias):
 @pytest.mark.parametrize("MNK,odt,with_bias", [
     ((300, 4096, 12288), torch.bfloat16, True),    # 2 x 32 tiles of 256 x 128, the second tile row mostly past M; 4 splits of 24
     ((384, 4096, 12416), torch.float32, False),    # 97 macro steps as 25 + 25 + 25 + 22
+    ((1000, 4096, 12288), torch.bfloat16, True),   # 2 x 32 tiles of 512 x 128, the second shifted up to end at row M - 1; 4 splits
+    ((1024, 4096, 12288), torch.float32, False),   # the same tiles, fp32 output
 ])
-def test_gemm_split_k_wide_tiles(mh, MNK, odt, with_bias):
-    """Long K and an output too large for more than two splits of its 128 x 128 tiles: the split runs on 256 x 128 tiles
-    (here four splits; 96 tiles of 128 x 128 would allow two).  The whole output against an fp32 dequantize-then-matmul
-    on the GPU, a sample of it against float64 accumulation, and the unsplit call."""
+def test_gemm_split_k_larger_tiles(mh, MNK, odt, with_bias):
+    """Long K and an output too large for more than two splits of its 128 x 128 tiles: the split runs on 256 x 128 or
+    512 x 128 tiles (here four splits each; the smaller tiles would allow two, or none).  The whole output against an fp32
+    dequantize-then-matmul on the GPU, a sample of it against float64 accumulation, and the unsplit call."""
     from mase_hip import _lib
 
     M, N, K = MNK
