@@ -582,9 +582,10 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             if (pick == 1) return launch_gemm_wide<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
             const int tall_tiles_m = (M + UM - 1) / UM;
             const int64_t tall_tiles = (int64_t)tall_tiles_m * (N / UN);
-            auto kern = mxfp_gemm_tall_kernel<FW, DT_OUT>;
-            static std::atomic<uint64_t> lds_allowed{0};
-            if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed)) return rc;
+            const bool sc4 = K % 512 == 0;
+            auto kern = sc4 ? mxfp_gemm_tall_kernel<FW, DT_OUT, true> : mxfp_gemm_tall_kernel<FW, DT_OUT, false>;
+            static std::atomic<uint64_t> lds_allowed[2] = {{0}, {0}};
+            if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed[sc4])) return rc;
             // one persistent workgroup per CU (a multiple of the 8 XCDs), never more than tiles
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
             hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,

@@ -111,9 +111,10 @@ int launch_gemm_split_k(const void* a_dense, const uint8_t* w_scales, const uint
                            static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
                            M, N, K, tiles_m, plan.k_len, mn * 4);
     } else {
-        auto kern = mxfp_gemm_tall_kernel<FW, F32>;
-        static std::atomic<uint64_t> lds_allowed{0};
-        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed)) return rc;
+        const bool sc4 = plan.k_len % 512 == 0;
+        auto kern = sc4 ? mxfp_gemm_tall_kernel<FW, F32, true> : mxfp_gemm_tall_kernel<FW, F32, false>;
+        static std::atomic<uint64_t> lds_allowed[2] = {{0}, {0}};
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed[sc4])) return rc;
         const int tiles_m = (M + UM - 1) / UM;
         const int walks = tiles_m * (N / UN) * plan.splits;          // at most one per CU (the plan splits only then)
         hipLaunchKernelGGL(kern, dim3((unsigned)((walks + 7) / 8 * 8)), dim3(kGemmThreads), U_LDS_BYTES, s,

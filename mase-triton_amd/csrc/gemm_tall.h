@@ -116,7 +116,9 @@ struct TallTile {
     int m0, n0;
 };
 
-template <class FW, int DT_OUT>
+// SC4: the k range of a walk is a multiple of 512, and the scales are fetched 16 bytes per row every fourth macro step
+// (a load of 4 bytes per row touches as many cache lines, one per row, and the address unit's time goes by lines)
+template <class FW, int DT_OUT, bool SC4>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_tall_kernel(
     const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, int splits, int64_t y_split_bytes) {
@@ -198,13 +200,27 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         constexpr int q = decltype(q_c)::value;
         async_load16(wn[q], w_voff, w_src + q * 32);
     };
+    // SC4: the scale bytes of four macro steps (16 per row) arrive in one load every fourth macro step; in the other three
+    // the same instruction reads one address for all lanes (one cache line instead of one per row), so that the number
+    // of vector-memory operations per macro step, which the waits count, stays the same
+    u32x4 sq, sn4;               // landing area of that load; the four dwords in use
+    uint32_t ws_voff_now = ws_voff;
+    bool sc_fresh = true;        // wave-uniform: the load in flight carries new scales
+    int sc_j = 0;                // which dword of sn4 the next macro step uses
     auto issue_w_scales = [&](const uint8_t* ws_src) {
-        asm volatile("global_load_dword %0, %1, %2" : "=v"(sn) : "v"(ws_voff), "s"(ws_src) : "memory");
+        if constexpr (SC4) asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sq) : "v"(ws_voff_now), "s"(ws_src) : "memory");
+        else asm volatile("global_load_dword %0, %1, %2" : "=v"(sn) : "v"(ws_voff), "s"(ws_src) : "memory");
+    };
+    auto take_scales = [&]() {   // after the wait for that load
+        if constexpr (SC4) {
+            if (sc_fresh) sn4 = sq;
+            sn = sc_j == 0 ? sn4.x : sc_j == 1 ? sn4.y : sc_j == 2 ? sn4.z : sn4.w;
+        }
     };
     auto issue_w = [&](const uint8_t* w_src, const uint8_t* ws_src) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) async_load16(wn[q], w_voff, w_src + q * 32);
-        asm volatile("global_load_dword %0, %1, %2" : "=v"(sn) : "v"(ws_voff), "s"(ws_src) : "memory");
+        issue_w_scales(ws_src);
     };
     // DMA i (rows 8i .. 8i+7 of the wave) of the 64-k half at `src` into stage `stage`
     auto issue_a = [&](const uint8_t* src, int stage, auto i_c) {
@@ -232,6 +248,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         wait_vmcnt<0>(wn[1], sn);
         wait_vmcnt<0>(wn[2], sn);
         wait_vmcnt<0>(wn[3], sn);
+        if constexpr (SC4) wait_vmcnt<0>(sq, sn);
+        take_scales();
         static_for<8>([&](auto i_c) { issue_a(cur.a + 128, 1, i_c); });
         compose_to(wn[0], sn & 0xFFu, 0, 0);
         compose_to(wn[1], (sn >> 8) & 0xFFu, 0, 1);
@@ -269,6 +287,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
             wait_vmcnt<16>(wn[1], sn);
             wait_vmcnt<16>(wn[2], sn);
             wait_vmcnt<16>(wn[3], sn);
+            if constexpr (SC4) wait_vmcnt<16>(sq, sn);
+            take_scales();
             // does any wavefront lane hold a scale of 255 (a block that held inf / NaN) among these four?  Checked once
             // per macro step; the patch-up code below runs only then.
             const uint32_t inv = ~sn;
@@ -425,7 +445,14 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         a0_nxt = (wrap ? next.a : cur.a) + (size_t)mn * (UMAC * 2);
         a1_nxt = a0_nxt + 128;
         w_nxt = (wrap ? next.w : cur.w) + (size_t)mn * UMAC;
-        ws_nxt = (wrap ? next.ws : cur.ws) + mn * (UMAC / 32);
+        if constexpr (SC4) {
+            sc_j = mn & 3;
+            sc_fresh = sc_j == 0;
+            ws_voff_now = sc_fresh ? ws_voff : 0u;
+            ws_nxt = (wrap ? next.ws : cur.ws) + (mn >> 2) * 16;
+        } else {
+            ws_nxt = (wrap ? next.ws : cur.ws) + mn * (UMAC / 32);
+        }
         step(IntC<0>{}, first_c);
         step(IntC<1>{}, IntC<0>{});
         step(IntC<2>{}, IntC<0>{});

@@ -150,6 +150,9 @@ def test_mxfp_linear_vs_cpu_reference_path(mh):
     ((3001, 5376, 384), "OCP_MXFP6_E3M2", torch.float16),    # 6 tile rows, the last one overlapping by 71 rows
     ((2048, 8320, 384), "MXFP8_E4M3_fn", torch.float32),     # fp32 output: 16 staging passes per tile, several tiles per workgroup
     ((1000, 12288, 128), "OCP_MXFP4_E2M1", torch.float32),   # fp32 output, shifted last tile row
+    ((2048, 8320, 1536), "MXFP8_E4M3_fn", torch.bfloat16),   # K % 512 == 0: scales fetched 16 bytes at a time, three fetches per tile, several tiles per workgroup
+    ((4096, 4096, 2560), "OCP_MXFP4_E2M1", torch.float32),   # the same with five fetches per tile, one tile per workgroup
+    ((1024, 8192, 2176), "OCP_MXFP6_E2M3", torch.bfloat16),  # 17 macro steps: not a multiple of four, scales fetched every step
 ])
 def test_gemm_large_tile_shapes(mh, MNK, w_tag, odt):
     """Shapes for which the launcher picks the 512 x 128 tile kernel (its tiles fill the CUs in whole rounds; dense A, no
@@ -369,20 +372,21 @@ def test_gemm_split_k(mh, MNK, splits, w_tag, odt, with_bias):
         assert torch.equal(y, y_plain)
 
 
-@pytest.mark.parametrize("MNK,odt,with_bias", [
-    ((300, 4096, 12288), torch.bfloat16, True),    # 2 x 32 tiles of 256 x 128, the second tile row mostly past M; 4 splits of 24
-    ((384, 4096, 12416), torch.float32, False),    # 97 macro steps as 25 + 25 + 25 + 22
-    ((1000, 4096, 12288), torch.bfloat16, True),   # 2 x 32 tiles of 512 x 128, the second shifted up to end at row M - 1; 4 splits
-    ((1024, 4096, 12288), torch.float32, False),   # the same tiles, fp32 output
+@pytest.mark.parametrize("MNK,splits,odt,with_bias", [
+    ((300, 4096, 12288), 4, torch.bfloat16, True),    # 2 x 32 tiles of 256 x 128, the second tile row mostly past M; 4 splits of 24
+    ((384, 4096, 12416), 4, torch.float32, False),    # 97 macro steps as 25 + 25 + 25 + 22
+    ((1000, 4096, 12288), 4, torch.bfloat16, True),   # 2 x 32 tiles of 512 x 128, the second shifted up to end at row M - 1; 4 splits
+    ((1024, 4096, 12288), 4, torch.float32, False),   # the same tiles, fp32 output
+    ((1024, 4096, 6400), 2, torch.bfloat16, True),    # 50 macro steps in two splits of 25 (256 x 128 tiles: 64 tiles of 512 x 128 price higher here)
 ])
-def test_gemm_split_k_larger_tiles(mh, MNK, odt, with_bias):
+def test_gemm_split_k_larger_tiles(mh, MNK, splits, odt, with_bias):
     """Long K and an output too large for more than two splits of its 128 x 128 tiles: the split runs on 256 x 128 or
-    512 x 128 tiles (here four splits each; the smaller tiles would allow two, or none).  The whole output against an fp32
+    512 x 128 tiles (the smaller tiles would allow fewer splits, or none).  The whole output against an fp32
     dequantize-then-matmul on the GPU, a sample of it against float64 accumulation, and the unsplit call."""
     from mase_hip import _lib
 
     M, N, K = MNK
-    assert _lib.load().mase_hip_mxfp_gemm_workspace_bytes(1, M, N, K) == 4 * M * N * 4
+    assert _lib.load().mase_hip_mxfp_gemm_workspace_bytes(1, M, N, K) == splits * M * N * 4
     g = torch.Generator().manual_seed(M + N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
