@@ -28,9 +28,9 @@ for p in (ROOT, os.path.join(ROOT, "mase-triton_amd"), os.path.join(ROOT, "tests
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # HBM-side bytes per launch of the C4 GEMM kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch
-# 933756.3 and 458946.5), scaled by what the same counters read for a plain 256 MiB copy (x2.000 and x1.000),
+# 934031.4 and 458935.5), scaled by what the same counters read for a plain 256 MiB copy (x2.000 and x1.000),
 # collected with `--counter-probe`.  Algorithmic bytes are 0.665e9.
-GEMM_C4_TRAFFIC_BYTES = int((933756.3 * 2.0 + 458946.5 * 1.0) * 1024)
+GEMM_C4_TRAFFIC_BYTES = int((934031.4 * 2.0 + 458935.5 * 1.0) * 1024)
 
 
 def parse_args():
