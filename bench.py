@@ -31,6 +31,13 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # 934031.4 and 458935.5), scaled by what the same counters read for a plain 256 MiB copy (x2.000 and x1.000),
 # collected with `--counter-probe`.  Algorithmic bytes are 0.665e9.
 GEMM_C4_TRAFFIC_BYTES = int((934031.4 * 2.0 + 458935.5 * 1.0) * 1024)
+# the same two counters for the C3 cast kernels (14336 x 4096 bf16, E2M1): extract 57364.5 / 59136.0, compose 30480.3 / 114690.5
+# KiB per dispatch; algorithmic bytes are 177995776 for either
+CAST_TRAFFIC_BYTES = {
+    ("extract_mxfp", "C3"): int((57364.5 * 2.0 + 59136.0 * 1.0) * 1024),
+    ("compose_mxfp", "C3"): int((30480.3 * 2.0 + 114690.5 * 1.0) * 1024),
+    ("extract+compose_mxfp", "C3"): int(((57364.5 + 30480.3) * 2.0 + (59136.0 + 114690.5) * 1.0) * 1024),
+}
 
 
 def parse_args():
@@ -189,7 +196,7 @@ def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
             "kernel": name, "workload": workload, "bytes_per_launch": bytes_per_launch,
             "avg_ms": round(avg_ms, 5), "best_ms": round(med_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": CAST_TRAFFIC_BYTES.get((name, workload.split(":")[0]))},
             "cache_resident_GBps": round(bytes_per_launch / (cached_ms * 1e-3) / 1e9, 1),
             "plain_copy_same_bytes_GBps": plain_copy_gbps(bytes_per_launch),
         })
