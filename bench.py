@@ -369,6 +369,45 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
     torch.cuda.synchronize()
 
 
+def bench_c5(torch, steps=20, warmup=8):
+    """Context, not the metric: a Llama-3-8B SwiGLU MLP block of MXFPLinearPTQ layers, down(silu(gate(x)) * up(x)),
+    weights gate / up [14336, 4096] and down [4096, 14336] ~N(0, 0.02) stored as MXFP6 E3M2, MXFP8 E4M3 activations,
+    block 32, x [4 x 2048, 4096] bf16 ~N(0, 1): three quantise kernels, three GEMMs and the activation per step."""
+    from mase_hip.mxfp.layers import MXFPLinearPTQ
+    from mase_hip.mxfp.meta import MXFP8_E4M3_fn, MXFPMeta
+
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev).manual_seed(11)
+    x = torch.randn(4, 2048, 4096, generator=gen, device=dev).to(torch.bfloat16)
+    wfmt = MXFPMeta(32, 8, 3, 2, True, "rn")
+    out = {}
+    for backend in ("fused", "separate"):
+        ls = []
+        for n_out, n_in in ((14336, 4096), (14336, 4096), (4096, 14336)):
+            lin = torch.nn.Linear(n_in, n_out, bias=False, dtype=torch.bfloat16, device=dev)
+            lin.weight.data.copy_((0.02 * torch.randn(n_out, n_in, generator=gen, device=dev)).to(torch.bfloat16))
+            ls.append(MXFPLinearPTQ.from_linear(lin, MXFP8_E4M3_fn, wfmt, None, "XqWqB", backend))
+            del lin
+        g, u, d = ls
+
+        def mlp():
+            return d(torch.nn.functional.silu(g(x)) * u(x))
+
+        for _ in range(warmup):
+            mlp()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            mlp()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        out[f"{backend}_ms"] = round(ms, 4)
+        out[f"{backend}_TFLOPs"] = round(3 * 2.0 * 8192 * 4096 * 14336 / (ms * 1e-3) / 1e12, 1)
+        del ls, g, u, d
+    out["note"] = "whole block per step (x quantised three times, SiLU and the product in torch); flop = the three GEMMs"
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -425,6 +464,7 @@ def main():
         },
     }
     if not args.skip_hbm:
+        result["context"]["c5_swiglu_mlp_block"] = bench_c5(torch)
         result["hbm_kernels"] = bench_hbm(
             torch, mxk, mfk,
             lambda e, m: MXFPMeta(32, 8, e, m, True, "rn"), lambda e, m: MinifloatMeta(e, m, True, "rn"))
