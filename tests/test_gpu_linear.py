@@ -377,6 +377,7 @@ def test_gemm_split_k(mh, MNK, splits, w_tag, odt, with_bias):
     ((384, 4096, 12416), 4, torch.float32, False),    # 97 macro steps as 25 + 25 + 25 + 22
     ((1000, 4096, 12288), 4, torch.bfloat16, True),   # 2 x 32 tiles of 512 x 128, the second shifted up to end at row M - 1; 4 splits
     ((1024, 4096, 12288), 4, torch.float32, False),   # the same tiles, fp32 output
+    ((1024, 4096, 12800), 4, torch.bfloat16, False),  # 512 x 128 tiles, four splits of 25 macro steps: not a multiple of four, scales fetched every step
     ((1024, 4096, 6400), 2, torch.bfloat16, True),    # 50 macro steps in two splits of 25 (256 x 128 tiles: 64 tiles of 512 x 128 price higher here)
 ])
 def test_gemm_split_k_larger_tiles(mh, MNK, splits, odt, with_bias):
