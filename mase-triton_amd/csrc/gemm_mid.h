@@ -180,9 +180,9 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
                     else async_load_u8(w_scale[ns][(k - A_DMAS) / 2], ws_voff[(k - A_DMAS) / 2], ws_src);
                 };
                 static_assert(OPS == 2 * QW, "two vector-memory operations beside each 16-k step");
-                bool any255 = false;
-                static_for<W_LOADS>([&](auto h_c) __attribute__((always_inline)) { any255 |= w_scale[cs][decltype(h_c)::value] == 255u; });
-                any255 = __builtin_amdgcn_ballot_w64(any255) != 0;
+                bool any_slow = false;
+                static_for<W_LOADS>([&](auto h_c) __attribute__((always_inline)) { any_slow |= Composer<FW>::is_slow(w_scale[cs][decltype(h_c)::value]); });
+                any_slow = __builtin_amdgcn_ballot_w64(any_slow) != 0;
                 const uint8_t* const pa = lds_a + (r % 3) * MD_A_STAGE + wave_m * (64 * MD_ROW);
                 const uint8_t* const pw = lds_w + (r % 2) * MD_W_STAGE + wave_n * (64 * MD_ROW);
                 uint8_t* const st = lds_w + w_stage * MD_W_STAGE;
@@ -218,8 +218,8 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
                     o[2 * d0 + 3] = cmp.pair_hi(c1);
                     if constexpr (q % 2 == 1) {  // the 16 codes of load h are done
                         uint4 lo = make_uint4(o[0], o[1], o[2], o[3]), hi = make_uint4(o[4], o[5], o[6], o[7]);
-                        if (any255)
-                            Composer<FW>::fix255(w_scale[cs][h], make_uint4(w_raw[cs][h].x, w_raw[cs][h].y, w_raw[cs][h].z, w_raw[cs][h].w), lo, hi);
+                        if (any_slow)
+                            Composer<FW>::fix_slow(w_scale[cs][h], make_uint4(w_raw[cs][h].x, w_raw[cs][h].y, w_raw[cs][h].z, w_raw[cs][h].w), lo, hi);
                         *reinterpret_cast<uint4*>(st + w_lds_off[h][0]) = lo;
                         *reinterpret_cast<uint4*>(st + w_lds_off[h][1]) = hi;
                     }

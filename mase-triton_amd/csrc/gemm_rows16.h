@@ -104,18 +104,10 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_rows16_kernel(
         uint32_t o[4];
         cmp.pair2(w_raw[slot].x, o[0], o[1]);
         cmp.pair2(w_raw[slot].y, o[2], o[3]);
-        if (FW{}.E() < 5 && __builtin_amdgcn_ballot_w64(scale == 255u) != 0 && scale == 255u) {
-            // scale 255 means "times +inf" in the reference: zero codes give NaN (non-zero ones already overflowed)
-            const uint32_t w[2] = {w_raw[slot].x, w_raw[slot].y};
-            const uint32_t mag = (1u << (FW{}.E() + FW{}.M())) - 1u;
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int b = 0; b < 4; ++b)
-                    if (((w[j] >> (8 * b)) & mag) == 0u) {
-                        uint32_t& d = o[2 * j + (b >> 1)];
-                        d = (b & 1) ? ((d & 0x0000FFFFu) | 0x7FC00000u) : ((d & 0xFFFF0000u) | 0x00007FC0u);
-                    }
+        if (__builtin_amdgcn_ballot_w64(Composer<FW>::is_slow(scale)) != 0 && Composer<FW>::is_slow(scale)) {
+            // rare scales (255, "times +inf" in the reference, among them) that the fast compose does not take
+            cmp.pair2_slow(w_raw[slot].x, o[0], o[1]);
+            cmp.pair2_slow(w_raw[slot].y, o[2], o[3]);
         }
         *reinterpret_cast<uint4*>(lds_w + (mac & 1) * W_STAGE + w_lds_off) = make_uint4(o[0], o[1], o[2], o[3]);
     };

@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     // during steps 2, 3 of the current one), `wc[2..3]`, `sc` keep slabs 2, 3 of the current one
     u32x4 wc[4], wn[4];
     uint32_t sc, sn;
-    bool any255_cur = true, any255_nxt = true;  // wave-uniform: a scale of 255 among the macro step's four
+    bool any_slow_cur = true, any_slow_nxt = true;  // wave-uniform: a scale among the macro step's four that the fast compose does not take
     auto issue_w_codes = [&](const uint8_t* w_src, auto q_c) {
         constexpr int q = decltype(q_c)::value;
         async_load16(wn[q], w_voff, w_src + q * 32);
@@ -289,10 +289,10 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
             wait_vmcnt<16>(wn[3], sn);
             if constexpr (SC4) wait_vmcnt<16>(sq, sn);
             take_scales();
-            // does any wavefront lane hold a scale of 255 (a block that held inf / NaN) among these four?  Checked once
+            // does any wavefront lane hold a scale among these four that needs the slow compose (255, a block that held inf /
+            // NaN, or one so large that the product leaves the bf16 range)?  Checked once
             // per macro step; the patch-up code below runs only then.
-            const uint32_t inv = ~sn;
-            any255_nxt = __builtin_amdgcn_ballot_w64(((inv - 0x01010101u) & sn & 0x80808080u) != 0u) != 0;
+            any_slow_nxt = __builtin_amdgcn_ballot_w64(Composer<FW>::any_slow4(sn)) != 0;
         }
         const u32x4& codes = S < 2 ? wc[(S + 2) & 3] : wn[(S + 2) & 3];
         const uint32_t scale = ((S < 2 ? sc : sn) >> (8 * ((S + 2) & 3))) & 0xFFu;
@@ -389,12 +389,12 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         if (S & 1) __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
         {
             uint4 lo = make_uint4(o[0], o[1], o[2], o[3]), hi = make_uint4(o[4], o[5], o[6], o[7]);
-            if (S < 2 ? any255_cur : any255_nxt) Composer<FW>::fix255(scale, make_uint4(cw[0], cw[1], cw[2], cw[3]), lo, hi);
+            if (S < 2 ? any_slow_cur : any_slow_nxt) Composer<FW>::fix_slow(scale, make_uint4(cw[0], cw[1], cw[2], cw[3]), lo, hi);
             *reinterpret_cast<uint4*>(wst + w_lds_off[PP][0]) = lo;
             *reinterpret_cast<uint4*>(wst + w_lds_off[PP][1]) = hi;
         }
         if (S == 3) {
-            any255_cur = any255_nxt;
+            any_slow_cur = any_slow_nxt;
             wc[2] = wn[2];
             wc[3] = wn[3];
             sc = sn;

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
                     else if constexpr (k == A_DMAS) async_load16(w_raw[ns], w_voff, w_src);
                     else async_load_u8(w_scale[ns], ws_voff, ws_src);
                 };
-                const bool any255 = __builtin_amdgcn_ballot_w64(w_scale[cs] == 255u) != 0;
+                const bool any_slow = __builtin_amdgcn_ballot_w64(Composer<FW>::is_slow(w_scale[cs])) != 0;
                 const Composer<FW> cmp(w_scale[cs]);
                 const uint8_t* const pa = lds_a + (r % 3) * WD_A_STAGE + wave_m * (64 * WD_ROW);
                 const uint8_t* const pw = lds_w + (r % 2) * WD_W_STAGE + wave_n * (64 * WD_ROW);
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
                     __builtin_amdgcn_sched_barrier(0);
                 });
                 uint4 lo = make_uint4(o[0], o[1], o[2], o[3]), hi = make_uint4(o[4], o[5], o[6], o[7]);
-                if (any255) Composer<FW>::fix255(w_scale[cs], make_uint4(w_raw[cs].x, w_raw[cs].y, w_raw[cs].z, w_raw[cs].w), lo, hi);
+                if (any_slow) Composer<FW>::fix_slow(w_scale[cs], make_uint4(w_raw[cs].x, w_raw[cs].y, w_raw[cs].z, w_raw[cs].w), lo, hi);
                 *reinterpret_cast<uint4*>(st + w_lds_off[0]) = lo;
                 *reinterpret_cast<uint4*>(st + w_lds_off[1]) = hi;
             }
