@@ -204,6 +204,30 @@ int mase_hip_mxfp_gemm_ws(const void* a_dense, int a_dtype, const uint8_t* a_sca
                           int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
                           void* workspace, int64_t workspace_bytes, void* stream);
 
+/*
+ * The same product as mase_hip_mxfp_gemm_ws for callers that cannot allocate device memory at all (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc): the partial sums of the K split live in a
+ * device array that is part of the library image, MASE_HIP_STATIC_WORKSPACE_BYTES on every GPU the library runs on,
+ * held until the process ends.  The call allocates and frees nothing.  A shape whose split asks for more
+ * (mase_hip_mxfp_gemm_workspace_bytes; on a 256-CU device the largest request of any shape is 64 MiB, made by 512-row
+ * tiles split two to four ways, e.g. [1024, 4096] over K = 14336) is refused with -2: pass your own workspace to
+ * mase_hip_mxfp_gemm_ws then, or call mase_hip_mxfp_gemm, which does not split and needs none.
+ * A shape that is not split does not touch the array.
+ * Every call on a GPU shares that GPU's array, which keeps the last call's partial sums (nothing in it has to start
+ * at zero): calls on one GPU must be ordered on one stream, calls that overlap there race.  The first call on a
+ * device looks up the array's address (it loads the library's code object there if nothing has yet): make it once
+ * outside any stream capture.
+ * No counterpart in the reference, whose GEMM is torch's and allocates its own workspace; it exists for the callers
+ * above, those that cannot allocate.
+ */
+#define MASE_HIP_STATIC_WORKSPACE_BYTES (32 * 1024 * 1024)
+int mase_hip_mxfp_gemm_static_ws(const void* a_dense, int a_dtype, const uint8_t* a_scales,
+                                 const uint8_t* a_elements, int a_exp_bits, int a_frac_bits,
+                                 const uint8_t* w_scales, const uint8_t* w_elements, int w_exp_bits,
+                                 int w_frac_bits, const void* bias, int bias_dtype, void* y,
+                                 int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
+                                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

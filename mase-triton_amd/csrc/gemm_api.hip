@@ -4,6 +4,8 @@
 
 using namespace mase;
 
+extern "C" int64_t mase_hip_mxfp_gemm_workspace_bytes(int a_is_dense, int64_t M, int64_t N, int64_t K);
+
 static int gemm_entry(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements, int a_exp_bits,
                       int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements, int w_exp_bits, int w_frac_bits,
                       const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
@@ -52,6 +54,44 @@ extern "C" int mase_hip_mxfp_gemm_ws(const void* a_dense, int a_dtype, const uin
                                      void* stream) {
     return gemm_entry(a_dense, a_dtype, a_scales, a_elements, a_exp_bits, a_frac_bits, w_scales, w_elements, w_exp_bits, w_frac_bits,
                       bias, bias_dtype, y, out_dtype, M, N, K, block_size, workspace, workspace_bytes, stream);
+}
+
+// ---- the same product for callers that cannot allocate: the partial sums of the K split live in a static device array
+static __device__ __align__(256) unsigned char scratch[MASE_HIP_STATIC_WORKSPACE_BYTES];
+
+// Device address of `scratch` on the current device (every device has its own copy of the array at its own address),
+// looked up once per device.  In host code the array's name is only a handle for this lookup, never an address.
+static int static_workspace(void** out) {
+    static std::atomic<void*> known[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(ERR_RUNTIME, std::string("hipGetDevice: ") + hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(ERR_UNSUPPORTED, "the static workspace serves device ordinals 0..63");
+    void* p = known[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return fail(ERR_RUNTIME, std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e));
+        known[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return OK;
+}
+
+extern "C" int mase_hip_mxfp_gemm_static_ws(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements,
+                                            int a_exp_bits, int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements,
+                                            int w_exp_bits, int w_frac_bits, const void* bias, int bias_dtype, void* y, int out_dtype,
+                                            int64_t M, int64_t N, int64_t K, int block_size, void* stream) {
+    const int64_t need = mase_hip_mxfp_gemm_workspace_bytes(a_dense != nullptr, M, N, K);
+    if (need > (int64_t)MASE_HIP_STATIC_WORKSPACE_BYTES)
+        return fail(ERR_UNSUPPORTED, "this shape splits K into " + std::to_string(need) + " bytes of partial sums, more than the " +
+                                         std::to_string((long long)MASE_HIP_STATIC_WORKSPACE_BYTES) +
+                                         " bytes of the static workspace: pass a workspace to mase_hip_mxfp_gemm_ws, or call mase_hip_mxfp_gemm (no split, no workspace)");
+    void* ws = nullptr;
+    if (need > 0)
+        if (int rc = static_workspace(&ws)) return rc;
+    // every split writes all of its [M, N] array before the second kernel reads it: nothing has to start at zero
+    return gemm_entry(a_dense, a_dtype, a_scales, a_elements, a_exp_bits, a_frac_bits, w_scales, w_elements, w_exp_bits, w_frac_bits,
+                      bias, bias_dtype, y, out_dtype, M, N, K, block_size, ws, ws ? (int64_t)MASE_HIP_STATIC_WORKSPACE_BYTES : 0, stream);
 }
 
 extern "C" int64_t mase_hip_mxfp_gemm_workspace_bytes(int a_is_dense, int64_t M, int64_t N, int64_t K) {

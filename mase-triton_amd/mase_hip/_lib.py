@@ -32,6 +32,8 @@ SIGNATURES = {
     "mase_hip_mxfp_gemm_ws": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
                                      _vp, _i32, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
     "mase_hip_mxfp_gemm_workspace_bytes": (_i64, [_i32, _i64, _i64, _i64]),
+    "mase_hip_mxfp_gemm_static_ws": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
+                                            _vp, _i32, _i64, _i64, _i64, _i32, _vp]),
 }
 
 
