@@ -27,17 +27,48 @@ for p in (ROOT, os.path.join(ROOT, "mase-triton_amd"), os.path.join(ROOT, "tests
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
-# HBM-side bytes per launch of the C4 GEMM kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch
-# 934031.4 and 458935.5), scaled by what the same counters read for a plain 256 MiB copy (x2.000 and x1.000),
-# collected with `--counter-probe`.  Algorithmic bytes are 0.665e9.
-GEMM_C4_TRAFFIC_BYTES = int((934031.4 * 2.0 + 458935.5 * 1.0) * 1024)
-# the same two counters for the C3 cast kernels (14336 x 4096 bf16, E2M1): extract 57364.5 / 59136.0, compose 30480.3 / 114690.5
-# KiB per dispatch; algorithmic bytes are 177995776 for either
-CAST_TRAFFIC_BYTES = {
-    ("extract_mxfp", "C3"): int((57364.5 * 2.0 + 59136.0 * 1.0) * 1024),
-    ("compose_mxfp", "C3"): int((30480.3 * 2.0 + 114690.5 * 1.0) * 1024),
-    ("extract+compose_mxfp", "C3"): int(((57364.5 + 30480.3) * 2.0 + (59136.0 + 114690.5) * 1.0) * 1024),
-}
+# HBM-side bytes per launch (roofline.traffic) are not measured by this run: they come from the committed summary of two
+# rocprofv3 --pmc runs of `bench.py --counter-probe` (FETCH_SIZE, then WRITE_SIZE), written by
+# `bench.py --summarize-counters`.  Every entry carries a fingerprint of the kernel sources it was taken with; when the
+# sources have changed since, the figure is reported as null (with a note on stderr) instead of a stale number.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_counters_gemm_c4_casts_c1_c2_c3.md")
+CSRC = os.path.join(ROOT, "mase-triton_amd", "csrc")
+GEMM_SOURCES = ("gemm_tall.h", "gemm_impl.h", "mxfp_compose.h", "mase_device.h")
+CAST_SOURCES = ("cast_kernels.hip", "mxfp_compose.h", "mase_device.h")
+
+
+def sources_fingerprint(names) -> str:
+    import hashlib
+
+    h = hashlib.sha256()
+    for n in names:
+        with open(os.path.join(CSRC, n), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+_traffic_table = None
+
+
+def traffic_bytes(key: str, sources):
+    """HBM bytes per launch of kernel/workload `key` from the committed counter summary, or None."""
+    global _traffic_table
+    if _traffic_table is None:
+        _traffic_table = {}
+        try:
+            text = open(TRAFFIC_SUMMARY).read()
+            block = text[text.index("```json") + 7:]
+            _traffic_table = json.loads(block[:block.index("```")])
+        except (OSError, ValueError) as exc:
+            print(f"bench.py: no usable counter summary at {TRAFFIC_SUMMARY} ({exc}): traffic reported as null", file=sys.stderr)
+    row = _traffic_table.get(key)
+    if row is None:
+        return None
+    if row.get("sources") != sources_fingerprint(sources):
+        print(f"bench.py: the kernel sources behind '{key}' changed after {os.path.basename(TRAFFIC_SUMMARY)} was taken: "
+              "traffic reported as null until the counters are collected again", file=sys.stderr)
+        return None
+    return int(row["traffic_bytes"])
 
 
 def parse_args():
@@ -52,6 +83,9 @@ def parse_args():
     ap.add_argument("--counter-probe", action="store_true",
                     help="profiling aid for rocprofv3 --pmc: a plain 256 MiB device copy (calibration), then 3 launches "
                          "each of the GEMM and of the C3 extract / compose kernels; prints nothing to time")
+    ap.add_argument("--summarize-counters", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="no GPU needed: turn the output folders of two `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of "
+                         "`bench.py --counter-probe` into the markdown summary kept under profiles/ (stdout)")
     ap.add_argument("--shape-sweep", action="store_true",
                     help="context run, not the metric: mxfp_linear fused vs separate over M at N=14336, K=4096, and the "
                          "in-place casts along a non-last axis against the permuted-copy route; prints its own JSON line")
@@ -60,6 +94,27 @@ def parse_args():
 
 def event_ms(pairs):
     return [a.elapsed_time(b) for a, b in pairs]
+
+
+def settle(torch, fn, group=5, tol=0.01, most=100):
+    """Run fn in groups until the time per call stops changing; returns what the first and the last group took."""
+    first = prev = ms = None
+    done = 0
+    while done < most:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(group):
+            fn()
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_time(e1) / group
+        done += group
+        if first is None:
+            first = ms
+        elif done >= 3 * group and abs(ms - prev) <= tol * prev:
+            break
+        prev = ms
+    return {"steps": done, "first_group_ms_per_step": round(first, 4), "settled_ms_per_step": round(ms, 4)}
 
 
 def bench_linear(args, torch, MXFP_F, kernels, fmt):
@@ -86,6 +141,10 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
     y_api = MXFP_F.mxfp_linear(**call)
     assert torch.equal(step().view(torch.int16), y_api.view(torch.int16)), "bench step differs from mxfp_linear"
     del y_api
+    # The shader clock settles over the first few dozen launches after idle (the step gets faster), so a short counted
+    # warm-up would time the ramp.  Before the counted warm-up: steps in groups of five until two consecutive groups agree
+    # within 1 %, at most 100 steps.  Both figures are reported.
+    prewarm = settle(torch, step)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -133,6 +192,7 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
     dense_ms = (time.perf_counter() - t3) * 1e3 / args.steps
     del a_dq, w_dq
     return {
+        "prewarm": prewarm,
         "separate_ms": sep_ms, "dense_ms": dense_ms,
         "ms_per_step": ms_per_step,
         "tflops_step": flop / (ms_per_step * 1e-3) / 1e12,
@@ -171,48 +231,120 @@ def time_kernel(torch, launch, n_variants, iters=48, warmup=8, reps=5):
     return sum(times) / len(times), min(times)
 
 
-def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
-    """Cast kernels on their own configurations.  Algorithmic bytes per element: MXFP extract from
-    bf16 2 + 1 + 1/32, compose to bf16 1 + 1/32 + 2, fused minifloat QDQ fp32->fp32 4 + 4."""
+def load_bench_lib():
+    """lib/libmase_bench.so: the tuned streaming copy used as the yardstick of the bandwidth-bound kernels."""
+    import ctypes
+
+    path = os.path.join(ROOT, "mase-triton_amd", "mase_hip", "lib", "libmase_bench.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build it with `python mase-triton_amd/build.py`")
+    lib = ctypes.CDLL(path)
+    lib.mase_bench_stream_copy.restype = ctypes.c_int
+    lib.mase_bench_stream_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    return lib
+
+
+def cpu_cast_baselines(torch):
+    """The reference's CPU path for the casts (tensor-op restatement under oracle/), on bounded samples of the same
+    workloads; GB/s by the same algorithmic bytes per element as the GPU rows.  Keyed by (kernel, config)."""
+    from oracle import torch_fake
+    import workloads
+
+    threads = torch.get_num_threads()
+    out = {}
+
+    def timed(fn):
+        fn()                      # first call pays for allocator growth
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    def entry(nbytes, dt, sample):
+        return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port", "sample": f"{sample}, {dt:.2f} s"}
+
+    for tag, full, rows, (e, m) in (("C1", workloads.make_c1, 2048, (4, 3)), ("C3", workloads.make_c3, 2048, (2, 1))):
+        x = full(rows, 4096).reshape(-1)
+        n = x.numel()
+        sc, el = torch_fake.mxfp_split(x, 32, e, m)
+        sample = f"{rows} rows x 4096 of {tag}'s distribution"
+        t_ext = timed(lambda: torch_fake.mxfp_split(x, 32, e, m))
+        t_cmp = timed(lambda: torch_fake.mxfp_join(sc, el, e, m, True, torch.bfloat16))
+        out[("extract_mxfp", tag)] = entry(n * (3 + 1 / 32), t_ext, sample)
+        out[("compose_mxfp", tag)] = entry(n * (3 + 1 / 32), t_cmp, sample)
+        out[("extract+compose_mxfp", tag)] = entry(n * (6 + 1 / 16), t_ext + t_cmp, sample)
+        out[("qdq_mxfp_fused", tag)] = entry(n * 4.0, t_ext + t_cmp, sample + " (the reference has no fused pass: extract then compose)")
+    x = workloads.make_c2(1 << 22)
+    n = x.numel()
+    for e, m in ((4, 3), (5, 2)):
+        codes = torch_fake.minifloat_encode(x, e, m)
+        sample = "2^22 of C2's 2^24 elements"
+        t_ext = timed(lambda: torch_fake.minifloat_encode(x, e, m))
+        t_cmp = timed(lambda: torch_fake.minifloat_decode(codes, e, m, True, torch.float32))
+        tag = f"C2/E{e}M{m}"
+        out[("extract_minifloat", tag)] = entry(n * 6.0, t_ext, sample)
+        out[("compose_minifloat", tag)] = entry(n * 6.0, t_cmp, sample)
+        out[("qdq_minifloat_fused", tag)] = entry(n * 8.0, t_ext + t_cmp, sample + " (encode then decode)")
+    return out
+
+
+def bench_hbm(torch, with_cpu):
+    """Cast kernels on their own configurations, on the configurations' own value distributions (tests/workloads.py: C3 with
+    its all-zero blocks and planted inf / NaN, C2 with its outliers, zeros and subnormals).  Algorithmic bytes per element:
+    MXFP extract from bf16 2 + 1 + 1/32, compose to bf16 1 + 1/32 + 2, fused minifloat QDQ fp32 -> fp32 4 + 4."""
+    import workloads
+    from mase_hip import _lib
+
     dev = "cuda:0"
     out = []
     copy_cache = {}
+    lib = _lib.load()
+    blib = load_bench_lib()
+    sp_of = lambda: _lib.stream_ptr(torch.device(dev))
+    cpu = cpu_cast_baselines(torch) if with_cpu else {}
 
-    def plain_copy_gbps(nbytes):
-        """What a plain device-to-device copy moving the same number of bytes (half read, half written) reaches,
-        timed the same way: the practical ceiling of a streaming kernel of this size on this machine."""
+    def tuned_copy_gbps(nbytes):
+        """The hand-tuned streaming copy (csrc/bench/stream_copy.hip) moving the same number of bytes, half read and half
+        written, timed the same way; the better of its two launch shapes."""
         half = int(nbytes // 2) // 16 * 16
         if half not in copy_cache:
             k = max(2, (320 << 20) // (2 * half) + 1)
             src = [torch.empty(half, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(k)]
             dst = [torch.empty_like(t) for t in src]
-            avg, _ = time_kernel(torch, lambda i: dst[i].copy_(src[i]), k)
-            copy_cache[half] = round(2 * half / (avg * 1e-3) / 1e9, 1)
+            best = 0.0
+            for form in (0, 1):
+                def cp(i):
+                    assert blib.mase_bench_stream_copy(src[i].data_ptr(), dst[i].data_ptr(), half, form, sp_of()) == 0
+                avg, _ = time_kernel(torch, cp, k)
+                best = max(best, 2 * half / (avg * 1e-3) / 1e9)
+            assert torch.equal(src[0], dst[0])
+            copy_cache[half] = round(best, 1)
         return copy_cache[half]
 
-    def roof(name, workload, bytes_per_launch, avg_ms, med_ms, cached_ms):
+    def roof(name, cfg, workload, bytes_per_launch, avg_ms, best_ms, cached_ms):
         gbs = bytes_per_launch / (avg_ms * 1e-3) / 1e9
+        copy = tuned_copy_gbps(bytes_per_launch)
         out.append({
             "kernel": name, "workload": workload, "bytes_per_launch": bytes_per_launch,
-            "avg_ms": round(avg_ms, 5), "best_ms": round(med_ms, 5),
+            "avg_ms": round(avg_ms, 5), "best_ms": round(best_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": CAST_TRAFFIC_BYTES.get((name, workload.split(":")[0]))},
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic_bytes(f"{name} {cfg}", CAST_SOURCES)},
             "cache_resident_GBps": round(bytes_per_launch / (cached_ms * 1e-3) / 1e9, 1),
-            "plain_copy_same_bytes_GBps": plain_copy_gbps(bytes_per_launch),
+            "tuned_copy_same_bytes_GBps": copy, "frac_of_tuned_copy": round(gbs / copy, 3),
+            "cpu_baseline": cpu.get((name, cfg)),
         })
 
-    def mxfp_case(tag, rows, cols, e, m, copies):
-        meta = mx_meta(e, m)
+    def mxfp_case(tag, x_cpu, e, m, copies):
+        rows, cols = x_cpu.shape
         n = rows * cols
-        gen = torch.Generator(device=dev).manual_seed(0)
-        xs = [(torch.randn(n, generator=gen, device=dev)).to(torch.bfloat16) for _ in range(copies)]
-        comps = [mxk.extract_mxfp_components(x, meta) for x in xs]
+        x0 = x_cpu.reshape(-1).to(dev)
+        xs = [x0] + [x0.clone() for _ in range(copies - 1)]      # the same values in rotating buffers
+        sc0 = torch.empty(n // 32, dtype=torch.uint8, device=dev)
+        el0 = torch.empty(n, dtype=torch.uint8, device=dev)
+        _lib.check(lib.mase_hip_extract_mxfp(x0.data_ptr(), 2, sc0.data_ptr(), el0.data_ptr(), n, 32, e, m, 1, 0, sp_of()))
+        comps = [(sc0, el0)] + [(sc0.clone(), el0.clone()) for _ in range(copies - 1)]
         ext_bytes = n * (2 + 1 + 1 / 32)
         cmp_bytes = n * (1 + 1 / 32 + 2)
         # pre-allocated outputs so that the timed region holds only the kernel
-        from mase_hip import _lib
-        lib = _lib.load()
-        sp_of = lambda: _lib.stream_ptr(torch.device(dev))
         sc_o = [torch.empty_like(c[0]) for c in comps]
         el_o = [torch.empty_like(c[1]) for c in comps]
         y_o = [torch.empty_like(x) for x in xs]
@@ -230,24 +362,21 @@ def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
         def qdq(i):
             _lib.check(lib.mase_hip_qdq_mxfp(xs[i].data_ptr(), 2, y_o[i].data_ptr(), 2, n, 32, e, m, 1, 0, sp_of()))
 
-        wl = f"{tag}: {rows}x{cols} bf16, E{e}M{m}, block 32"
+        wl = f"{tag}: {rows}x{cols} bf16, E{e}M{m}, block 32, the configuration's value distribution"
         for name, fn, nbytes in (("extract_mxfp", ext, ext_bytes), ("compose_mxfp", cmp, cmp_bytes),
                                  ("extract+compose_mxfp", both, ext_bytes + cmp_bytes), ("qdq_mxfp_fused", qdq, n * 4.0)):
-            avg, med = time_kernel(torch, fn, copies)
+            avg, best = time_kernel(torch, fn, copies)
             cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
-            roof(name, wl, nbytes, avg, med, cavg)
+            roof(name, tag, wl, nbytes, avg, best, cavg)
         assert torch.equal(sc_o[0], comps[0][0]) and torch.equal(el_o[0], comps[0][1])
 
-    mxfp_case("C1", 4096, 4096, 4, 3, copies=12)   # 12 x (32 + 16.5) MiB in flight > 256 MiB cache
-    mxfp_case("C3", 14336, 4096, 2, 1, copies=4)
+    mxfp_case("C1", workloads.make_c1(), 4, 3, copies=12)   # 12 x (32 + 16.5) MiB in flight > 256 MiB cache
+    mxfp_case("C3", workloads.make_c3(), 2, 1, copies=4)
 
-    # C2: fused minifloat QDQ on 2^24 fp32
+    # C2: minifloat casts on 2^24 fp32
     n = 1 << 24
-    from mase_hip import _lib
-    lib = _lib.load()
-    sp_of = lambda: _lib.stream_ptr(torch.device(dev))
-    gen = torch.Generator(device=dev).manual_seed(1)
-    xs = [torch.randn(n, generator=gen, device=dev) for _ in range(6)]
+    x0 = workloads.make_c2().to(dev)
+    xs = [x0] + [x0.clone() for _ in range(5)]
     ys = [torch.empty_like(x) for x in xs]
     cs = [torch.empty(n, dtype=torch.uint16, device=dev) for _ in xs]
     for e, m in ((4, 3), (5, 2)):
@@ -260,12 +389,14 @@ def bench_hbm(torch, mxk, mfk, mx_meta, mf_meta):
         def cmp(i):
             _lib.check(lib.mase_hip_compose_minifloat(cs[i].data_ptr(), ys[i].data_ptr(), 0, n, e, m, 1, sp_of()))
 
-        wl = f"C2: 2^24 fp32, FP8 E{e}M{m}"
+        wl = f"C2: 2^24 fp32 with outliers, zeros and subnormals, FP8 E{e}M{m}"
+        for i in range(len(xs)):
+            ext(i)                # codes for the compose rows
         for name, fn, nbytes in (("qdq_minifloat_fused", qdq, n * 8.0), ("extract_minifloat", ext, n * 6.0),
                                  ("compose_minifloat", cmp, n * 6.0)):
-            avg, med = time_kernel(torch, fn, len(xs))
+            avg, best = time_kernel(torch, fn, len(xs))
             cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
-            roof(name, wl, nbytes, avg, med, cavg)
+            roof(name, f"C2/E{e}M{m}", wl, nbytes, avg, best, cavg)
     return out
 
 
@@ -348,12 +479,19 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
 
 
 def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
-    """Few launches of each kernel next to a copy of known size, for hardware-counter runs."""
+    """Three launches of each kernel next to a copy of known size, for hardware-counter runs (see --summarize-counters)."""
+    import workloads
+    from mase_hip import _lib
+
     dev = "cuda:0"
+    lib = _lib.load()
+    blib = load_bench_lib()
+    sp = _lib.stream_ptr(torch.device(dev))
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
     dst = torch.empty_like(src)
-    for _ in range(3):
-        dst.copy_(src)                                   # reads 256 MiB, writes 256 MiB
+    for _ in range(3):                                      # calibration: reads 256 MiB, writes 256 MiB
+        assert blib.mase_bench_stream_copy(src.data_ptr(), dst.data_ptr(), src.numel(), 1, sp) == 0
+    del src, dst
     M, K, N = 16384, 4096, 14336
     gen = torch.Generator(device=dev).manual_seed(3)
     x = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
@@ -362,11 +500,92 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
     a = mxk.quantize_dequantize(x.view(-1), fmt8, torch.bfloat16).view(M, K)
     for _ in range(3):
         mxk.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt8, None, M, N, K, torch.bfloat16)
-    w1 = w.view(-1)
+    del x, w, w_sc, w_el, a
+    for make, fmt in ((workloads.make_c1, fmt8), (workloads.make_c3, fmt4)):
+        t = make().reshape(-1).to(dev)
+        for _ in range(3):
+            sc, el = mxk.extract_mxfp_components(t, fmt)
+            mxk.compose_mxfp_tensor(sc, el, fmt, torch.bfloat16)
+        del t
+    x2 = workloads.make_c2().to(dev)
+    y2 = torch.empty_like(x2)
+    c2 = torch.empty(x2.numel(), dtype=torch.uint16, device=dev)
     for _ in range(3):
-        sc, el = mxk.extract_mxfp_components(w1, fmt4)
-        mxk.compose_mxfp_tensor(sc, el, fmt4, torch.bfloat16)
+        _lib.check(lib.mase_hip_qdq_minifloat(x2.data_ptr(), 0, y2.data_ptr(), 0, x2.numel(), 4, 3, 1, 0, sp))
+        _lib.check(lib.mase_hip_extract_minifloat(x2.data_ptr(), 0, c2.data_ptr(), x2.numel(), 4, 3, 1, 0, sp))
+        _lib.check(lib.mase_hip_compose_minifloat(c2.data_ptr(), y2.data_ptr(), 0, x2.numel(), 4, 3, 1, sp))
     torch.cuda.synchronize()
+
+
+# kernel-name fragments of the counter probe's launches ('a|b': both must occur; extract is MODE 0 of a kernel whose MODE 1 is
+# the fused QDQ) -> (key in the summary, algorithmic bytes read, written, sources)
+_N1, _N3, _N2 = 4096 * 4096, 14336 * 4096, 1 << 24
+COUNTER_ROWS = (
+    ("stream_copy_kernel", "calibration copy (256 MiB read, 256 MiB written)", 256 << 20, 256 << 20, None),
+    ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", 16384 * 4096 * 2 + 14336 * 4096 + 14336 * 128, 16384 * 14336 * 2, GEMM_SOURCES),
+    ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 0>(", "extract_mxfp C1", _N1 * 2, _N1 + _N1 // 32, CAST_SOURCES),
+    ("compose_mxfp_bf16_kernel<mase::SFmt<4, 3", "compose_mxfp C1", _N1 + _N1 // 32, _N1 * 2, CAST_SOURCES),
+    ("mxfp_bf16_b32_kernel<mase::SFmt<2, 1|, 0>(", "extract_mxfp C3", _N3 * 2, _N3 + _N3 // 32, CAST_SOURCES),
+    ("compose_mxfp_bf16_kernel<mase::SFmt<2, 1", "compose_mxfp C3", _N3 + _N3 // 32, _N3 * 2, CAST_SOURCES),
+    ("minifloat_f32_kernel<2", "qdq_minifloat_fused C2/E4M3", _N2 * 4, _N2 * 4, CAST_SOURCES),
+    ("minifloat_f32_kernel<0", "extract_minifloat C2/E4M3", _N2 * 4, _N2 * 2, CAST_SOURCES),
+    ("minifloat_f32_kernel<1", "compose_minifloat C2/E4M3", _N2 * 2, _N2 * 4, CAST_SOURCES),
+)
+
+
+def summarize_counters(fetch_dir, write_dir):
+    """Markdown summary (stdout) of the two rocprofv3 --pmc runs of `--counter-probe`: KiB per dispatch of FETCH_SIZE and
+    WRITE_SIZE for each kernel, scaled by what the same counters read for the calibration copy, next to the algorithmic
+    bytes; ends with the machine-readable block that the benchmark reads roofline.traffic from."""
+    import csv
+    import glob
+
+    csv.field_size_limit(1 << 30)
+
+    def per_kernel(folder, counter):
+        files = glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise SystemExit(f"no *counter_collection.csv under {folder}")
+        vals = {}
+        for r in csv.DictReader(open(files[0])):
+            if r["Counter_Name"] == counter:   # keyed by kernel name and launch size: the probe also extracts the GEMM's weight
+                vals.setdefault((r["Kernel_Name"], int(r["Grid_Size"])), []).append(float(r["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in vals.items()}
+
+    fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
+
+    def pick(table, frag, threads):
+        hits = [(k[0], v) for k, v in table.items() if all(part in k[0] for part in frag.split("|")) and (threads is None or k[1] == threads)]
+        if len(hits) != 1:
+            raise SystemExit(f"{len(hits)} launches match '{frag}' with {threads} threads: {[k[:80] for k, _ in hits]}")
+        return hits[0]
+
+    rows = []
+    for frag, key, rd, wr, sources in COUNTER_ROWS:
+        threads = {"extract_mxfp C1": _N1 // 8, "extract_mxfp C3": _N3 // 8}.get(key)   # one lane per 8 elements
+        (name, f_kib), (_, w_kib) = pick(fetch, frag, threads), pick(write, frag, threads)
+        rows.append((key, name, f_kib, w_kib, rd, wr, sources))
+    cal = rows[0]
+    f_fac, w_fac = (cal[4] / 1024) / cal[2], (cal[5] / 1024) / cal[3]
+    print("| kernel / workload | FETCH_SIZE (KiB) | WRITE_SIZE (KiB) | fetched (scaled) | written (scaled) | algorithmic read / write (KiB) | ratio |")
+    print("|---|---|---|---|---|---|---|")
+    table = {}
+    for key, name, f_kib, w_kib, rd, wr, sources in rows:
+        fs, ws = f_kib * f_fac, w_kib * w_fac
+        print(f"| {key} (`{name.split('(')[0][:70]}`) | {f_kib:.1f} | {w_kib:.1f} | {fs:.0f} KiB | {ws:.0f} KiB | {rd / 1024:.0f} / {wr / 1024:.0f} | "
+              f"{fs * 1024 / rd:.2f} / {ws * 1024 / wr:.2f} |")
+        if sources is not None:
+            table[key] = {"traffic_bytes": int((fs + ws) * 1024), "fetch_bytes": int(fs * 1024), "write_bytes": int(ws * 1024),
+                          "algorithmic_bytes": rd + wr, "sources": sources_fingerprint(sources)}
+    table["extract+compose_mxfp C1"] = {k: (table["extract_mxfp C1"][k] + table["compose_mxfp C1"][k]) if k != "sources" else table["extract_mxfp C1"][k]
+                                        for k in table["extract_mxfp C1"]}
+    table["extract+compose_mxfp C3"] = {k: (table["extract_mxfp C3"][k] + table["compose_mxfp C3"][k]) if k != "sources" else table["extract_mxfp C3"][k]
+                                        for k in table["extract_mxfp C3"]}
+    print(f"\nCalibration: the copy of known size gives the factors {f_fac:.3f} (FETCH_SIZE) and {w_fac:.3f} (WRITE_SIZE).\n")
+    print("Read by `bench.py` (`roofline.traffic`; `sources` = fingerprint of the kernel sources the counters were taken with):\n")
+    print("```json")
+    print(json.dumps(table, indent=1))
+    print("```")
 
 
 def bench_c5(torch, steps=20, warmup=8):
@@ -410,6 +629,9 @@ def bench_c5(torch, steps=20, warmup=8):
 
 def main():
     args = parse_args()
+    if args.summarize_counters:
+        summarize_counters(*args.summarize_counters)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this pool has a single MI355X and the path has no "
               "cross-GPU step; run with --gpus 1", file=sys.stderr)
@@ -452,8 +674,10 @@ def main():
                                "fp32 accumulate; step = fused QDQ kernel + dequant-fused GEMM kernel",
                    "M": M, "N": N, "K": K},
         "roofline": {"bound": "mfma", "achieved": round(lin["tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": GEMM_C4_TRAFFIC_BYTES,
+                     "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic_bytes("mxfp_gemm_tall_kernel C4", GEMM_SOURCES),
                      "kernel": "mxfp_gemm_tall_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4)},
+        "prewarm": dict(lin["prewarm"], note="uncounted steps before the counted warm-up, in groups of five until two groups agree "
+                                             "within 1 % (the shader clock settles over the first launches after idle)"),
         "context": {
             "separate_backend_ms_per_step": round(lin["separate_ms"], 4),
             "separate_backend_TFLOPs": round(2.0 * M * N * K / (lin["separate_ms"] * 1e-3) / 1e12, 2),
@@ -465,9 +689,7 @@ def main():
     }
     if not args.skip_hbm:
         result["context"]["c5_swiglu_mlp_block"] = bench_c5(torch)
-        result["hbm_kernels"] = bench_hbm(
-            torch, mxk, mfk,
-            lambda e, m: MXFPMeta(32, 8, e, m, True, "rn"), lambda e, m: MinifloatMeta(e, m, True, "rn"))
+        result["hbm_kernels"] = bench_hbm(torch, with_cpu=not args.no_cpu)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch)
     else:

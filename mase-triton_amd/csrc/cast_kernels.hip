@@ -7,6 +7,7 @@
 // lanes, which agree on the block maximum with xor-shuffles; one of them stores the scale byte.
 #include "../../include/mase_hip.h"
 #include "mase_host.h"
+#include "mxfp_compose.h"
 
 namespace mase {
 
@@ -212,6 +213,45 @@ __global__ __launch_bounds__(kThreads) void qdq_minifloat_kernel(const void* x, 
         }
     }
     if (has_tail) store_val_scalar<DT_OUT>(out, n_chunks * EPT + threadIdx.x, decode_f32(encode_f32_bits(tail_bits, f), f));
+}
+
+// fp32 sides.  With 8 consecutive elements per lane a lane's two 16-byte fp32 accesses are 32 bytes apart from its neighbour's, so
+// every load or store instruction of a wavefront covers 2 KB and uses half of it (the stores then reach memory as partial
+// lines: 1.10 x the output bytes measured).  Here a wavefront owns 512 consecutive elements and a lane two runs of four, 256
+// elements apart: every instruction covers one contiguous kilobyte on the fp32 side (512 bytes on the 16-bit side).
+// MODE 0: fp32 -> codes, 1: codes -> fp32, 2: fp32 -> fp32 (quantise-dequantise; `out` may alias `x`: a lane reads what it writes).
+// n must be a multiple of 512; the callers give the rest to the kernels above.
+template <int MODE, class F>
+__global__ __launch_bounds__(kThreads) void minifloat_f32_kernel(const void* x, void* out, int64_t n, F f) {
+    const int64_t wave_first = ((int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6)) * 512;
+    if (wave_first >= n) return;
+    const int lane = threadIdx.x & 63;
+    uint32_t code[8];
+    if (MODE == 1) {
+        const uint16_t* c = static_cast<const uint16_t*>(x) + wave_first + 4 * lane;
+        const uint2 a = ld64(c), b = ld64(c + 256);
+        const uint32_t w[4] = {a.x, a.y, b.x, b.y};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { code[2 * j] = w[j] & 0xFFFFu; code[2 * j + 1] = w[j] >> 16; }
+    } else {
+        const uint32_t* p = static_cast<const uint32_t*>(x) + wave_first + 4 * lane;
+        const uint4 a = ld128<MODE == 0>(p), b = ld128<MODE == 0>(p + 256);
+        const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) code[j] = encode_f32_bits(u[j], f);
+    }
+    if (MODE == 0) {
+        uint16_t* c = static_cast<uint16_t*>(out) + wave_first + 4 * lane;
+        st64(c, make_uint2(code[0] | (code[1] << 16), code[2] | (code[3] << 16)));
+        st64(c + 256, make_uint2(code[4] | (code[5] << 16), code[6] | (code[7] << 16)));
+    } else {
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = decode_f32(code[j], f);
+        float* o = static_cast<float*>(out) + wave_first + 4 * lane;
+        st128<MODE == 1>(o, make_uint4(f32_bits(y[0]), f32_bits(y[1]), f32_bits(y[2]), f32_bits(y[3])));
+        st128<MODE == 1>(o + 256, make_uint4(f32_bits(y[4]), f32_bits(y[5]), f32_bits(y[6]), f32_bits(y[7])));
+    }
 }
 
 // ------------------------------------------------------------------------------ MXFP
@@ -454,6 +494,55 @@ __global__ __launch_bounds__(kThreads) void compose_mxfp_kernel(const uint8_t* _
             for (int j = 0; j < EPT; ++j) y[j] = mxfp_value((w[r][j / 4] >> (8 * (j % 4))) & 0xFFu, s, f);
             store_vals<DT_OUT, EPT>(out, c * EPT, y);
         }
+    }
+}
+
+// does the format have a compile-time Composer that takes the hardware convert route?
+template <class F, bool STATIC = F::kStatic> struct HwCompose { static constexpr bool value = false; };
+template <class F> struct HwCompose<F, true> { static constexpr bool value = Composer<F>::HW; };
+
+// bf16 output, a preset format with at most four exponent bits: the hardware's scaled fp8 -> bf16 convert does a pair of
+// codes per instruction (Composer, mxfp_compose.h).  A lane owns 8 codes (one 64-bit load) of one block; lanes whose scale
+// the convert does not take (from Composer::SLOW_FROM up: 255, "times +inf", among them) redo theirs with the exact
+// per-element routine, behind a wave-uniform test.
+template <class F, int UNROLL>
+__global__ __launch_bounds__(kThreads) void compose_mxfp_bf16_kernel(const uint8_t* __restrict__ scales,
+                                                                      const uint8_t* __restrict__ elements, void* __restrict__ out,
+                                                                      int64_t n, int chunks_per_block, F f) {
+    typedef Composer<F> C;
+    constexpr uint32_t KEEP4 = ((1u << (1 + C::E + C::M)) - 1u) * 0x01010101u;   // the reference ignores the bits above the code
+    const int64_t n_chunks = n / 8;
+    const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint2 w[UNROLL];
+    uint32_t sc[UNROLL];
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        w[r] = make_uint2(0u, 0u);
+        sc[r] = 127u;
+        if (c < n_chunks) {
+            w[r] = ld64(elements + c * 8);
+            sc[r] = scales[c / chunks_per_block];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < UNROLL; ++r) {
+        const int64_t c = chunk0 + (int64_t)r * kThreads;
+        const uint32_t w0 = w[r].x & KEEP4, w1 = w[r].y & KEEP4;
+        const C cmp(sc[r]);
+        uint32_t o[4];
+        cmp.pair2(w0, o[0], o[1]);
+        cmp.pair2(w1, o[2], o[3]);
+        if (__builtin_amdgcn_ballot_w64(C::is_slow(sc[r])) != 0 && C::is_slow(sc[r])) {
+            const float s = scale_f32(sc[r]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t ww = j < 2 ? w0 : w1;
+                const int b0 = 16 * (j & 1);
+                o[j] = pack_bf16(mxfp_value((ww >> b0) & 0xFFu, s, f), mxfp_value((ww >> (b0 + 8)) & 0xFFu, s, f));
+            }
+        }
+        if (c < n_chunks) st128(static_cast<uint8_t*>(out) + c * 16, make_uint4(o[0], o[1], o[2], o[3]));
     }
 }
 
@@ -778,6 +867,18 @@ int mase_hip_extract_minifloat(const void* x, int x_dtype, uint16_t* codes, int6
     const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
         return dispatch_dtype(x_dtype, [&](auto dt) {
+            if constexpr (decltype(dt)::value == F32) {
+                // whole runs of 512 elements: the kernel whose fp32 accesses are contiguous over the wavefront; the rest below
+                const int64_t n_main = n & ~(int64_t)511;
+                if (n_main > 0) {
+                    hipLaunchKernelGGL((minifloat_f32_kernel<0, decltype(f)>), dim3(grid_for(n_main / 512, kThreads / 64)), dim3(kThreads), 0,
+                                       s, x, static_cast<void*>(codes), n_main, f);
+                    if (n_main == n) return check_launch("extract_minifloat");
+                    hipLaunchKernelGGL((extract_minifloat_kernel<F32, decltype(f), UNROLL>), dim3(1), dim3(kThreads), 0, s,
+                                       static_cast<const void*>(static_cast<const float*>(x) + n_main), codes + n_main, n - n_main, f);
+                    return check_launch("extract_minifloat");
+                }
+            }
             hipLaunchKernelGGL((extract_minifloat_kernel<decltype(dt)::value, decltype(f), UNROLL>), dim3(grid), dim3(kThreads), 0, s, x,
                                codes, n, f);
             return check_launch("extract_minifloat");
@@ -798,6 +899,17 @@ int mase_hip_compose_minifloat(const uint16_t* codes, void* out, int out_dtype, 
     const unsigned grid = grid_for(n / 8 + 1, UNROLL * kThreads);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, RN, [&](auto f) {
         return dispatch_dtype(out_dtype, [&](auto dt) {
+            if constexpr (decltype(dt)::value == F32) {
+                const int64_t n_main = n & ~(int64_t)511;
+                if (n_main > 0) {
+                    hipLaunchKernelGGL((minifloat_f32_kernel<1, decltype(f)>), dim3(grid_for(n_main / 512, kThreads / 64)), dim3(kThreads), 0,
+                                       s, static_cast<const void*>(codes), out, n_main, f);
+                    if (n_main == n) return check_launch("compose_minifloat");
+                    hipLaunchKernelGGL((compose_minifloat_kernel<F32, decltype(f), UNROLL>), dim3(1), dim3(kThreads), 0, s, codes + n_main,
+                                       static_cast<void*>(static_cast<float*>(out) + n_main), n - n_main, f);
+                    return check_launch("compose_minifloat");
+                }
+            }
             hipLaunchKernelGGL((compose_minifloat_kernel<decltype(dt)::value, decltype(f), UNROLL>), dim3(grid), dim3(kThreads), 0, s,
                                codes, out, n, f);
             return check_launch("compose_minifloat");
@@ -821,6 +933,18 @@ int mase_hip_qdq_minifloat(const void* x, int x_dtype, void* out, int out_dtype,
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
         return dispatch_dtype(x_dtype, [&](auto di) {
             return dispatch_dtype(out_dtype, [&](auto dout) {
+                if constexpr (decltype(di)::value == F32 && decltype(dout)::value == F32) {
+                    const int64_t n_main = n & ~(int64_t)511;
+                    if (n_main > 0) {
+                        hipLaunchKernelGGL((minifloat_f32_kernel<2, decltype(f)>), dim3(grid_for(n_main / 512, kThreads / 64)), dim3(kThreads),
+                                           0, s, x, out, n_main, f);
+                        if (n_main == n) return check_launch("qdq_minifloat");
+                        hipLaunchKernelGGL((qdq_minifloat_kernel<F32, F32, decltype(f), UNROLL>), dim3(1), dim3(kThreads), 0, s,
+                                           static_cast<const void*>(static_cast<const float*>(x) + n_main),
+                                           static_cast<void*>(static_cast<float*>(out) + n_main), n - n_main, f);
+                        return check_launch("qdq_minifloat");
+                    }
+                }
                 hipLaunchKernelGGL((qdq_minifloat_kernel<decltype(di)::value, decltype(dout)::value, decltype(f), UNROLL>), dim3(grid),
                                    dim3(kThreads), 0, s, x, out, n, f);
                 return check_launch("qdq_minifloat");
@@ -876,6 +1000,13 @@ int mase_hip_compose_mxfp(const uint8_t* scales, const uint8_t* elements, void* 
     return dispatch_fmt(exp_bits, frac_bits, is_finite, RN, [&](auto f) {
         return dispatch_dtype(out_dtype, [&](auto dt) {
             // 8 codes per lane: a wavefront then stores 1 KB contiguous per instruction (16 per lane would leave gaps)
+            if constexpr (decltype(dt)::value == BF16 && HwCompose<decltype(f)>::value) {
+                if (al && B % 8 == 0) {
+                    hipLaunchKernelGGL((compose_mxfp_bf16_kernel<decltype(f), UNROLL>), dim3(grid_for(n / 8, UNROLL * kThreads)),
+                                       dim3(kThreads), 0, s, scales, elements, out, n, B / 8, f);
+                    return check_launch("compose_mxfp");
+                }
+            }
             if (al && B % 8 == 0) {
                 hipLaunchKernelGGL((compose_mxfp_kernel<decltype(dt)::value, decltype(f), 8, UNROLL>),
                                    dim3(grid_for(n / 8, UNROLL * kThreads)), dim3(kThreads), 0, s, scales, elements, out, n, B / 8, f);
