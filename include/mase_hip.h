@@ -158,7 +158,12 @@ int mase_hip_unpack_codes(const uint8_t* packed, uint8_t* elements, int64_t n, i
  *
  *   A: either dense (a_dense != NULL, dtype a_dtype, row-major [M,K], NOT yet quantised: it is
  *      used as is), or MXFP components (a_dense == NULL; a_scales[M*K/block], a_elements[M*K],
- *      blocks along K).
+ *      blocks along K).  The dense form is the fast one: mxfp_linear quantises its activations to
+ *      bfloat16 with mase_hip_qdq_mxfp (exact: MXFP values have at most 4 significant bits) and
+ *      passes them dense, which lets every tile kernel stream A straight into LDS.  A in component
+ *      form is a compatibility path for callers that hold pre-quantised activations: it always
+ *      takes the general 256 x 256 tile kernel (about 0.7 of the dense form's rate on large
+ *      shapes) and is never split over K.
  *   W: MXFP components w_scales[N*K/block], w_elements[N*K], blocks along K, as produced by
  *      mase_hip_extract_mxfp on the row-major [N,K] weight.
  *   bias: NULL or bias[N] of dtype bias_dtype, added in fp32 before the output rounding.
@@ -203,6 +208,25 @@ int mase_hip_mxfp_gemm_ws(const void* a_dense, int a_dtype, const uint8_t* a_sca
                           int w_frac_bits, const void* bias, int bias_dtype, void* y,
                           int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
                           void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * `batches` products in one launch: y_b[M,N] = A_b[M,K] * W_b[N,K]^T for b = 0 .. batches-1, with A_b, the components of
+ * W_b and y_b lying a_batch_stride, w_batch_stride and y_batch_stride ELEMENTS after those of product b-1 (the scales
+ * of W_b: w_batch_stride / 32 bytes).  A stride of 0 shares that operand between all products (a_batch_stride = 0: one
+ * A against many weights; w_batch_stride = 0: equivalent to one product with batches * M rows when the A_b are
+ * contiguous).  A is dense bfloat16; no bias; K is never split (no workspace).  Strides must be multiples of 8 (A),
+ * 32 (W) and 16 bytes (y) so that every product's operands are aligned like the first one's; batches <= 65535.
+ * Replaces the torch.matmul over leading batch axes at the end of mxfp_matmul
+ *   src/mase_triton/mxfp/functional/matmul.py:24-35
+ * (with `other` already extracted along its second-to-last axis into [.., N, K] order by
+ * mase_hip_extract_mxfp_strided, and `input` quantised by mase_hip_qdq_mxfp); the reference's 4-D use is
+ * test/test_mxfp_functional.py:229-230.
+ */
+int mase_hip_mxfp_gemm_batched(const void* a_dense, int a_dtype, const uint8_t* w_scales,
+                               const uint8_t* w_elements, int w_exp_bits, int w_frac_bits, void* y,
+                               int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
+                               int64_t batches, int64_t a_batch_stride, int64_t w_batch_stride,
+                               int64_t y_batch_stride, void* stream);
 
 /*
  * The same product as mase_hip_mxfp_gemm_ws for callers that cannot allocate device memory at all (code under HIP

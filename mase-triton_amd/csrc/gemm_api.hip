@@ -9,7 +9,8 @@ extern "C" int64_t mase_hip_mxfp_gemm_workspace_bytes(int a_is_dense, int64_t M,
 static int gemm_entry(const void* a_dense, int a_dtype, const uint8_t* a_scales, const uint8_t* a_elements, int a_exp_bits,
                       int a_frac_bits, const uint8_t* w_scales, const uint8_t* w_elements, int w_exp_bits, int w_frac_bits,
                       const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
-                      void* workspace, int64_t workspace_bytes, void* stream) {
+                      void* workspace, int64_t workspace_bytes, void* stream, int64_t batches = 1, int64_t a_batch_stride = 0,
+                      int64_t w_batch_stride = 0, int64_t y_batch_stride = 0) {
     if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(ERR_INVALID, "M, N, K must fit in 31 bits");
     if (block_size != 32) return fail(ERR_UNSUPPORTED, "the GEMM supports block_size 32 only");
@@ -29,8 +30,21 @@ static int gemm_entry(const void* a_dense, int a_dtype, const uint8_t* a_scales,
     if (workspace_bytes < 0) return fail(ERR_INVALID, "workspace_bytes must not be negative");
     if (workspace && !aligned(workspace, 16)) return fail(ERR_INVALID, "workspace must be 16-byte aligned");
     if (!workspace) workspace_bytes = 0;
+    GemmBatch gb{0, 0, 0, 0};
+    if (batches != 1) {
+        if (batches < 1 || batches > 65535) return fail(ERR_INVALID, "batches must be between 1 and 65535");
+        if (!a_is_dense) return fail(ERR_UNSUPPORTED, "a batched product takes a dense A");
+        const int64_t ysz = dtype_size(out_dtype);
+        if (a_batch_stride != 0 && a_batch_stride < M * K) return fail(ERR_INVALID, "a_batch_stride must be 0 (A shared by every product) or at least M * K");
+        if (w_batch_stride != 0 && w_batch_stride < N * K) return fail(ERR_INVALID, "w_batch_stride must be 0 (W shared by every product) or at least N * K");
+        if (y_batch_stride < M * N) return fail(ERR_INVALID, "y_batch_stride must be at least M * N");
+        // every product's operands must be aligned like the first one's
+        if (a_batch_stride % 8 != 0 || w_batch_stride % 32 != 0 || (y_batch_stride * ysz) % 16 != 0)
+            return fail(ERR_INVALID, "batch strides must be multiples of 8 (A), 32 (W) and 16 bytes (y)");
+        gb = GemmBatch{a_batch_stride, w_batch_stride / 32, w_batch_stride, y_batch_stride * ysz};
+    }
     const GemmArgs g{a_dense, a_scales, a_elements, a_is_dense ? 0 : a_exp_bits, a_frac_bits, w_scales, w_elements, bias, bias_dtype,
-                     y, out_dtype, (int)M, (int)N, (int)K, workspace, workspace_bytes, static_cast<hipStream_t>(stream)};
+                     y, out_dtype, (int)M, (int)N, (int)K, workspace, workspace_bytes, static_cast<hipStream_t>(stream), (int)batches, gb};
     if (w_exp_bits == 4 && w_frac_bits == 3) return gemm_w_e4m3(g);
     if (w_exp_bits == 5 && w_frac_bits == 2) return gemm_w_e5m2(g);
     if (w_exp_bits == 2 && w_frac_bits == 3) return gemm_w_e2m3(g);
@@ -54,6 +68,15 @@ extern "C" int mase_hip_mxfp_gemm_ws(const void* a_dense, int a_dtype, const uin
                                      void* stream) {
     return gemm_entry(a_dense, a_dtype, a_scales, a_elements, a_exp_bits, a_frac_bits, w_scales, w_elements, w_exp_bits, w_frac_bits,
                       bias, bias_dtype, y, out_dtype, M, N, K, block_size, workspace, workspace_bytes, stream);
+}
+
+extern "C" int mase_hip_mxfp_gemm_batched(const void* a_dense, int a_dtype, const uint8_t* w_scales, const uint8_t* w_elements, int w_exp_bits,
+                                          int w_frac_bits, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
+                                          int64_t batches, int64_t a_batch_stride, int64_t w_batch_stride, int64_t y_batch_stride,
+                                          void* stream) {
+    if (!a_dense) return fail(ERR_INVALID, "a batched product takes a dense A");
+    return gemm_entry(a_dense, a_dtype, nullptr, nullptr, 0, 0, w_scales, w_elements, w_exp_bits, w_frac_bits, nullptr, 0, y, out_dtype, M, N,
+                      K, block_size, nullptr, 0, stream, batches, a_batch_stride, w_batch_stride, y_batch_stride);
 }
 
 // ---- the same product for callers that cannot allocate: the partial sums of the K split live in a static device array

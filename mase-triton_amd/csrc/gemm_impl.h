@@ -23,6 +23,12 @@ namespace mase {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// Offsets between consecutive products of a batched launch (grid plane z = product z): elements of A, bytes of the W
+// scales, of the W codes and of y.  All zero for a single product; an operand shared by every product has offset 0.
+struct GemmBatch {
+    int64_t a, ws, we, y;
+};
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which
 // would make every wave wait for its outstanding output stores; here those are meant to drain in
 // the background while the next tile starts.
@@ -71,10 +77,15 @@ constexpr int SLAB_BYTES = TM * ROW_BYTES;  // one operand, one buffer (TM == TN
 // A_MODE: 0 = dense bf16 A, 1 = MXFP A (format FA).  W is always MXFP (format FW).
 template <int A_MODE, class FA, class FW, int DT_OUT, bool GUARD_K>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ a_elements,
-    const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements, const void* __restrict__ bias,
-    int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
+    const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ a_elements,
+    const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0, const void* __restrict__ bias,
+    int bias_dtype, void* __restrict__ y0, int M, int N, int K, int tiles_m, int tiles_n, GemmBatch gb) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
+    const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
+    const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
+    const uint8_t* __restrict__ const w_elements = w_elements0 + (int64_t)blockIdx.z * gb.we;
+    void* __restrict__ const y = static_cast<uint8_t*>(y0) + (int64_t)blockIdx.z * gb.y;
     uint8_t* const lds_a = lds;                    // [2][TM][ROW_BYTES]
     uint8_t* const lds_w = lds + 2 * SLAB_BYTES;   // [2][TN][ROW_BYTES]
 
@@ -333,9 +344,14 @@ constexpr int S_STRIDE = SBK + 8;  // bf16 elements per tile row: 80 bytes
 
 template <int A_MODE, class FA, class FW, int DT_OUT>
 __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ a_elements,
-    const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements, const void* __restrict__ bias,
-    int bias_dtype, void* __restrict__ y, int M, int N, int K) {
+    const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ a_elements,
+    const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0, const void* __restrict__ bias,
+    int bias_dtype, void* __restrict__ y0, int M, int N, int K, GemmBatch gb) {
+    // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
+    const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
+    const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
+    const uint8_t* __restrict__ const w_elements = w_elements0 + (int64_t)blockIdx.z * gb.we;
+    void* __restrict__ const y = static_cast<uint8_t*>(y0) + (int64_t)blockIdx.z * gb.y;
     __shared__ __attribute__((aligned(16))) uint16_t lds_a[SBM * S_STRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t lds_w[SBN * S_STRIDE];
 
@@ -427,7 +443,9 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_small_kernel(
 template <int A_MODE, class FA, class FW, int DT_OUT>
 int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_elements, const uint8_t* w_scales,
                 const uint8_t* w_elements, const void* bias, int bias_dtype, void* y, int M, int N, int K, void* workspace,
-                int64_t workspace_bytes, hipStream_t s) {
+                int64_t workspace_bytes, int batches, const GemmBatch& gb, hipStream_t s) {
+    // batches > 1: the same product for `batches` operand sets, gb apart, in one launch (grid plane z = product z); dense A only,
+    // never split over K (the caller checks both)
     const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
     const int64_t big_tiles = (int64_t)tiles_m * tiles_n;
     // 256 x 256 tiles need enough of them to occupy the 256 CUs; smaller problems use 128 x 128
@@ -435,7 +453,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     const bool use_big = fits32 && (big_tiles >= 128 || (int64_t)M * N >= (int64_t)4096 * 4096);
     if constexpr (A_MODE == 0) {
         // few tiles and a long K: with a workspace, K is split over several workgroups per tile
-        if (workspace && K <= (1 << 23) && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
+        if (workspace && batches == 1 && K <= (1 << 23) && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0) {
             // (the 512 x 128 kernel reads four scale bytes at a time)
             const SplitPlan plan = plan_split_k(M, N, K, device_cu_count(), (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0);
             if (plan.splits > 1 && workspace_bytes >= plan.workspace_bytes(M, N))
@@ -447,9 +465,9 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         // (the 32-row kernel below has N / 32; measured better up to N = 12288 for M <= 16 and up to N = 8192 for M <= 64)
         if (M <= 64 && N % R16_N == 0 && N <= (M <= 16 ? 12288 : 8192) && K % 128 == 0 && K <= (1 << 24) &&
             (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 && (reinterpret_cast<uintptr_t>(w_elements) & 7) == 0) {
-            if (M <= 16) return launch_gemm_rows16<FW, DT_OUT, 1, 8>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
-            if (M <= 32) return launch_gemm_rows16<FW, DT_OUT, 2, 4>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
-            return launch_gemm_rows16<FW, DT_OUT, 4, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+            if (M <= 16) return launch_gemm_rows16<FW, DT_OUT, 1, 8>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, batches, gb, s);
+            if (M <= 32) return launch_gemm_rows16<FW, DT_OUT, 2, 4>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, batches, gb, s);
+            return launch_gemm_rows16<FW, DT_OUT, 4, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, batches, gb, s);
         }
     }
     if constexpr (A_MODE == 0) {
@@ -457,7 +475,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         // (K bound: both kernels address a row of A or W with a 32-bit byte offset from a per-workgroup base)
         if (M <= 128 && N % SK_N == 0 && K % SK_MAC == 0 && K <= (1 << 24) && (reinterpret_cast<uintptr_t>(a_dense) & 15) == 0 &&
             (reinterpret_cast<uintptr_t>(w_elements) & 15) == 0)
-            return launch_gemm_skinny<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+            return launch_gemm_skinny<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, batches, gb, s);
     }
     if constexpr (A_MODE == 0) {
         // More rows: three tile shapes.  The larger the tile the fewer instructions per MFMA (a composed W row serves more
@@ -471,7 +489,8 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         const bool mid_ok = reach && al && M > 128 && N % MD_N == 0 && K % MD_MAC == 0;
         const bool wide_ok = reach && al && M > 128 && N % WD_N == 0 && K % WD_K == 0;
         const bool tall_ok = reach && al && M >= UM && N % UN == 0 && K % UMAC == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 &&
-                             (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0 && (int64_t)((M + UM - 1) / UM) * (N / UN) < (1 << 30);
+                             (reinterpret_cast<uintptr_t>(w_scales) & 3) == 0 && (gb.ws & 3) == 0 &&
+                             (int64_t)((M + UM - 1) / UM) * (N / UN) < (1 << 30);
         if (mid_ok || wide_ok || tall_ok) {
             const int cus = device_cu_count();
             if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
@@ -485,8 +504,8 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             if (mid_ok) { pick = 0; best = cost(MD_M, 1.0); }
             if (wide_ok) { const double c = cost(WD_M, 1.4); if (pick < 0 || c <= best) { pick = 1; best = c; } }
             if (tall_ok) { const double c = cost(UM, 2.05); if (pick < 0 || c <= best) { pick = 2; best = c; } }
-            if (pick == 0) return launch_gemm_mid<FW, DT_OUT, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
-            if (pick == 1) return launch_gemm_wide<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, s);
+            if (pick == 0) return launch_gemm_mid<FW, DT_OUT, 2>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, batches, gb, s);
+            if (pick == 1) return launch_gemm_wide<FW, DT_OUT>(a_dense, w_scales, w_elements, bias, bias_dtype, y, M, N, K, batches, gb, s);
             const int tall_tiles_m = (M + UM - 1) / UM;
             const int64_t tall_tiles = (int64_t)tall_tiles_m * (N / UN);
             const bool sc4 = K % 512 == 0;
@@ -495,8 +514,8 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed[sc4])) return rc;
             // one persistent workgroup per CU (a multiple of the 8 XCDs), never more than tiles
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
-            hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                               w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN, 1, (int64_t)0);
+            hipLaunchKernelGGL(kern, dim3(grid, 1u, (unsigned)batches), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense),
+                               w_scales, w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN, 1, (int64_t)0, gb);
             return check_launch("mxfp_gemm");
         }
     }
@@ -511,14 +530,14 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
         // one persistent workgroup per CU (rounded down to a multiple of 8 XCD slots), never more than tiles
         const int64_t want = big_tiles < n_cus ? ((big_tiles + 7) / 8) * 8 : (n_cus / 8) * 8;
         const unsigned grid = (unsigned)want;
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), a_scales,
-                           a_elements, w_scales, w_elements, bias, bias_dtype, y, M, N, K, tiles_m, tiles_n);
+        hipLaunchKernelGGL(kern, dim3(grid, 1u, (unsigned)batches), dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), a_scales,
+                           a_elements, w_scales, w_elements, bias, bias_dtype, y, M, N, K, tiles_m, tiles_n, gb);
     } else {
-        const dim3 grid((unsigned)((N + SBN - 1) / SBN), (unsigned)((M + SBM - 1) / SBM));
+        const dim3 grid((unsigned)((N + SBN - 1) / SBN), (unsigned)((M + SBM - 1) / SBM), (unsigned)batches);
         if (grid.y > 65535u) return fail(ERR_UNSUPPORTED, "M too large for the launch grid");
         hipLaunchKernelGGL((mxfp_gemm_small_kernel<A_MODE, FA, FW, DT_OUT>), grid, dim3(kGemmThreads), 0, s,
                            static_cast<const uint16_t*>(a_dense), a_scales, a_elements, w_scales, w_elements, bias, bias_dtype, y, M,
-                           N, K);
+                           N, K, gb);
     }
     return check_launch("mxfp_gemm");
 }
@@ -530,6 +549,7 @@ struct GemmArgs {
     const void* a_dense; const uint8_t* a_scales; const uint8_t* a_elements; int a_exp_bits, a_frac_bits;
     const uint8_t* w_scales; const uint8_t* w_elements; const void* bias; int bias_dtype; void* y; int out_dtype;
     int M, N, K; void* workspace; int64_t workspace_bytes; hipStream_t stream;
+    int batches; GemmBatch batch;   // batches > 1: one launch for that many products, operands `batch` apart (dense A only)
 };
 int gemm_w_e4m3(const GemmArgs& g);
 int gemm_w_e5m2(const GemmArgs& g);
@@ -543,12 +563,12 @@ int gemm_for_weight_format(const GemmArgs& g) {
         constexpr int DO = decltype(dout)::value;
         if (g.a_dense)
             return launch_gemm<0, SFmt<4, 3>, FW, DO>(g.a_dense, nullptr, nullptr, g.w_scales, g.w_elements, g.bias, g.bias_dtype, g.y,
-                                                      g.M, g.N, g.K, g.workspace, g.workspace_bytes, g.stream);
+                                                      g.M, g.N, g.K, g.workspace, g.workspace_bytes, g.batches, g.batch, g.stream);
         const int E = g.a_exp_bits, M = g.a_frac_bits;
 #define MASE_A_FMT(e, m)                                                                                                       \
         if (E == e && M == m)                                                                                                  \
             return launch_gemm<1, SFmt<e, m>, FW, DO>(nullptr, g.a_scales, g.a_elements, g.w_scales, g.w_elements, g.bias,     \
-                                                      g.bias_dtype, g.y, g.M, g.N, g.K, nullptr, 0, g.stream);
+                                                      g.bias_dtype, g.y, g.M, g.N, g.K, nullptr, 0, 1, GemmBatch{0, 0, 0, 0}, g.stream);
         MASE_A_FMT(4, 3) MASE_A_FMT(5, 2) MASE_A_FMT(2, 3) MASE_A_FMT(3, 2) MASE_A_FMT(2, 1)
 #undef MASE_A_FMT
         return fail(ERR_INVALID, "MXFP element (exp_bits, frac_bits) must be one of (4,3) (5,2) (2,3) (3,2) (2,1)");

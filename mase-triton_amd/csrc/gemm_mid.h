@@ -31,9 +31,13 @@ constexpr int MD_LDS_BYTES = MD_A_STAGES * MD_A_STAGE + 2 * MD_W_STAGE;  // 160 
 
 template <class FW, int DT_OUT, int KS>
 __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
+    const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ y_all, int M, int N, int K, int tiles_m, int k_len,
-    int64_t y_split_bytes) {
+    int64_t y_split_bytes, GemmBatch gb) {
+    // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
+    const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
+    const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
+    const uint8_t* __restrict__ const w_elements = w_elements0 + (int64_t)blockIdx.z * gb.we;
     constexpr int WAVES = 4 * KS, QW = 8 / KS;             // 16-k steps per wavefront and macro step
     constexpr int A_DMAS = MD_A_STAGE / 1024 / WAVES;      // per wavefront and macro step
     constexpr int W_LOADS = MD_N * MD_MAC / 16 / (64 * WAVES);  // code loads (and as many scale loads) per lane
@@ -58,7 +62,7 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
     const int kblocks = K / 32, nmac = min(k_len, K - k_begin) / MD_MAC;
     // 64-bit base of the tile's first row (and the split's first k): the per-lane offsets below stay within the tile's rows
     const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)m0 * K + k_begin) * 2;
-    void* const y = static_cast<uint8_t*>(y_all) + (size_t)blockIdx.y * (size_t)y_split_bytes;
+    void* const y = static_cast<uint8_t*>(y_all) + (size_t)blockIdx.y * (size_t)y_split_bytes + (int64_t)blockIdx.z * gb.y;
 
     // A DMA: an instruction moves 1 KB = 4 rows; lane l fills position l % 16 of row 4 (8 w + j) + l / 16, which must
     // hold chunk (l % 16) ^ (row & 15).  Rows past M re-read row M - 1 (their products are never stored).
@@ -278,14 +282,14 @@ __global__ __launch_bounds__(256 * KS) void mxfp_gemm_mid_kernel(
 
 template <class FW, int DT_OUT, int KS>
 int launch_gemm_mid(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
-                    void* y, int M, int N, int K, hipStream_t s) {
+                    void* y, int M, int N, int K, int batches, const GemmBatch& gb, hipStream_t s) {
     auto kern = mxfp_gemm_mid_kernel<FW, DT_OUT, KS>;
     static std::atomic<uint64_t> lds_allowed{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), MD_LDS_BYTES, lds_allowed)) return rc;
     const int tiles_m = (M + MD_M - 1) / MD_M;
     const int64_t tiles = (int64_t)tiles_m * (N / MD_N);
     if (tiles > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "too many tiles for one launch");
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(256 * KS), MD_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                       w_elements, bias, bias_dtype, y, M, N, K, tiles_m, K, (int64_t)0);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1u, (unsigned)batches), dim3(256 * KS), MD_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense),
+                       w_scales, w_elements, bias, bias_dtype, y, M, N, K, tiles_m, K, (int64_t)0, gb);
     return check_launch("mxfp_gemm");
 }

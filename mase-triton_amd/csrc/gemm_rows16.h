@@ -35,8 +35,13 @@ __device__ inline void wait_vmcnt8(u32x2& a, uint32_t& b) {
 // MT = 16-row tiles of A (M <= 16 MT), D = look-ahead in macro steps
 template <class FW, int DT_OUT, int MT, int D>
 __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_rows16_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K) {
+    const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y0, int M, int N, int K, GemmBatch gb) {
+    // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
+    const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
+    const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
+    const uint8_t* __restrict__ const w_elements = w_elements0 + (int64_t)blockIdx.z * gb.we;
+    void* __restrict__ const y = static_cast<uint8_t*>(y0) + (int64_t)blockIdx.z * gb.y;
     constexpr int KM = 128, ROW = 2 * KM;
     constexpr int R = D + 1;                       // ring size: register sets of W, LDS stages of A
     constexpr int A_DMAS = MT;                     // per wavefront and macro step: 16 MT rows x 256 B / 1 KB / 4
@@ -176,12 +181,12 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_rows16_kernel(
 
 template <class FW, int DT_OUT, int MT, int D>
 int launch_gemm_rows16(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
-                       void* y, int M, int N, int K, hipStream_t s) {
+                       void* y, int M, int N, int K, int batches, const GemmBatch& gb, hipStream_t s) {
     constexpr int lds_bytes = (D + 1) * 16 * MT * 256 + 2 * R16_N * 256;  // >= the 3 MT KB the final reduction needs
     auto kern = mxfp_gemm_rows16_kernel<FW, DT_OUT, MT, D>;
     static std::atomic<uint64_t> lds_allowed{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed)) return rc;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(N / R16_N)), dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                       w_elements, bias, bias_dtype, y, M, N, K);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(N / R16_N), 1u, (unsigned)batches), dim3(kGemmThreads), lds_bytes, s,
+                       static_cast<const uint16_t*>(a_dense), w_scales, w_elements, bias, bias_dtype, y, M, N, K, gb);
     return check_launch("mxfp_gemm");
 }

@@ -23,8 +23,13 @@ constexpr int SK_MAC = 128;     // k granularity the launcher requires
 
 template <class FW, int DT_OUT, int MT, int D, int L, int AR>
 __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K) {
+    const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y0, int M, int N, int K, GemmBatch gb) {
+    // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
+    const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
+    const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
+    const uint8_t* __restrict__ const w_elements = w_elements0 + (int64_t)blockIdx.z * gb.we;
+    void* __restrict__ const y = static_cast<uint8_t*>(y0) + (int64_t)blockIdx.z * gb.y;
     // L = 128-byte lines of W codes per row and macro step: the macro step covers KM = 128 L k, LDS rows are 256 L bytes
     // AR = rows of A kept per m-tile: 32, or 16 when M <= 16 (rows 16..31 of the MFMA operand then re-read rows 0..15)
     static_assert(AR == 32 || (AR == 16 && MT == 1), "16-row stages only with one m-tile");
@@ -204,8 +209,8 @@ __global__ __launch_bounds__(kGemmThreads) void mxfp_gemm_skinny_kernel(
 
 template <class FW, int DT_OUT>
 int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
-                       void* y, int M, int N, int K, hipStream_t s) {
-    const dim3 grid((unsigned)(N / SK_N));
+                       void* y, int M, int N, int K, int batches, const GemmBatch& gb, hipStream_t s) {
+    const dim3 grid((unsigned)(N / SK_N), 1u, (unsigned)batches);
     auto go = [&](auto mt_c, auto d_c) {
         constexpr int MT = decltype(mt_c)::value, D = decltype(d_c)::value, L = 1, AR = 32;
         constexpr int lds_bytes = (D + 1) * AR * MT * 256 * L + 2 * SK_N * 256 * L;
@@ -213,7 +218,7 @@ int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8
         static std::atomic<uint64_t> lds_allowed{0};
         if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed)) return rc;
         hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
-                           bias, bias_dtype, y, M, N, K);
+                           bias, bias_dtype, y, M, N, K, gb);
         return check_launch("mxfp_gemm");
     };
     if (M <= 16) {  // 16-row A stages leave LDS for a look-ahead of 8 macro steps
@@ -223,7 +228,7 @@ int launch_gemm_skinny(const void* a_dense, const uint8_t* w_scales, const uint8
         static std::atomic<uint64_t> lds_allowed{0};
         if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed)) return rc;
         hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), lds_bytes, s, static_cast<const uint16_t*>(a_dense), w_scales, w_elements,
-                           bias, bias_dtype, y, M, N, K);
+                           bias, bias_dtype, y, M, N, K, gb);
         return check_launch("mxfp_gemm");
     }
     // Look-ahead in macro steps.  With more workgroups than CUs the A stages must leave LDS for two workgroups per CU, which

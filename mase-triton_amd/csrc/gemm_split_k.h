@@ -101,7 +101,7 @@ int launch_gemm_split_k(const void* a_dense, const uint8_t* w_scales, const uint
         const int tiles_m = (M + MD_M - 1) / MD_M;
         hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * (N / MD_N)), (unsigned)plan.splits), dim3(512), MD_LDS_BYTES, s,
                            static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
-                           M, N, K, tiles_m, plan.k_len, mn * 4);
+                           M, N, K, tiles_m, plan.k_len, mn * 4, GemmBatch{0, 0, 0, 0});
     } else if (plan.kind == 1) {
         auto kern = mxfp_gemm_wide_kernel<FW, F32>;
         static std::atomic<uint64_t> lds_allowed{0};
@@ -109,7 +109,7 @@ int launch_gemm_split_k(const void* a_dense, const uint8_t* w_scales, const uint
         const int tiles_m = (M + WD_M - 1) / WD_M;
         hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * (N / WD_N)), (unsigned)plan.splits), dim3(WD_THREADS), WD_LDS_BYTES, s,
                            static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
-                           M, N, K, tiles_m, plan.k_len, mn * 4);
+                           M, N, K, tiles_m, plan.k_len, mn * 4, GemmBatch{0, 0, 0, 0});
     } else {
         const bool sc4 = plan.k_len % 512 == 0;
         auto kern = sc4 ? mxfp_gemm_tall_kernel<FW, F32, true> : mxfp_gemm_tall_kernel<FW, F32, false>;
@@ -119,7 +119,7 @@ int launch_gemm_split_k(const void* a_dense, const uint8_t* w_scales, const uint
         const int walks = tiles_m * (N / UN) * plan.splits;          // at most one per CU (the plan splits only then)
         hipLaunchKernelGGL(kern, dim3((unsigned)((walks + 7) / 8 * 8)), dim3(kGemmThreads), U_LDS_BYTES, s,
                            static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
-                           M, N, K, tiles_m, N / UN, plan.splits, mn * 4);
+                           M, N, K, tiles_m, N / UN, plan.splits, mn * 4, GemmBatch{0, 0, 0, 0});
     }
     if (int rc = check_launch("mxfp_gemm")) return rc;
     hipLaunchKernelGGL(split_k_reduce_kernel<DT_OUT>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s,

@@ -120,8 +120,14 @@ struct TallTile {
 // (a load of 4 bytes per row touches as many cache lines, one per row, and the address unit's time goes by lines)
 template <class FW, int DT_OUT, bool SC4>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_tall_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, int splits, int64_t y_split_bytes) {
+    const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y0, int M, int N, int K, int tiles_m, int tiles_n, int splits, int64_t y_split_bytes,
+    GemmBatch gb) {
+    // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
+    const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
+    const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
+    const uint8_t* __restrict__ const w_elements = w_elements0 + (int64_t)blockIdx.z * gb.we;
+    void* __restrict__ const y = static_cast<uint8_t*>(y0) + (int64_t)blockIdx.z * gb.y;
     // splits > 1: every tile is walked `splits` times, each time over K / splits of k and into its own [M, N] output array
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;

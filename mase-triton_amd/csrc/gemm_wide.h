@@ -23,8 +23,13 @@ constexpr int WD_THREADS = 512;
 
 template <class FW, int DT_OUT>
 __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
-    const uint16_t* __restrict__ a_dense, const uint8_t* __restrict__ w_scales, const uint8_t* __restrict__ w_elements,
-    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y_all, int M, int N, int K, int tiles_m, int k_len, int64_t y_split_bytes) {
+    const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0,
+    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y_all, int M, int N, int K, int tiles_m, int k_len, int64_t y_split_bytes,
+    GemmBatch gb) {
+    // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
+    const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
+    const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
+    const uint8_t* __restrict__ const w_elements = w_elements0 + (int64_t)blockIdx.z * gb.we;
     constexpr int A_DMAS = WD_A_STAGE / 1024 / 8;          // 4 per wavefront and step
     constexpr int OPS = A_DMAS + 2;                        // vector-memory operations per wavefront and step
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -45,7 +50,7 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
     // and writes its sums to its own [M, N] array, y_split_bytes apart.  One split: k_len = K.
     const int k_begin = (int)blockIdx.y * k_len;
     const int kblocks = K / 32, nsteps = min(k_len, K - k_begin) / WD_K;
-    void* const y = static_cast<uint8_t*>(y_all) + (size_t)blockIdx.y * (size_t)y_split_bytes;
+    void* const y = static_cast<uint8_t*>(y_all) + (size_t)blockIdx.y * (size_t)y_split_bytes + (int64_t)blockIdx.z * gb.y;
     // 64-bit base of the tile's first row (and the split's first k): the per-lane offsets below stay within the tile's rows
     const uint8_t* const a_tile = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)m0 * K + k_begin) * 2;
 
@@ -220,14 +225,14 @@ __global__ __launch_bounds__(WD_THREADS) void mxfp_gemm_wide_kernel(
 
 template <class FW, int DT_OUT>
 int launch_gemm_wide(const void* a_dense, const uint8_t* w_scales, const uint8_t* w_elements, const void* bias, int bias_dtype,
-                     void* y, int M, int N, int K, hipStream_t s) {
+                     void* y, int M, int N, int K, int batches, const GemmBatch& gb, hipStream_t s) {
     auto kern = mxfp_gemm_wide_kernel<FW, DT_OUT>;
     static std::atomic<uint64_t> lds_allowed{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), WD_LDS_BYTES, lds_allowed)) return rc;
     const int tiles_m = (M + WD_M - 1) / WD_M;
     const int64_t tiles = (int64_t)tiles_m * (N / WD_N);
     if (tiles > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "too many tiles for one launch");
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(WD_THREADS), WD_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), w_scales,
-                       w_elements, bias, bias_dtype, y, M, N, K, tiles_m, K, (int64_t)0);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1u, (unsigned)batches), dim3(WD_THREADS), WD_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense),
+                       w_scales, w_elements, bias, bias_dtype, y, M, N, K, tiles_m, K, (int64_t)0, gb);
     return check_launch("mxfp_gemm");
 }

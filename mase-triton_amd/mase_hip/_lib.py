@@ -32,6 +32,8 @@ SIGNATURES = {
     "mase_hip_mxfp_gemm_ws": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
                                      _vp, _i32, _i64, _i64, _i64, _i32, _vp, _i64, _vp]),
     "mase_hip_mxfp_gemm_workspace_bytes": (_i64, [_i32, _i64, _i64, _i64]),
+    "mase_hip_mxfp_gemm_batched": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _i32, _i64, _i64, _i64, _i32,
+                                          _i64, _i64, _i64, _i64, _vp]),
     "mase_hip_mxfp_gemm_static_ws": (_i32, [_vp, _i32, _vp, _vp, _i32, _i32, _vp, _vp, _i32, _i32, _vp, _i32,
                                             _vp, _i32, _i64, _i64, _i64, _i32, _vp]),
 }
@@ -113,10 +115,22 @@ def on_device(device: torch.device):
     return torch.cuda.device(device)
 
 
+# how often dense() had to copy an operand because its storage was not 16-byte aligned (a full extra pass over it)
+realignment_copies = 0
+
+
 def dense(t: torch.Tensor) -> torch.Tensor:
-    """Contiguous and 16-byte aligned (what the vector kernels assume)."""
+    """Contiguous and 16-byte aligned (what the vector kernels assume).  A misaligned operand (a view that starts at an odd
+    offset of its storage) is copied: counted in ``realignment_copies``, and the first one is reported with a warning."""
+    global realignment_copies
     t = t.contiguous()
     if t.data_ptr() % 16:
+        if realignment_copies == 0:
+            import warnings
+
+            warnings.warn("mase_hip: an operand is not 16-byte aligned and is copied before the kernel runs (further copies are "
+                          "counted in mase_hip._lib.realignment_copies without a warning)", RuntimeWarning, stacklevel=3)
+        realignment_copies += 1
         t = t.clone()
     return t
 

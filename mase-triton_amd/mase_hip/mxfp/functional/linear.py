@@ -47,6 +47,8 @@ def _gemm_eligible(x: Tensor, quantised_x: bool, w_tensor_meta: MXFPTensorMeta, 
     activations, so a dense X must already be bf16."""
     if x.device.type != "cuda" or w_tensor_meta.meta.block_size != 32 or len(w_tensor_meta.shape) != 2:
         return False
+    if not w_tensor_meta.meta.element_is_finite:
+        return False  # the GEMM decodes the top exponent field as an ordinary binade, this format reads it as inf / NaN
     if w_tensor_meta.block_dim % 2 != 1 or w_tensor_meta.shape[1] % 32 != 0:
         return False
     if x.dtype not in _GEMM_DTYPES or getattr(torch, w_tensor_meta.dtype) != x.dtype:

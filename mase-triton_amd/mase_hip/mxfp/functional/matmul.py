@@ -5,11 +5,11 @@ contraction axis of both).
 backend="separate" follows the reference: extract + compose each quantised operand, then
 ``torch.matmul``.
 backend="fused" (NotImplementedError in the reference, :21-22) quantises ``other`` in place
-along its second-to-last axis (no transposed copy).  When ``other`` is quantised and either is a
-matrix or has the batch shape of ``input`` with few batches, it stays in MXFP form: its codes
-come out as [.., N, K], the layout the GEMM kernels read, and each batch is one GEMM launch that
-composes the codes to bf16 on their way to the MFMA units.  Everything else goes through the
-one-pass quantise-dequantise kernels and ``torch.matmul``.
+along its second-to-last axis (no transposed copy).  When ``other`` is quantised it stays in MXFP
+form: its codes come out as [.., N, K], the layout the GEMM kernels read, and all leading batch
+axes (broadcast ones included) go into ONE batched GEMM launch that composes the codes to bf16
+on their way to the MFMA units.  Everything else goes through the one-pass quantise-dequantise
+kernels and ``torch.matmul``.
 """
 from __future__ import annotations
 
@@ -22,9 +22,6 @@ from .. import kernels
 from ..meta import MXFPMeta
 from .cast import compose_mxfp_tensor, extract_mxfp_components, quantize_dequantize
 
-# more batches than this and one batched dense GEMM beats a launch per batch
-_MAX_GEMM_BATCHES = 16
-
 
 def _gemm_route(input: Tensor, other: Tensor, quantised_input: bool, other_meta: MXFPMeta) -> bool:
     if input.device.type != "cuda" or other.device != input.device or input.ndim < 2 or other.ndim < 2:
@@ -35,35 +32,63 @@ def _gemm_route(input: Tensor, other: Tensor, quantised_input: bool, other_meta:
         return False  # the MFMA path would round a dense fp32 operand to bf16
     if input.shape[-1] != other.shape[-2] or input.numel() == 0 or other.numel() == 0:
         return False
-    if not kernels.strided_blocks_supported(tuple(other.shape), -2, other_meta):
+    if not kernels.strided_blocks_supported(tuple(other.shape), -2, other_meta) or not other_meta.element_is_finite:
         return False
     if other.ndim == 2:
         return True
-    batches = 1
-    for d in other.shape[:-2]:
-        batches *= d
-    return tuple(other.shape[:-2]) == tuple(input.shape[:-2]) and batches <= _MAX_GEMM_BATCHES
+    try:
+        torch.broadcast_shapes(tuple(input.shape[:-2]), tuple(other.shape[:-2]))
+    except RuntimeError:
+        return False
+    M, N = input.shape[-2], other.shape[-1]
+    return (M * N * input.element_size()) % 16 == 0       # every product's output 16-byte aligned
+
+
+def _prod(shape) -> int:
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+def gemm_over_batches(a: Tensor, w_scales: Tensor, w_elements: Tensor, w_meta: MXFPMeta, w_batch: tuple, N: int,
+                      output_dtype: torch.dtype) -> Tensor:
+    """``a [*bi, M, K]`` (dense bfloat16, contiguous) against weights held as components in [*w_batch, N, K] order: one GEMM
+    when the weight is a matrix, else ONE batched launch over the broadcast of the two batch shapes."""
+    K = a.shape[-1]
+    if len(w_batch) == 0:
+        y = kernels.mxfp_gemm(a.view(-1, K), None, None, None, w_scales, w_elements, w_meta, None, a.numel() // K, N, K, output_dtype)
+        return y.view(*a.shape[:-1], N)
+    M = a.shape[-2]
+    bi, bo = tuple(a.shape[:-2]), tuple(w_batch)
+    batch = tuple(torch.broadcast_shapes(bi, bo))
+    # an operand whose batch axes are all 1 is shared through a zero stride; one that is broadcast along some axes only
+    # is expanded (a copy of that operand)
+    if _prod(bi) == 1:
+        a_stride = 0
+    else:
+        if bi != batch:
+            a = a.expand(*batch, M, K).contiguous()
+        a_stride = M * K
+    if _prod(bo) == 1:
+        w_stride = 0
+    else:
+        if bo != batch:
+            w_scales = w_scales.view(*bo, N * K // 32).expand(*batch, N * K // 32).contiguous()
+            w_elements = w_elements.view(*bo, N * K).expand(*batch, N * K).contiguous()
+        w_stride = N * K
+    y = kernels.mxfp_gemm_batched(a.reshape(-1), w_scales.reshape(-1), w_elements.reshape(-1), w_meta, _prod(batch), M, N, K,
+                                  output_dtype, a_stride, w_stride)
+    return y.view(*batch, M, N)
 
 
 def _matmul_through_gemm(input: Tensor, other: Tensor, input_meta: MXFPMeta | None, other_meta: MXFPMeta) -> Tensor:
-    K, N = other.shape[-2], other.shape[-1]
     a = input
     if input_meta is not None:
         # MXFP values are exact in bf16 whatever input.dtype is
         a = quantize_dequantize(input, block_dim=-1, mxfp_meta=input_meta, output_dtype=torch.bfloat16)
-    a = a.contiguous()
     w_scales, w_elements = kernels.extract_mxfp_components_strided(other, -2, other_meta)  # [.., N, K] order
-    if other.ndim == 2:
-        y = kernels.mxfp_gemm(a.view(-1, K), None, None, None, w_scales, w_elements, other_meta, None,
-                              a.numel() // K, N, K, input.dtype)
-        return y.view(*input.shape[:-1], N)
-    M = input.shape[-2]
-    y = torch.empty(*input.shape[:-1], N, dtype=input.dtype, device=input.device)
-    a3, y3 = a.view(-1, M, K), y.view(-1, M, N)
-    sc3, el3 = w_scales.view(-1, N * K // 32), w_elements.view(-1, N * K)
-    for b in range(a3.shape[0]):
-        kernels.mxfp_gemm(a3[b], None, None, None, sc3[b], el3[b], other_meta, None, M, N, K, input.dtype, out=y3[b])
-    return y
+    return gemm_over_batches(a.contiguous(), w_scales, w_elements, other_meta, tuple(other.shape[:-2]), other.shape[-1], input.dtype)
 
 
 def mxfp_matmul(

@@ -158,6 +158,7 @@ def mxfp_gemm(
     _lib.require_gpu(w_elements, "w_elements")
     assert w_scales.dtype == torch.uint8 and w_elements.dtype == torch.uint8
     assert w_meta.block_size == 32 and K % 32 == 0
+    assert w_meta.element_is_finite, "the GEMM decodes finite-only element formats (the top exponent field is an ordinary binade)"
     assert w_elements.numel() == N * K and w_scales.numel() == N * K // 32
     w_scales, w_elements = _lib.dense(w_scales), _lib.dense(w_elements)
     a_ptr = a_sc_ptr = a_el_ptr = None
@@ -192,4 +193,32 @@ def mxfp_gemm(
             a_ptr, a_dt, a_sc_ptr, a_el_ptr, a_e, a_m, w_scales.data_ptr(), w_elements.data_ptr(),
             w_meta.element_exp_bits, w_meta.element_frac_bits, b_ptr, b_dt, y.data_ptr(),
             _lib.dtype_code(output_dtype), M, N, K, 32, None if ws is None else ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
+    return y
+
+
+def mxfp_gemm_batched(a: Tensor, w_scales: Tensor, w_elements: Tensor, w_meta: MXFPMeta, batches: int, M: int, N: int, K: int,
+                      output_dtype: torch.dtype, a_batch_stride: int, w_batch_stride: int) -> Tensor:
+    """``batches`` products y[b] = A[b] @ W[b]^T in one launch.  ``a`` holds the dense bfloat16 A operands
+    ``a_batch_stride`` elements apart, the components hold the weights ``w_batch_stride`` elements apart (blocks along
+    K); a stride of 0 shares the operand between all products.  Returns y [batches, M, N]."""
+    dev = w_elements.device
+    _lib.require_gpu(w_elements, "w_elements")
+    _lib.require_gpu(a, "activations")
+    assert a.dtype == torch.bfloat16 and w_scales.dtype == torch.uint8 and w_elements.dtype == torch.uint8
+    assert w_meta.block_size == 32 and K % 32 == 0
+    assert w_meta.element_is_finite, "the GEMM decodes finite-only element formats (the top exponent field is an ordinary binade)"
+    a, w_scales, w_elements = _lib.dense(a), _lib.dense(w_scales), _lib.dense(w_elements)
+    assert a.numel() >= (batches - 1) * a_batch_stride + M * K
+    assert w_elements.numel() >= (batches - 1) * w_batch_stride + N * K
+    y = torch.empty((batches, M, N), dtype=output_dtype, device=dev)
+    lib = _lib.load()
+    with _lib.on_device(dev):
+        for first in range(0, batches, 65535):      # one launch takes at most 65535 products
+            count = min(65535, batches - first)
+            esz = 2
+            _lib.check(lib.mase_hip_mxfp_gemm_batched(
+                a.data_ptr() + first * a_batch_stride * esz, _lib.dtype_code(a.dtype),
+                w_scales.data_ptr() + first * (w_batch_stride // 32), w_elements.data_ptr() + first * w_batch_stride,
+                w_meta.element_exp_bits, w_meta.element_frac_bits, y[first].data_ptr(), _lib.dtype_code(output_dtype),
+                M, N, K, 32, count, a_batch_stride, w_batch_stride, M * N, _lib.stream_ptr(dev)))
     return y

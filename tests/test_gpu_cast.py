@@ -172,13 +172,22 @@ def test_unaligned_views(mh):
     base = torch.randn(32 * 64 + 3, generator=g).to(torch.bfloat16)
     x = base[3:]
     xd = base.to(DEV)[3:]
+    import warnings
+
+    from mase_hip import _lib
+
     meta = mx_meta(mh, 4, 3)
     sc_w, el_w = oracle.extract_mxfp(x.clone(), 32, 4, 3)
-    sc, el = mh.mxk.extract_mxfp_components(xd, meta)
-    assert_int_equal(sc, sc_w, "scales")
-    assert_int_equal(el, el_w, "elements")
-    mm = mh.MinifloatMeta(4, 3, True, "rn")
-    assert_int_equal(mh.mfk.extract_minifloat_component(xd, mm), oracle.extract_minifloat(x.clone(), 4, 3), "codes")
+    copies = _lib.realignment_copies
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)      # the first realignment copy of a process warns
+        sc, el = mh.mxk.extract_mxfp_components(xd, meta)
+        assert _lib.realignment_copies == copies + 1, "the copy that realigns the operand is counted"
+        assert_int_equal(sc, sc_w, "scales")
+        assert_int_equal(el, el_w, "elements")
+        mm = mh.MinifloatMeta(4, 3, True, "rn")
+        assert_int_equal(mh.mfk.extract_minifloat_component(xd, mm), oracle.extract_minifloat(x.clone(), 4, 3), "codes")
+        assert _lib.realignment_copies == copies + 2
 
 
 # ----------------------------------------------------------------------------- full-size configurations

@@ -512,7 +512,13 @@ def test_config_c4_full_size(mh):
 
 
 def test_config_c5_swiglu_chain(mh):
-    """down(silu(gate(x)) * up(x)) with MXFP6 E3M2 weights and MXFP8 E4M3 activations."""
+    """down(silu(gate(x)) * up(x)) with MXFP6 E3M2 weights and MXFP8 E4M3 activations.
+
+    Each of the three GEMMs (the down projection sums over K = 14336, the longest accumulation of any configuration) is held
+    to 1e-3 against a float64 dequantize-then-matmul built from the checker's components, on a sample of rows and columns and
+    on the very activations the GPU layer saw.  The chain's output is held to 1e-3 against backend="separate" over the whole
+    tensor, and to 3e-3 against the checker's own chain on the sampled rows: there the three per-layer errors add up, and an
+    intermediate that differs in its last bit can land in another MXFP8 code when the next layer quantises it."""
     from workloads import make_c5
 
     x, wg, wu, wd = make_c5()
@@ -531,10 +537,37 @@ def test_config_c5_swiglu_chain(mh):
         return d(torch.nn.functional.silu(g(inp)) * u(inp))
 
     xd = x.to(DEV)
-    y = mlp(layers("fused"), xd)
+    fused = layers("fused")
+    y = mlp(fused, xd)
     y_sep = mlp(layers("separate"), xd)
     assert y.shape == (4, 2048, 4096)
-    assert rel_fro(y, y_sep) <= 3 * REL_FRO_TOL  # three chained GEMMs, each within 1e-3
+    assert rel_fro(y, y_sep) <= REL_FRO_TOL
+
+    # ---- per layer, against the checker (float64 accumulation, bf16 output like the layer's)
+    x2 = x.view(-1, 4096)
+    rows = torch.arange(5, 8192, 523)                       # 16 rows of the 8192
+    cols_wide = torch.arange(3, 14336, 389)                 # 37 of the 14336 outputs of gate / up
+    cols_down = torch.arange(1, 4096, 111)                  # 37 of the 4096 outputs of down
+    g_gpu, u_gpu = fused[0](xd).view(-1, 14336), fused[1](xd).view(-1, 14336)
+    h_gpu = torch.nn.functional.silu(g_gpu) * u_gpu         # what the down layer is given
+    d_gpu = fused[2](h_gpu)
+    x_dq = oracle.qdq_mxfp(x2[rows], 32, 4, 3)
+    for name, w, got in (("gate", wg, g_gpu), ("up", wu, u_gpu)):
+        ref = oracle.matmul_nt(x_dq, oracle.qdq_mxfp(w[cols_wide], 32, 3, 2)).to(torch.bfloat16)
+        err = rel_fro(got[rows.to(DEV)][:, cols_wide.to(DEV)], ref)
+        assert err <= REL_FRO_TOL, f"{name}: {err}"
+    h_dq = oracle.qdq_mxfp(h_gpu[rows.to(DEV)].cpu(), 32, 4, 3)
+    ref = oracle.matmul_nt(h_dq, oracle.qdq_mxfp(wd[cols_down], 32, 3, 2)).to(torch.bfloat16)
+    err = rel_fro(d_gpu[rows.to(DEV)][:, cols_down.to(DEV)], ref)
+    assert err <= REL_FRO_TOL, f"down: {err}"
+
+    # ---- the whole chain on the sampled rows, every step from the checker
+    g_ref = oracle.matmul_nt(x_dq, oracle.qdq_mxfp(wg, 32, 3, 2)).to(torch.bfloat16)
+    u_ref = oracle.matmul_nt(x_dq, oracle.qdq_mxfp(wu, 32, 3, 2)).to(torch.bfloat16)
+    h_ref = torch.nn.functional.silu(g_ref) * u_ref
+    y_ref = oracle.matmul_nt(oracle.qdq_mxfp(h_ref, 32, 4, 3), oracle.qdq_mxfp(wd, 32, 3, 2)).to(torch.bfloat16)
+    err = rel_fro(y.view(-1, 4096)[rows.to(DEV)], y_ref)
+    assert err <= 3 * REL_FRO_TOL, f"chain: {err}"
 
 
 @pytest.mark.parametrize("func_type", ["XW", "XqW", "XWq", "XqWq"])
@@ -562,10 +595,15 @@ def test_mxfp_matmul(mh, func_type, backend):
 
 @pytest.mark.parametrize("a_shape,b_shape,dtype", [
     ((3, 40, 256), (256, 192), torch.bfloat16),          # matrix `other`: one GEMM over all rows
-    ((2, 600, 128), (2, 128, 320), torch.bfloat16),      # a launch per batch, 256 x 256 tiles
-    ((40, 16, 64), (40, 64, 96), torch.bfloat16),        # many batches: one batched dense GEMM
-    ((2, 4, 24, 96), (4, 96, 64), torch.bfloat16),       # broadcast batch axes: dense GEMM
+    ((2, 600, 128), (2, 128, 320), torch.bfloat16),      # batched launch, 256 x 256 tiles (N not a multiple of 128)
+    ((40, 16, 64), (40, 64, 96), torch.bfloat16),        # many batches, few rows each (16-row weight-streaming kernel)
+    ((2, 4, 24, 96), (4, 96, 64), torch.bfloat16),       # `other` broadcast along the first batch axis (its components are expanded)
+    ((3, 1, 24, 96), (1, 5, 96, 64), torch.bfloat16),    # both operands broadcast along one axis each
+    ((24, 96), (5, 96, 64), torch.bfloat16),             # matrix `input` against batched `other`: A shared (stride 0)
+    ((1, 1, 24, 96), (2, 3, 96, 64), torch.bfloat16),    # the same with explicit unit batch axes
+    ((6, 200, 256), (6, 256, 256), torch.bfloat16),      # 128 x 128 tile kernel, batched
     ((2, 50, 128), (2, 128, 72), torch.float32),         # fp32 in and out
+    ((2, 3, 32), (2, 32, 4), torch.bfloat16),            # outputs of a product not 16-byte aligned: dense route
     ((4, 48), (48, 40), torch.bfloat16),                 # contraction axis not a multiple of 32
 ])
 def test_mxfp_matmul_fused_routes(mh, a_shape, b_shape, dtype):
@@ -586,6 +624,77 @@ def test_mxfp_matmul_fused_routes(mh, a_shape, b_shape, dtype):
         assert rel_fro(y, y_chk) <= tol, func_type
         y_sep = mh.F.mxfp_matmul(a.to(DEV), b.to(DEV), fmt if func_type == "XqWq" else None, fmt, func_type, "separate")
         assert rel_fro(y, y_sep) <= tol, func_type
+
+
+def test_linear_with_inf_nan_element_format_takes_the_dense_route(mh):
+    """element_is_finite=False: codes with the top exponent field mean inf / NaN.  The GEMM decodes that field as an ordinary
+    binade, so such weights must not reach it: fused equals separate bit for bit (both compose, then F.linear)."""
+    g = torch.Generator().manual_seed(12)
+    M, N, K = 64, 128, 256
+    meta = mh.meta.MXFPMeta(block_size=32, scale_exp_bits=8, element_exp_bits=4, element_frac_bits=3, element_is_finite=False,
+                            round_mode="rn")
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w_el = torch.randint(0, 0x78, (N * K // 32, 32), generator=g, dtype=torch.uint8)
+    w_el[5, 7] = 0x78                                   # +inf in this format, 256 in the finite one
+    w_el[9, 1] = 0xFB                                   # NaN
+    w_sc = torch.randint(120, 130, (N * K // 32, 1), generator=g, dtype=torch.uint8)
+    tm = mh.meta.MXFPTensorMeta(device="cuda:0", dtype="bfloat16", shape=(N, K), block_dim=1, meta=meta)
+    args = dict(x=x, x_meta=preset(mh, "MXFP8_E4M3_fn"), w=None, w_scales=w_sc.to(DEV), w_elements=w_el.to(DEV), w_tensor_meta=tm,
+                b=None, b_scales=None, b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
+    y_f = mh.F.mxfp_linear(**args, backend="fused")
+    y_s = mh.F.mxfp_linear(**args, backend="separate")
+    row_inf, row_nan = (5 * 32 + 7) // K, (9 * 32 + 1) // K
+    assert y_f[:, row_nan].isnan().all() and not torch.isfinite(y_f[:, row_inf]).any()
+    same = (y_f.view(torch.int16) == y_s.view(torch.int16)) | (y_f.isnan() & y_s.isnan())
+    assert same.all()
+    with pytest.raises(AssertionError):
+        mh.mxk.mxfp_gemm(x, None, None, None, w_sc.to(DEV), w_el.to(DEV), meta, None, M, N, K, torch.bfloat16)
+
+
+def test_gemm_batched_entry_point(mh):
+    """mase_hip_mxfp_gemm_batched through the C ABI: every product bit-identical to the single-product entry point on the same
+    operands (the same kernel runs on every grid plane), with per-product, shared (stride 0) and padded strides, on shapes that
+    take different kernels; and its argument checks."""
+    from mase_hip import _lib
+
+    lib = _lib.load()
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    stream = _lib.stream_ptr(torch.device(DEV))
+    g = torch.Generator(device=DEV).manual_seed(21)
+    for (B, M, N, K), a_shared, w_shared, pad in (((8, 128, 512, 1024), False, False, 0), ((5, 16, 256, 256), True, False, 0),
+                                                  ((3, 300, 256, 128), False, True, 0), ((4, 640, 1536, 256), False, False, 64),
+                                                  ((20, 1, 32, 32), False, False, 0), ((3, 70, 96, 160), False, False, 32)):
+        a_stride = 0 if a_shared else M * K + pad
+        w_stride = 0 if w_shared else N * K + pad
+        y_stride = M * N + pad
+        n_a = -(-((B - 1) * a_stride + M * K) // 32) * 32
+        a = mh.mxk.quantize_dequantize(torch.randn(n_a, generator=g, device=DEV).to(torch.bfloat16), fmt, torch.bfloat16)
+        w_el = torch.randint(0, 256, ((B - 1) * w_stride + N * K,), generator=g, device=DEV, dtype=torch.uint8)
+        w_el[w_el % 128 == 127] = 0x3F                                  # keep the products finite
+        w_sc = torch.randint(118, 130, (((B - 1) * w_stride + N * K) // 32,), generator=g, device=DEV, dtype=torch.uint8)
+        y = torch.full(((B - 1) * y_stride + M * N,), float("nan"), dtype=torch.bfloat16, device=DEV)
+        rc = lib.mase_hip_mxfp_gemm_batched(a.data_ptr(), 2, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, y.data_ptr(), 2, M, N, K, 32, B,
+                                            a_stride, w_stride, y_stride, stream)
+        assert rc == 0, lib.mase_hip_last_error()
+        for b in range(B):
+            y1 = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            rc = lib.mase_hip_mxfp_gemm(a.data_ptr() + 2 * b * a_stride, 2, None, None, 0, 0, w_sc.data_ptr() + b * w_stride // 32,
+                                        w_el.data_ptr() + b * w_stride, 4, 3, None, 0, y1.data_ptr(), 2, M, N, K, 32, stream)
+            assert rc == 0, lib.mase_hip_last_error()
+            got = y[b * y_stride: b * y_stride + M * N].view(M, N)
+            assert torch.isfinite(got.float()).all(), (B, M, N, K, b)
+            assert torch.equal(got.view(torch.int16), y1.view(torch.int16)), (B, M, N, K, b)
+        if pad:                                                          # the gaps between the products are left alone
+            assert y[M * N: y_stride].isnan().all()
+    p = a.data_ptr()
+    bad = lambda **kw: lib.mase_hip_mxfp_gemm_batched(p, 2, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, y.data_ptr(), 2, 16, 32, 32, 32,
+                                                      kw.get("B", 2), kw.get("a", 512), kw.get("w", 1024), kw.get("y", 512), stream)
+    assert bad(B=0) == -1 and bad(B=70000) == -1
+    assert bad(a=100) == -1 and bad(w=1000) == -1 and bad(y=100) == -1   # products would overlap
+    assert bad(a=516) == -1 and bad(w=1040) == -1 and bad(y=516) == -1   # misaligned products
+    assert lib.mase_hip_mxfp_gemm_batched(None, 2, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, y.data_ptr(), 2, 16, 32, 32, 32, 2, 512, 1024, 512,
+                                          stream) == -1
+    torch.cuda.synchronize()
 
 
 def test_gemm_dispatch_boundaries(mh):

@@ -175,3 +175,47 @@ def test_minifloat_matmul(mf, func_type, backend):
     b_dq = oracle.qdq_minifloat(b, bm.exp_bits, bm.frac_bits) if "Wq" in func_type else b
     assert y.shape == (4, 48, 80) and y.dtype == torch.bfloat16
     assert rel_fro(y, (a_dq.double() @ b_dq.double()).to(y.dtype)) <= REL_FRO_TOL
+
+
+@pytest.mark.parametrize("w_tag", W_TAGS)
+@pytest.mark.parametrize("a_shape,b_shape,dtype", [
+    ((4, 48, 96), (96, 80), torch.bfloat16),             # matrix `other`: one GEMM over all rows
+    ((3, 40, 128), (3, 128, 64), torch.bfloat16),        # one batched launch
+    ((2, 1, 24, 64), (1, 5, 64, 32), torch.bfloat16),    # broadcast batch axes
+    ((24, 64), (5, 64, 32), torch.bfloat16),             # matrix `input` shared by every product
+    ((2, 50, 128), (2, 128, 72), torch.float32),         # fp32 in and out
+    ((4, 48), (48, 40), torch.bfloat16),                 # contraction axis not a multiple of 32: dense route
+])
+def test_minifloat_matmul_fused_routes(mf, w_tag, a_shape, b_shape, dtype):
+    """backend="fused" with `other` in every one-byte format the GEMM decodes: the codes go through the MFMA GEMM with unit
+    block scales, whatever the batch axes; against fp64 on the checker's quantised values and against backend="separate"."""
+    g = torch.Generator().manual_seed(sum(a_shape) + len(w_tag))
+    a = torch.randn(*a_shape, generator=g).to(dtype)
+    b = (2.0 * torch.randn(*b_shape, generator=g)).to(dtype)
+    am, bm = mf.meta.FP8_E4M3_fn, getattr(mf.meta, w_tag)
+    b_dq = oracle.qdq_minifloat(b, bm.exp_bits, bm.frac_bits)
+    for func_type in ("XqWq", "XWq"):
+        if func_type == "XWq" and dtype == torch.float32:
+            continue                                     # a dense fp32 input is not rounded to bf16: dense route, covered above
+        y = mf.F.minifloat_matmul(a.to(DEV), b.to(DEV), am if func_type == "XqWq" else None, bm, func_type, "fused")
+        a_dq = oracle.qdq_minifloat(a, am.exp_bits, am.frac_bits) if func_type == "XqWq" else a
+        y_chk = torch.matmul(a_dq.double(), b_dq.double()).to(dtype)
+        assert y.shape == y_chk.shape and y.dtype == dtype
+        tol = REL_FRO_TOL if dtype == torch.bfloat16 else 1e-5
+        assert rel_fro(y, y_chk) <= tol, func_type
+        y_sep = mf.F.minifloat_matmul(a.to(DEV), b.to(DEV), am if func_type == "XqWq" else None, bm, func_type, "separate")
+        assert rel_fro(y, y_sep) <= tol, func_type
+
+
+def test_minifloat_matmul_fused_takes_the_gemm(mf, monkeypatch):
+    """The fused backend really leaves `other` in code form: torch.matmul is not called on the GEMM route."""
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(3, 40, 128, generator=g).to(torch.bfloat16).to(DEV)
+    b = torch.randn(3, 128, 64, generator=g).to(torch.bfloat16).to(DEV)
+
+    def boom(*args, **kwargs):
+        raise AssertionError("dense matmul called")
+
+    monkeypatch.setattr(torch, "matmul", boom)
+    y = mf.F.minifloat_matmul(a, b, mf.meta.FP8_E4M3_fn, mf.meta.FP8_E4M3_fn, "XqWq", "fused")
+    assert y.shape == (3, 40, 64)
