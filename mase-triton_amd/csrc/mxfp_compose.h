@@ -76,13 +76,16 @@ struct Composer {
         return ((w & SIGN4) << (7 - E - M)) | ((w & MAG4) << (3 - M));
     }
     template <bool HI>
-    __device__ inline uint32_t hw_pair(uint32_t w, uint32_t e4) const {  // e4 = embed4(w), or for E4M3 w & 0x7F7F7F7F
+    __device__ inline uint32_t hw_pair(uint32_t w, uint32_t e4) const {  // e4 = embed4(w)
         typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
         const uint32_t r = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(e4, hw_scale, HI));
         if (!TOP_IS_NAN) return r;
-        const uint32_t c = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(ushort2_t, r), __builtin_bit_cast(ushort2_t, top2)));
+        // magnitude 0x7F comes back as 0xFFC0 whatever its sign; every other code as the right bf16, sign included.  As
+        // unsigned 16-bit numbers 0xFFC0 is above every finite pattern of either sign and (sign | top) is the largest
+        // finite one of its sign, so the minimum with (sign of the code | top) replaces exactly the NaNs.
         const uint32_t sg = __builtin_amdgcn_perm(0u, w, HI ? 0x030C020Cu : 0x010C000Cu);  // the pair's code bytes in the high byte of each half
-        return (sg & 0x80008000u) | c;
+        const uint32_t cand = (sg & 0x80008000u) | top2;
+        return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(ushort2_t, r), __builtin_bit_cast(ushort2_t, cand)));
     }
     __device__ inline uint32_t bf16_pair_fp16(uint32_t x) const {  // x: each 16-bit half = (code << PRE) << 8
         typedef short shortx2 __attribute__((ext_vector_type(2)));
@@ -100,15 +103,15 @@ struct Composer {
     // codes 0,1 (pair_lo) / 2,3 (pair_hi) of a dword of 4 codes -> 2 bf16; any code; any scale below SLOW_FROM
     __device__ inline uint32_t pair_lo(uint32_t w) const {
         if (!HW) return bf16_pair_wide(w, 0);
-        return hw_pair<false>(w, TOP_IS_NAN ? w & 0x7F7F7F7Fu : embed4(w));
+        return hw_pair<false>(w, embed4(w));
     }
     __device__ inline uint32_t pair_hi(uint32_t w) const {
         if (!HW) return bf16_pair_wide(w, 1);
-        return hw_pair<true>(w, TOP_IS_NAN ? w & 0x7F7F7F7Fu : embed4(w));
+        return hw_pair<true>(w, embed4(w));
     }
     __device__ inline void pair2(uint32_t w, uint32_t& o0, uint32_t& o1) const {
         if (!HW) { o0 = bf16_pair_wide(w, 0); o1 = bf16_pair_wide(w, 1); return; }
-        const uint32_t e4 = TOP_IS_NAN ? w & 0x7F7F7F7Fu : embed4(w);
+        const uint32_t e4 = embed4(w);
         o0 = hw_pair<false>(w, e4);
         o1 = hw_pair<true>(w, e4);
     }
