@@ -346,14 +346,16 @@ struct PackedBf16 {
     // code magnitudes (exponent and mantissa fields, no sign) of two elements, one per 16-bit half,
     // plus, through `t_q`, the quantised magnitude back in the t domain for the fused QDQ
     __device__ static inline uint32_t magnitude(uint32_t a, uint32_t ssb2, uint32_t& t_q) {
-        i16x2 t = as_i16x2(a) - as_i16x2(ssb2);
-        t = __builtin_elementwise_max(t, (i16x2){0, 0});                    // underflow -> 0
-        const uint32_t tu = as_u32(t);
+        // a - ssb2 clamped at 0 (underflow -> 0); the caller guarantees ssb2 >= 0 in both halves
+        const uint32_t tu = as_u32(__builtin_elementwise_sub_sat(as_u16x2(a), as_u16x2(ssb2)));
+        const i16x2 t = as_i16x2(tu);
         const uint32_t u = as_u32(as_u16x2(tu) >> (unsigned short)SH);    // (ye << M) | truncated mantissa
         const uint32_t r = tu + (((1u << (SH - 1)) - 1u) * LSB) + (u & LSB);  // round half to even
         const uint32_t v = as_u32(as_u16x2(r) >> (unsigned short)SH);     // (ye << M) + rounded mantissa
-        // a carry out of the mantissa into an odd exponent field is lost by the reference's OR
-        const uint32_t code_n = v - (((v ^ u) >> 1) & ((1u << M) * LSB));
+        // the reference ORs the exponent field with the rounded mantissa, so a carry out of the mantissa into an odd
+        // exponent field is lost
+        const uint32_t ef = u & (0xFFFFu & ~((1u << M) - 1u)) * LSB;
+        const uint32_t code_n = ef | (v - ef);
         // ye == 0: the mantissa (with its carry) is shifted down under an explicit leading one
         const uint32_t w = as_u32(as_u16x2(v | ((1u << M) * LSB)) >> (unsigned short)1);
         const uint32_t code_s = as_u32(as_u16x2(w) * __builtin_elementwise_min(as_u16x2(v), (u16x2){1, 1}));
@@ -412,7 +414,8 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
         amax = max(amax, (uint32_t)__builtin_amdgcn_mov_dpp((int)amax, 0x4E, 0xF, 0xF, true));  // lane ^ 2
         const int ef_max = (int)(amax >> 7);
         const int scale_n = max(ef_max - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
-        const bool hard = amax >= 0x7F80u || scale_n >= 151 || (MODE == 1 && amax != 0u && scale_n <= fmt_bias(f));
+        // (scale_n < bias: the packed arithmetic subtracts (scale_n - bias) << 7 with unsigned saturation)
+        const bool hard = amax >= 0x7F80u || scale_n >= 151 || (amax != 0u && scale_n < fmt_bias(f) + (MODE == 1 ? 1 : 0));
         uint32_t o[4];
         uint32_t scale = (uint32_t)scale_n;
         if (__builtin_amdgcn_ballot_w64(hard) == 0) {
@@ -703,7 +706,7 @@ __device__ inline void strided_bf16_block(const uint16_t* x, int64_t first, int6
     for (int c = 0; c < 2; ++c) {
         amax[c] = m[c];
         const int scale_n = max((int)(amax[c] >> 7) - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
-        hard |= amax[c] >= 0x7F80u || scale_n >= 151 || (MODE == 1 && amax[c] != 0u && scale_n <= fmt_bias(f));
+        hard |= amax[c] >= 0x7F80u || scale_n >= 151 || (amax[c] != 0u && scale_n < fmt_bias(f) + (MODE == 1 ? 1 : 0));
         scale[c] = (uint32_t)scale_n;
     }
     if (__builtin_amdgcn_ballot_w64(hard) == 0) {
