@@ -345,10 +345,22 @@ struct PackedBf16 {
     static constexpr uint32_t LSB = 0x00010001u;
     // code magnitudes (exponent and mantissa fields, no sign) of two elements, one per 16-bit half,
     // plus, through `t_q`, the quantised magnitude back in the t domain for the fused QDQ
+    // Packed 16-bit operations written as asm: given the plain expressions the compiler replaces each of them by one
+    // compare and one conditional move per 16-bit half plus a byte permute to put the halves together again.
+    __device__ static inline uint32_t pk_min_u16(uint32_t a, uint32_t b) {
+        uint32_t d;
+        asm("v_pk_min_u16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+        return d;
+    }
+    // all ones in the halves where a < b (as signed 16-bit numbers whose difference fits 16 bits)
+    __device__ static inline uint32_t pk_less_mask(uint32_t a, uint32_t b) {
+        uint32_t d;
+        asm("v_pk_sub_i16 %0, %1, %2\n\tv_pk_ashrrev_i16 %0, 15, %0 op_sel_hi:[0,1]" : "=&v"(d) : "v"(a), "v"(b));
+        return d;
+    }
     __device__ static inline uint32_t magnitude(uint32_t a, uint32_t ssb2, uint32_t& t_q) {
-        // a - ssb2 clamped at 0 (underflow -> 0); the caller guarantees ssb2 >= 0 in both halves
+        // t = a - ssb2 clamped at 0 (underflow -> 0); the caller guarantees ssb2 >= 0 in both halves
         const uint32_t tu = as_u32(__builtin_elementwise_sub_sat(as_u16x2(a), as_u16x2(ssb2)));
-        const i16x2 t = as_i16x2(tu);
         const uint32_t u = as_u32(as_u16x2(tu) >> (unsigned short)SH);    // (ye << M) | truncated mantissa
         const uint32_t r = tu + (((1u << (SH - 1)) - 1u) * LSB) + (u & LSB);  // round half to even
         const uint32_t v = as_u32(as_u16x2(r) >> (unsigned short)SH);     // (ye << M) + rounded mantissa
@@ -356,10 +368,11 @@ struct PackedBf16 {
         // exponent field is lost
         const uint32_t ef = u & (0xFFFFu & ~((1u << M) - 1u)) * LSB;
         const uint32_t code_n = ef | (v - ef);
-        // ye == 0: the mantissa (with its carry) is shifted down under an explicit leading one
-        const uint32_t w = as_u32(as_u16x2(v | ((1u << M) * LSB)) >> (unsigned short)1);
-        const uint32_t code_s = as_u32(as_u16x2(w) * __builtin_elementwise_min(as_u16x2(v), (u16x2){1, 1}));
-        const uint32_t is_norm = as_u32(((i16x2){127, 127} - t) >> (short)15);  // all ones where ye >= 1
+        // ye == 0: the mantissa (with its carry) is shifted down under an explicit leading one; zero stays zero
+        const uint32_t m01 = pk_min_u16(v, LSB);
+        const uint32_t code_s = as_u32(as_u16x2((m01 << M) | v) >> (unsigned short)1);
+        // all ones where ye >= 1, i.e. u >= 2^M
+        const uint32_t is_norm = pk_less_mask(((1u << M) - 1u) * LSB, u);
         // t-domain value of the code: normal codes keep their fields; subnormal code xf' (>= 2^(M-1))
         // is 2^-bias * xf' / 2^(M-1), i.e. exponent field 0 and mantissa (xf' << (8 - M)) & 0x7F
         const uint32_t tq_n = code_n << SH;
@@ -383,7 +396,7 @@ struct PackedBf16 {
         const uint32_t a = h & 0x7FFF7FFFu;
         uint32_t t_q;
         const uint32_t mag = magnitude(a, ssb2, t_q);
-        const uint32_t nonzero = as_u32((i16x2){0, 0} - as_i16x2(as_u32(__builtin_elementwise_min(as_u16x2(mag), (u16x2){1, 1}))));
+        const uint32_t nonzero = pk_less_mask(0u, mag);                    // code magnitudes are small positive numbers
         const uint32_t body = (t_q + ssb2) & nonzero;                      // code 0 -> +-0.0
         return (body | (h & 0x80008000u)) & live_mask(a);
     }
