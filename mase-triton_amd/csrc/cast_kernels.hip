@@ -13,6 +13,9 @@ namespace mase {
 
 constexpr int kThreads = 256;
 // 128-bit steps per lane and launch: one is fastest on every measured size (more, smaller workgroups in flight)
+#ifndef MASE_QDQ_NT
+#define MASE_QDQ_NT 1
+#endif
 #ifndef MASE_UNROLL_SMALL
 #define MASE_UNROLL_SMALL 1
 #endif
@@ -235,10 +238,24 @@ __global__ __launch_bounds__(kThreads) void minifloat_f32_kernel(const void* x, 
         for (int j = 0; j < 4; ++j) { code[2 * j] = w[j] & 0xFFFFu; code[2 * j + 1] = w[j] >> 16; }
     } else {
         const uint32_t* p = static_cast<const uint32_t*>(x) + wave_first + 4 * lane;
-        const uint4 a = ld128<MODE == 0>(p), b = ld128<MODE == 0>(p + 256);
+        const uint4 a = ld128<MASE_QDQ_NT || MODE == 0>(p), b = ld128<MASE_QDQ_NT || MODE == 0>(p + 256);
         const uint32_t u[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        // inf / NaN anywhere in the wavefront's 512 elements: the per-element routine for all of them
+        uint32_t amax = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) code[j] = encode_f32_bits(u[j], f);
+        for (int j = 0; j < 8; ++j) amax = max(amax, u[j] & 0x7FFFFFFFu);
+        bool fast = false;
+        if constexpr (F::kStatic) {
+            fast = __builtin_amdgcn_ballot_w64(amax >= 0x7F800000u) == 0;
+            if (fast) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) code[j] = encode_f32_finite_rn(u[j], f);
+            }
+        }
+        if (!fast) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) code[j] = encode_f32_bits(u[j], f);
+        }
     }
     if (MODE == 0) {
         uint16_t* c = static_cast<uint16_t*>(out) + wave_first + 4 * lane;
@@ -249,8 +266,8 @@ __global__ __launch_bounds__(kThreads) void minifloat_f32_kernel(const void* x, 
 #pragma unroll
         for (int j = 0; j < 8; ++j) y[j] = decode_f32(code[j], f);
         float* o = static_cast<float*>(out) + wave_first + 4 * lane;
-        st128<MODE == 1>(o, make_uint4(f32_bits(y[0]), f32_bits(y[1]), f32_bits(y[2]), f32_bits(y[3])));
-        st128<MODE == 1>(o + 256, make_uint4(f32_bits(y[4]), f32_bits(y[5]), f32_bits(y[6]), f32_bits(y[7])));
+        st128<MASE_QDQ_NT || MODE == 1>(o, make_uint4(f32_bits(y[0]), f32_bits(y[1]), f32_bits(y[2]), f32_bits(y[3])));
+        st128<MASE_QDQ_NT || MODE == 1>(o + 256, make_uint4(f32_bits(y[4]), f32_bits(y[5]), f32_bits(y[6]), f32_bits(y[7])));
     }
 }
 

@@ -142,6 +142,30 @@ __device__ inline uint32_t encode_f32_bits(uint32_t u, const F& f) {
     return encode_normal(sgn, (int)ef - 127, a & 0x7FFFFFu, f);
 }
 
+// The same code for a compile-time format (finite, round to nearest even) and any input that is not inf / NaN, without
+// branches.  With a15 = |u| >> 8 (exponent field above the 15 mantissa bits the reference keeps) and
+//     t = a15 - ((127 - bias) << 15)            (clamped at 0: e < -bias gives code 0)
+// t is (ye << 15) | f15, the exponent field in the target format above those 15 bits, and the rounding, the lost
+// carry of the final OR, the subnormal binade ye == 0 and the saturation are functions of t.  Zero and subnormal
+// inputs have a15 < 2^15 and fall to t = 0; they keep the sign code when negative and not -0.0 (fake.py:21-77).
+template <class F>
+__device__ inline uint32_t encode_f32_finite_rn(uint32_t u, const F& f) {
+    static_assert(F::kStatic, "compile-time formats only");
+    static_assert(F{}.finite() && F{}.rmode() == RN, "finite formats, round to nearest even");
+    constexpr int E = F{}.E(), M = F{}.M(), SH = 15 - M, BIAS = (1 << (E - 1)) - 1;
+    constexpr uint32_t TOP = (1u << (E + M)) - 1u, SIGN = 1u << (E + M);   // top exponent field 2^E - 1, mantissa all ones
+    constexpr uint32_t OFFSET = (uint32_t)(127 - BIAS) << 15;
+    const uint32_t a15 = (u >> 8) & 0x7FFFFFu;
+    const uint32_t t = a15 > OFFSET ? a15 - OFFSET : 0u;
+    const uint32_t q = t >> SH;                                               // (ye << M) | truncated mantissa
+    const uint32_t v = (t + ((1u << (SH - 1)) - 1u) + (q & 1u)) >> SH;        // (ye << M) + rounded mantissa
+    const uint32_t ef = q & ~((1u << M) - 1u);
+    const uint32_t code_n = min(ef | (v - ef), TOP);   // a carry into an odd exponent field is lost; ye above the top field saturates
+    const uint32_t code_s = ((min(v, 1u) << M) | v) >> 1;  // ye == 0: the mantissa under an explicit leading one
+    const uint32_t mag = q < (1u << M) ? code_s : code_n;
+    return mag | (u > 0x80000000u ? SIGN : 0u);
+}
+
 // ---------------------------------------------------------------------------------------
 // Decode (minifloat/fake.py:97-123): 2^(xe - bias [+1 if subnormal]) * (xf / 2^M [+1]).
 // ---------------------------------------------------------------------------------------
