@@ -494,6 +494,13 @@ __global__ __launch_bounds__(kThreads) void extract_mxfp_block_kernel(const void
     for (int j = 0; j < B; ++j) elements[b * B + j] = (uint8_t)encode_mxfp_element(load_bits_scalar<DT_IN>(x, b * B + j), se, f);
 }
 
+// block index of chunk c with `per_block` chunks to a block: a shift when per_block is a power of two (a 64-bit
+// division costs more instructions than the rest of a lane's work); the test is uniform over the launch
+__device__ inline int64_t block_of_chunk(int64_t c, int per_block) {
+    if ((per_block & (per_block - 1)) == 0) return c >> (31 - __builtin_clz((unsigned)per_block));
+    return c / per_block;
+}
+
 // Vector path: B % EPT == 0 (a lane's run lies inside one block).
 template <int DT_OUT, class F, int EPT, int UNROLL>
 __global__ __launch_bounds__(kThreads) void compose_mxfp_kernel(const uint8_t* __restrict__ scales,
@@ -514,7 +521,7 @@ __global__ __launch_bounds__(kThreads) void compose_mxfp_kernel(const uint8_t* _
                 const uint2 v = ld64(elements + c * EPT);
                 w[r][0] = v.x; w[r][1] = v.y;
             }
-            sc[r] = scales[c / chunks_per_block];
+            sc[r] = scales[block_of_chunk(c, chunks_per_block)];
         }
     }
 #pragma unroll
@@ -555,7 +562,7 @@ __global__ __launch_bounds__(kThreads) void compose_mxfp_bf16_kernel(const uint8
         sc[r] = 127u;
         if (c < n_chunks) {
             w[r] = ld64(elements + c * 8);
-            sc[r] = scales[c / chunks_per_block];
+            sc[r] = scales[block_of_chunk(c, chunks_per_block)];
         }
     }
 #pragma unroll
