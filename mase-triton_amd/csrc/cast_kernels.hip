@@ -16,6 +16,9 @@ constexpr int kThreads = 256;
 #ifndef MASE_QDQ_NT
 #define MASE_QDQ_NT 1
 #endif
+#ifndef MASE_UNROLL_COMPOSE
+#define MASE_UNROLL_COMPOSE 2
+#endif
 #ifndef MASE_UNROLL_SMALL
 #define MASE_UNROLL_SMALL 1
 #endif
@@ -23,7 +26,7 @@ constexpr int kThreads = 256;
 #define MASE_UNROLL_MXFP 1
 #endif
 #ifndef MASE_UNROLL_PACKED
-#define MASE_UNROLL_PACKED 1
+#define MASE_UNROLL_PACKED 2
 #endif
 
 typedef float floatx2 __attribute__((ext_vector_type(2)));
@@ -1034,7 +1037,7 @@ int mase_hip_compose_mxfp(const uint8_t* scales, const uint8_t* elements, void* 
     if (n == 0) return OK;
     if (!scales || !elements || !out) return fail(ERR_INVALID, "null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    constexpr int UNROLL = MASE_UNROLL_SMALL;
+    constexpr int UNROLL = MASE_UNROLL_COMPOSE;
     const int B = block_size;
     const bool al = aligned(elements, 8) && aligned(out, 16);
     return dispatch_fmt(exp_bits, frac_bits, is_finite, RN, [&](auto f) {
