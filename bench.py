@@ -562,7 +562,7 @@ def summarize_counters(fetch_dir, write_dir):
 
     rows = []
     for frag, key, rd, wr, sources in COUNTER_ROWS:
-        threads = {"extract_mxfp C1": _N1 // 8, "extract_mxfp C3": _N3 // 8}.get(key)   # one lane per 8 elements
+        threads = {"extract_mxfp C1": _N1 // 16, "extract_mxfp C3": _N3 // 16}.get(key)   # one lane per 2 x 8 elements
         (name, f_kib), (_, w_kib) = pick(fetch, frag, threads), pick(write, frag, threads)
         rows.append((key, name, f_kib, w_kib, rd, wr, sources))
     cal = rows[0]
