@@ -11,6 +11,11 @@ activations go through the single-pass QDQ kernel and the GEMM composes the MXFP
 to bf16 in registers on their way to the MFMA units (fp32 accumulation).  Every MXFP value has
 at most four significant bits, so bf16 operands are exact and the result differs from
 "separate" only by the summation order.
+backend="auto" (not in the reference) is "fused" up to ``AUTO_DENSE_FROM_ROWS`` rows of x and, from there on, the
+single-pass QDQ of x, ONE compose of W to bf16 in HBM and the library's dense GEMM: the fused kernel composes every W
+element once per 512 rows of x, and on this power-limited chip that in-loop work costs more than writing W out once when
+there are thousands of rows (measured cross-over between 2048 and 4096 rows for N x K = 14336 x 4096 and 4096 x 14336).
+It needs N * K * 2 bytes of temporary memory per call.
 """
 from __future__ import annotations
 
@@ -25,6 +30,7 @@ from .cast import compose_mxfp_tensor, extract_mxfp_components, quantize_dequant
 
 _LAYER_TYPES = ("XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq")
 _GEMM_DTYPES = (torch.bfloat16, torch.float32)
+AUTO_DENSE_FROM_ROWS = 3072
 
 
 def parse_mxfp_linear_type(x_meta: MXFPMeta | None, w_tensor_meta: MXFPTensorMeta | None,
@@ -70,11 +76,11 @@ def mxfp_linear(
     b_elements: Tensor | None,
     b_tensor_meta: MXFPTensorMeta | None,
     layer_type: Literal["XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq"],
-    backend: Literal["separate", "fused"],
+    backend: Literal["separate", "fused", "auto"],
 ) -> Tensor:
     if layer_type not in _LAYER_TYPES:
         raise NotImplementedError(f"Layer type {layer_type} not implemented")
-    if backend not in ("separate", "fused"):
+    if backend not in ("separate", "fused", "auto"):
         raise NotImplementedError(f"backend {backend!r} not implemented")
     quantised_x = layer_type.startswith("Xq")
     quantised_w = "Wq" in layer_type
@@ -88,8 +94,10 @@ def mxfp_linear(
             w = compose_mxfp_tensor(w_scales, w_elements, w_tensor_meta)
         return torch.nn.functional.linear(x, w, bias)
 
-    # ---- fused
-    if quantised_w and _gemm_eligible(x, quantised_x, w_tensor_meta, bias):
+    # ---- fused (auto: only while the rows of x are few enough for the in-loop compose to pay)
+    rows = x.numel() // x.shape[-1] if x.numel() else 0
+    through_kernel = backend == "fused" or rows < AUTO_DENSE_FROM_ROWS
+    if through_kernel and quantised_w and _gemm_eligible(x, quantised_x, w_tensor_meta, bias):
         out_features, in_features = w_tensor_meta.shape
         assert x.shape[-1] == in_features
         lead = x.shape[:-1]

@@ -36,7 +36,7 @@ class MXFPLinearPTQ(nn.Module):
         w_mxfp_meta: MXFPMeta | None,
         b_mxfp_meta: MXFPMeta | None,
         layer_type: LayerType,
-        backend: Literal["separate", "fused"] = "fused",
+        backend: Literal["separate", "fused", "auto"] = "fused",
         dtype: torch.dtype | None = None,
         device: torch.device | None = None,
         w_scales: Tensor | None = None,
@@ -119,7 +119,7 @@ class MXFPLinearPTQ(nn.Module):
 
     @classmethod
     def from_linear(cls, layer: nn.Linear, x_mxfp_meta: MXFPMeta | None, w_mxfp_meta: MXFPMeta | None,
-                    b_mxfp_meta: MXFPMeta | None, layer_type: LayerType, backend: Literal["separate", "fused"]):
+                    b_mxfp_meta: MXFPMeta | None, layer_type: LayerType, backend: Literal["separate", "fused", "auto"]):
         """Quantise a trained ``nn.Linear``."""
         assert isinstance(layer, nn.Linear), "layer must be an instance of nn.Linear"
         with torch.no_grad():
@@ -144,7 +144,7 @@ class MXFPLinearPTQ(nn.Module):
         return d
 
     @classmethod
-    def from_exported(cls, d: dict, backend: Literal["separate", "fused"] = "fused", device=None):
+    def from_exported(cls, d: dict, backend: Literal["separate", "fused", "auto"] = "fused", device=None):
         """Inverse of :meth:`export_quantized`."""
         from . import packing
 
@@ -167,7 +167,7 @@ class MXFPLinearPTQ(nn.Module):
                        bias: Tensor | None, b_scales: Tensor | None, b_elements: Tensor | None,
                        b_tensor_meta: MXFPTensorMeta | None, x_mxfp_meta: MXFPMeta | None,
                        layer_type: Literal["XWqB", "XWqBq", "XqWqB", "XqWqBq"],
-                       backend: Literal["separate", "fused"]):
+                       backend: Literal["separate", "fused", "auto"]):
         """Re-hydrate from stored components (tensor metas are not part of ``state_dict``)."""
         assert w_scales is not None and w_elements is not None and w_tensor_meta is not None
         return cls(weight=None, bias=bias, x_mxfp_meta=x_mxfp_meta, w_mxfp_meta=None, b_mxfp_meta=None,

@@ -509,6 +509,30 @@ def test_config_c4_full_size(mh):
     w_dq = oracle.qdq_mxfp(w[cols], 32, 4, 3)
     y_ref = oracle.matmul_nt(x_dq, w_dq).to(torch.bfloat16)
     assert rel_fro(y[rows.to(DEV)][:, cols.to(DEV)], y_ref) <= REL_FRO_TOL
+    # backend="auto" takes the compose-once route at this many rows; same bar
+    y_auto = mh.F.mxfp_linear(**args, backend="auto")
+    assert rel_fro(y_auto[rows.to(DEV)][:, cols.to(DEV)], y_ref) <= REL_FRO_TOL
+
+
+def test_backend_auto_switches_on_rows(mh):
+    """backend="auto": the fused kernel below AUTO_DENSE_FROM_ROWS rows of x (bit-identical to backend="fused"), the single-pass QDQ
+    + one compose of W + library GEMM from there on (within the tolerance of the float64 checker)."""
+    from mase_hip.mxfp.functional import linear as lin
+
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    g = torch.Generator().manual_seed(11)
+    w = torch.randn(256, 512, generator=g).mul(0.02).to(torch.bfloat16)
+    w_sc, w_el, w_tm = mh.F.extract_mxfp_components(w.to(DEV), block_dim=1, mxfp_meta=fmt)
+    for rows in (lin.AUTO_DENSE_FROM_ROWS - 64, lin.AUTO_DENSE_FROM_ROWS):
+        x = torch.randn(rows, 512, generator=g).to(torch.bfloat16)
+        args = dict(x=x.to(DEV), x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
+                    b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
+        y_auto = mh.F.mxfp_linear(**args, backend="auto")
+        y_fused = mh.F.mxfp_linear(**args, backend="fused")
+        if rows < lin.AUTO_DENSE_FROM_ROWS:
+            assert torch.equal(y_auto, y_fused)
+        y_ref = oracle.matmul_nt(oracle.qdq_mxfp(x, 32, 4, 3), oracle.qdq_mxfp(w, 32, 4, 3)).to(torch.bfloat16)
+        assert rel_fro(y_auto, y_ref) <= REL_FRO_TOL
 
 
 def test_config_c5_swiglu_chain(mh):
