@@ -145,6 +145,51 @@ def test_minifloat_random_vs_checker(mh, dt, n):
             assert_bits_equal(mh.mfk.quantize_dequantize(xd, meta, odt), w, name, f"qdq {dt}->{name} n={n}")
 
 
+@pytest.mark.parametrize("tag", list(PRESETS))
+def test_mxfp_bf16_every_pattern_under_chosen_block_maxima(mh, tag):
+    """Every bf16 bit pattern as an element of a block whose first element is a chosen value (exponent fields from the
+    subnormal edge to the top, smallest and largest mantissa): elements above it become the block maximum themselves, the
+    others land in every binade below it, inf / NaN patterns make special blocks.  Extract, compose and the fused pass
+    against the checker, bit for bit: pins the packed 16-bit arithmetic of the bf16 kernels."""
+    e, m = PRESETS[tag]
+    pats = torch.arange(1 << 16, dtype=torch.int32)
+    pats = torch.cat([pats, torch.zeros(31 * 2115 - (1 << 16), dtype=torch.int32)]).view(2115, 31)
+    blocks = []
+    for ef in (1, 2, 9, 60, 126, 127, 128, 140, 200, 253, 254):
+        for mant in (0x00, 0x7F):
+            first = torch.full((2115, 1), (ef << 7) | mant, dtype=torch.int32)
+            blocks.append(torch.cat([first, pats], dim=1))
+    bits = torch.cat(blocks).reshape(-1)
+    x = bits.to(torch.int16).view(torch.bfloat16)
+    xd = x.to(DEV)
+    meta = mx_meta(mh, e, m)
+    w_sc, w_el = oracle.extract_mxfp(x, 32, e, m)
+    g_sc, g_el = mh.mxk.extract_mxfp_components(xd, meta)
+    assert_int_equal(g_sc.flatten(), w_sc.flatten(), f"scales {tag}")
+    assert_int_equal(g_el.flatten(), w_el.flatten(), f"elements {tag}")
+    want = oracle.compose_mxfp(w_sc, w_el, 32, e, m, True, torch.bfloat16)
+    assert_bits_equal(mh.mxk.compose_mxfp_tensor(g_sc, g_el, meta, torch.bfloat16), want, "bfloat16", f"compose {tag}")
+    assert_bits_equal(mh.mxk.quantize_dequantize(xd, meta, torch.bfloat16), want, "bfloat16", f"qdq {tag}")
+
+
+@pytest.mark.parametrize("tag", list(PRESETS))
+def test_minifloat_every_fp32_class(mh, tag):
+    """The code of an fp32 input depends on its sign, its exponent field and the top 15 bits of its mantissa only
+    (the reference truncates the mantissa to 15 bits before it rounds): 2^24 classes.  One input of every class, the low
+    8 mantissa bits filled from a hash of the class, through extract and the fused pass against the checker: pins the
+    branch-free encode of the preset formats, ties, lost carries, the subnormal binade and saturation included."""
+    e, m = PRESETS[tag]
+    cls = torch.arange(1 << 24, dtype=torch.int64)
+    low = (cls * 2654435761 >> 11) & 0xFF
+    x = ((cls << 8) | low).to(torch.int32).view(torch.float32)   # classes with exponent field 255 are inf / NaN inputs
+    xd = x.to(DEV)
+    meta = mh.MinifloatMeta(e, m, True, "rn")
+    want = oracle.extract_minifloat(x, e, m, True, "rn")
+    assert_int_equal(mh.mfk.extract_minifloat_component(xd, meta), want, f"codes {tag}")
+    assert_bits_equal(mh.mfk.quantize_dequantize(xd, meta, torch.float32), oracle.compose_minifloat(want, e, m, True, torch.float32),
+                      "float32", f"qdq {tag}")
+
+
 @pytest.mark.parametrize("dt", ["float32", "bfloat16", "float16"])
 @pytest.mark.parametrize("block,n_blocks", [(32, 1), (32, 5), (32, 1025), (32, 40000), (16, 77), (64, 33), (8, 3),
                                              (4, 10), (3, 7), (1, 5), (96, 9), (256, 17), (1024, 3)])
