@@ -252,6 +252,50 @@ int mase_hip_mxfp_gemm_static_ws(const void* a_dense, int a_dtype, const uint8_t
                                  int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
                                  void* stream);
 
+/*
+ * ---- The same product on the block-scaled matrix instruction (v_mfma_scale_f32_16x16x128_f8f6f4).
+ *
+ * Both operands stay MXFP up to the matrix unit: FP8 (E4M3) bytes and one E8M0 scale per 32 elements along K, which
+ * the instruction applies itself; products are exact and accumulate in fp32.  Nothing is composed to bfloat16, so
+ * an operand byte costs half the LDS and cache traffic of the bf16 kernels and the instruction runs at twice the
+ * bf16 rate.  The operands are handed over in a prepared form, built by one of two calls:
+ *
+ *   mase_hip_scaled_operand_from_dense(x, BF16, E, M, rows, K, out_codes, out_scales, stream)
+ *       extract of the row-major [rows, K] bfloat16 matrix x (blocks of 32 along K, element format (E, M), finite,
+ *       round to nearest: what mase_hip_extract_mxfp computes) written straight into the prepared form;
+ *   mase_hip_scaled_operand_from_mxfp(scales, elements, E, M, rows, K, out_codes, out_scales, stream)
+ *       the same from MXFP components in the reference's layout (scales[rows * K / 32], elements[rows * K]).
+ *
+ * Prepared form: out_codes [rows_pad, K] bytes, out_scales [K / 128, rows_pad] dwords, rows_pad =
+ * mase_hip_scaled_padded_rows(rows) (the next multiple of 256; rows past `rows` are never written and may hold
+ * anything).  Byte (k / 32) % 4 of dword [k / 128][row] is the scale of block k / 32 of that row.  Element formats
+ * (2,1) (2,3) (3,2) are embedded into E4M3 bytes of the same value under the same scale (exact).  E4M3 itself: the
+ * matrix unit reads the code S.1111.111 as NaN where the reference has +-480, so a block that holds it is stored one
+ * scale step up with every code halved.  That is exact except for a block's odd codes below 16 (elements 2^13 and
+ * more below the block's largest), which round half to even: a change of at most 2^-14 of the block's largest
+ * element.  E5M2 is not taken (-2): every block of it reaches the binade the matrix unit reads as inf / NaN.
+ * A block with scale byte 255 (it held inf or NaN) makes its row of the product NaN, as in the reference whenever
+ * the block also holds a zero code (always, unless all 32 inputs were inf / NaN).
+ *
+ *   mase_hip_mxfp_gemm_scaled(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, out_dtype, M, N, K, stream)
+ *       y[M,N] = A[M,K] * W[N,K]^T (+ bias), A and W prepared as above with rows M and N.
+ *
+ * K % 256 == 0 and K >= 512; N a multiple of 8 (4 for fp32 output); codes and y 16-byte aligned.  Other shapes: -2,
+ * use mase_hip_mxfp_gemm.
+ * Replaces, like mase_hip_mxfp_gemm, the unimplemented backend="fused" of mxfp_linear_XqWq
+ *   src/mase_triton/mxfp/functional/linear.py:36-64
+ * (extract of x :50-52, the two composes :53-54 and the linear :61 in one prepare call and one GEMM).
+ */
+int64_t mase_hip_scaled_padded_rows(int64_t rows);
+int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits, int frac_bits, int64_t rows,
+                                       int64_t K, uint8_t* out_codes, uint32_t* out_scales, void* stream);
+int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elements, int exp_bits,
+                                      int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
+                                      uint32_t* out_scales, void* stream);
+int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes,
+                              const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
+                              int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

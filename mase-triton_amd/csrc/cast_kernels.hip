@@ -422,12 +422,68 @@ struct PackedBf16 {
     }
 };
 
-// MODE 0: extract (scales + elements); MODE 1: fused quantise-dequantise to bf16
+// ------------------------------------------------------------------------------ operands of the block-scaled GEMM
+// The block-scaled matrix instruction takes FP8 (E4M3) bytes and one E8M0 scale per 32 of them.  It reads the code
+// S.1111.111 as NaN where the reference's finite E4M3 has +-480, so a block that holds that code is stored one scale
+// step up with every code halved: exact for codes of 16 and more (exponent field - 1) and for even codes below 16
+// (whose value is code * 2^-9 in units of the block scale); an odd code below 16 rounds half to even.  The narrower
+// element formats are embedded into E4M3 bytes with the same value and the same block scale (their subnormals are
+// E4M3 normals).  Scales go out transposed for the GEMM's DMA: dword [k / 128][row], byte (k / 32) % 4.
+__device__ inline uint32_t e4m3_top_bits(uint32_t w) { return ((w & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u; }
+__device__ inline uint32_t e4m3_halve4(uint32_t w) {
+    const uint32_t mag = w & 0x7F7F7F7Fu, sign = w & 0x80808080u;
+    const uint32_t big = (((mag + 0x70707070u) & 0x80808080u) >> 7) * 0xFFu;      // all ones in the bytes with mag >= 16
+    const uint32_t mag_n = ((mag | 0x80808080u) - 0x08080808u) & 0x7F7F7F7Fu;     // exponent field - 1 (the guard bit stops the borrow)
+    const uint32_t q = (mag >> 1) & 0x7F7F7F7Fu;
+    const uint32_t mag_s = q + (mag & q & 0x01010101u);                           // mag / 2, half to even
+    return sign | (big & mag_n) | (~big & mag_s);
+}
+// one code of format F as the E4M3 byte of the same value
+template <class F>
+__device__ inline uint32_t embed_e4m3(uint32_t c, const F& f) {
+    constexpr int E = F{}.E(), M = F{}.M(), bias = (1 << (E - 1)) - 1;
+    if constexpr (E == 4 && M == 3) return c & 0xFFu;
+    const uint32_t s = (c >> (E + M)) & 1u, e = (c >> M) & ((1u << E) - 1u), fr = c & ((1u << M) - 1u);
+    uint32_t mag = 0;
+    if (e != 0) mag = ((e + 7 - bias) << 3) | (fr << (3 - M));
+    else if (fr != 0) {
+        const int p = 31 - __clz(fr);   // value 2^(p - M + 1 - bias) * (1 + rest / 2^p)
+        mag = ((uint32_t)(p - M + 8 - bias) << 3) | ((fr << (3 - p)) & 7u);
+    }
+    return (s << 7) | mag;
+}
+template <class F>
+__device__ inline uint32_t embed_e4m3_x4(uint32_t w, const F& f) {
+    return embed_e4m3(w & 0xFFu, f) | (embed_e4m3((w >> 8) & 0xFFu, f) << 8) | (embed_e4m3((w >> 16) & 0xFFu, f) << 16) |
+           (embed_e4m3(w >> 24, f) << 24);
+}
+// where the scale byte of block `b0 + i` goes: b0 = (row0, kb0) is uniform, i small; kblocks = K / 32
+struct ScaledGeom {
+    uint32_t kblocks, rows_pad;
+    float inv_kblocks;
+};
+__device__ inline size_t scaled_scale_offset(uint32_t row0, uint32_t kb0, uint32_t i, const ScaledGeom& g) {
+    const uint32_t x = kb0 + i;   // below 2^23: exact in fp32
+    uint32_t q = (uint32_t)((float)x * g.inv_kblocks);
+    int32_t r = (int32_t)(x - q * g.kblocks);
+    if (r < 0) { r += (int32_t)g.kblocks; --q; }
+    else if (r >= (int32_t)g.kblocks) { r -= (int32_t)g.kblocks; ++q; }
+    return ((size_t)((uint32_t)r >> 2) * g.rows_pad + row0 + q) * 4 + ((uint32_t)r & 3u);
+}
+
+// MODE 0: extract (scales + elements); MODE 1: fused quantise-dequantise to bf16; MODE 2: extract as an operand of the
+// block-scaled GEMM (E4M3 bytes without the NaN code, scales transposed)
 template <class F, int UNROLL, int MODE>
 __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __restrict__ x, uint8_t* __restrict__ scales,
                                                                   uint2* __restrict__ elements, uint4* __restrict__ out,
-                                                                  int64_t n_chunks, F f) {
+                                                                  int64_t n_chunks, F f, ScaledGeom sg) {
     const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
+    uint32_t sg_row0 = 0, sg_kb0 = 0;
+    if constexpr (MODE == 2) {   // (row, k block) of the workgroup's first block
+        const uint32_t b0 = blockIdx.x * (uint32_t)(UNROLL * kThreads / 4);
+        sg_row0 = b0 / sg.kblocks;
+        sg_kb0 = b0 - sg_row0 * sg.kblocks;
+    }
     uint4 raw[UNROLL];
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
@@ -455,7 +511,7 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
             const uint32_t ssb = (uint32_t)((scale_n - fmt_bias(f)) << 7) & 0xFFFFu;
             const uint32_t ssb2 = ssb | (ssb << 16);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) o[j] = MODE == 0 ? PackedBf16<F>::codes(h[j], ssb2) : PackedBf16<F>::qdq(h[j], ssb2);
+            for (int j = 0; j < 4; ++j) o[j] = MODE != 1 ? PackedBf16<F>::codes(h[j], ssb2) : PackedBf16<F>::qdq(h[j], ssb2);
         } else {
             // exact per-element routine (the block's lanes agree on amax, so they agree on the result)
             const uint32_t amax32 = amax << 16;
@@ -465,7 +521,7 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t c0 = encode_mxfp_element(h[j] << 16, se, f), c1 = encode_mxfp_element(h[j] & 0xFFFF0000u, se, f);
-                o[j] = MODE == 0 ? (c0 | (c1 << 16)) : pack_bf16(mxfp_value(c0, sc, f), mxfp_value(c1, sc, f));
+                o[j] = MODE != 1 ? (c0 | (c1 << 16)) : pack_bf16(mxfp_value(c0, sc, f), mxfp_value(c1, sc, f));
             }
         }
         if (c < n_chunks) {
@@ -473,8 +529,28 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
                 // o[j] holds two codes in the low bytes of its halves: gather the 8 code bytes
                 st64(elements + c, make_uint2(__builtin_amdgcn_perm(o[1], o[0], 0x06040200u), __builtin_amdgcn_perm(o[3], o[2], 0x06040200u)));
                 if ((c & 3) == 0) scales[c >> 2] = (uint8_t)scale;
-            } else {
+            } else if (MODE == 1) {
                 st128(out + c, make_uint4(o[0], o[1], o[2], o[3]));
+            }
+        }
+        if constexpr (MODE == 2) {
+            uint32_t w0 = __builtin_amdgcn_perm(o[1], o[0], 0x06040200u), w1 = __builtin_amdgcn_perm(o[3], o[2], 0x06040200u);
+            if constexpr (F{}.E() == 4 && F{}.M() == 3) {
+                uint32_t top = e4m3_top_bits(w0) | e4m3_top_bits(w1);
+                top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xF, 0xF, true);
+                top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0x4E, 0xF, 0xF, true);
+                if (top != 0u && scale < 254u) {   // (a block of scale 255 holds inf / NaN: its row of the product is NaN either way)
+                    w0 = e4m3_halve4(w0);
+                    w1 = e4m3_halve4(w1);
+                    scale += 1u;
+                }
+            } else {
+                w0 = embed_e4m3_x4(w0, f);
+                w1 = embed_e4m3_x4(w1, f);
+            }
+            if (c < n_chunks) {
+                st64(elements + c, make_uint2(w0, w1));
+                if ((c & 3) == 0) scales[scaled_scale_offset(sg_row0, sg_kb0, (uint32_t)((threadIdx.x + r * kThreads) >> 2), sg)] = (uint8_t)scale;
             }
         }
     }
@@ -872,6 +948,34 @@ __global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_lines_kernel(const
     }
 }
 
+// MXFP components (reference layout: one code byte per element, scales [rows, K / 32]) -> operand of the block-scaled
+// GEMM.  A lane owns 16 codes, two adjacent lanes a block.
+template <class F>
+__global__ __launch_bounds__(kThreads) void scaled_operand_kernel(const uint8_t* __restrict__ scales, const uint4* __restrict__ elements,
+                                                                   uint4* __restrict__ out_codes, uint8_t* __restrict__ out_scales,
+                                                                   int64_t n_chunks, F f, ScaledGeom sg) {
+    const uint32_t b0 = blockIdx.x * (uint32_t)(kThreads / 2);
+    const uint32_t row0 = b0 / sg.kblocks, kb0 = b0 - row0 * sg.kblocks;
+    const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const bool live = c < n_chunks;
+    uint4 w = live ? ld128(elements + c) : make_uint4(0, 0, 0, 0);
+    uint32_t scale = live ? (uint32_t)scales[c >> 1] : 0u;
+    if constexpr (F{}.E() == 4 && F{}.M() == 3) {
+        uint32_t top = e4m3_top_bits(w.x) | e4m3_top_bits(w.y) | e4m3_top_bits(w.z) | e4m3_top_bits(w.w);
+        top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xF, 0xF, true);  // lane ^ 1
+        if (top != 0u && scale < 254u) {
+            w = make_uint4(e4m3_halve4(w.x), e4m3_halve4(w.y), e4m3_halve4(w.z), e4m3_halve4(w.w));
+            scale += 1u;
+        }
+    } else {
+        w = make_uint4(embed_e4m3_x4(w.x, f), embed_e4m3_x4(w.y, f), embed_e4m3_x4(w.z, f), embed_e4m3_x4(w.w, f));
+    }
+    if (live) {
+        st128(out_codes + c, w);
+        if ((c & 1) == 0) out_scales[scaled_scale_offset(row0, kb0, threadIdx.x >> 1, sg)] = (uint8_t)scale;
+    }
+}
+
 // ------------------------------------------------------------------------------ launch helpers
 inline unsigned grid_for(int64_t items, int per_block) {
     return (unsigned)((items + per_block - 1) / per_block);
@@ -1011,7 +1115,7 @@ int mase_hip_extract_mxfp(const void* x, int x_dtype, uint8_t* scales, uint8_t* 
             if (x_dtype == BF16 && B == 32 && vec) {
                 constexpr int U = MASE_UNROLL_PACKED;
                 hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 0>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
-                                   static_cast<const uint4*>(x), scales, reinterpret_cast<uint2*>(elements), nullptr, n / 8, f);
+                                   static_cast<const uint4*>(x), scales, reinterpret_cast<uint2*>(elements), nullptr, n / 8, f, ScaledGeom{});
                 return check_launch("extract_mxfp");
             }
         }
@@ -1079,7 +1183,7 @@ int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int6
             if (x_dtype == BF16 && out_dtype == BF16 && B == 32 && vec) {
                 constexpr int U = MASE_UNROLL_PACKED;
                 hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 1>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
-                                   static_cast<const uint4*>(x), nullptr, nullptr, static_cast<uint4*>(out), n / 8, f);
+                                   static_cast<const uint4*>(x), nullptr, nullptr, static_cast<uint4*>(out), n / 8, f, ScaledGeom{});
                 return check_launch("qdq_mxfp");
             }
         }
@@ -1198,5 +1302,60 @@ int mase_hip_qdq_mxfp_strided(const void* x, int x_dtype, void* out, int out_dty
     });
 }
 
+// ---- operands of the block-scaled GEMM (mase_hip_mxfp_gemm_scaled)
+int64_t mase_hip_scaled_padded_rows(int64_t rows) { return rows <= 0 ? 0 : (rows + 255) / 256 * 256; }
+
+static int scaled_operand_args(int64_t rows, int64_t K, int exp_bits, int frac_bits, ScaledGeom& sg) {
+    if (rows < 1 || K < 1) return fail(ERR_INVALID, "rows and K must be positive");
+    if (K % 128 != 0) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM needs K to be a multiple of 128");
+    if (K >= ((int64_t)1 << 27) || rows * (K / 32) >= ((int64_t)1 << 31)) return fail(ERR_UNSUPPORTED, "operand too large for the block-scaled GEMM");
+    const bool ok = (exp_bits == 4 && frac_bits == 3) || (exp_bits == 2 && frac_bits == 3) || (exp_bits == 3 && frac_bits == 2) ||
+                    (exp_bits == 2 && frac_bits == 1);
+    if (!ok) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM takes element formats (4,3) (2,3) (3,2) (2,1)");
+    sg.kblocks = (uint32_t)(K / 32);
+    sg.rows_pad = (uint32_t)mase_hip_scaled_padded_rows(rows);
+    sg.inv_kblocks = 1.0f / (float)sg.kblocks;
+    return OK;
+}
+
+int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elements, int exp_bits, int frac_bits, int64_t rows, int64_t K,
+                                      uint8_t* out_codes, uint32_t* out_scales, void* stream) {
+    ScaledGeom sg;
+    if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, sg)) return rc;
+    if (!scales || !elements || !out_codes || !out_scales) return fail(ERR_INVALID, "null pointer");
+    if (!aligned(elements, 16) || !aligned(out_codes, 16) || !aligned(out_scales, 4)) return fail(ERR_INVALID, "elements and out_codes must be 16-byte aligned, out_scales 4-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t n_chunks = rows * K / 16;
+    return dispatch_fmt(exp_bits, frac_bits, 1, RN, [&](auto f) {
+        if constexpr (decltype(f)::kStatic && decltype(f){}.E() != 5) {
+            hipLaunchKernelGGL((scaled_operand_kernel<decltype(f)>), dim3(grid_for(n_chunks, kThreads)), dim3(kThreads), 0, s, scales,
+                               reinterpret_cast<const uint4*>(elements), reinterpret_cast<uint4*>(out_codes), reinterpret_cast<uint8_t*>(out_scales),
+                               n_chunks, f, sg);
+            return check_launch("scaled_operand_from_mxfp");
+        }
+        return fail(ERR_UNSUPPORTED, "element format not supported by the block-scaled GEMM");
+    });
+}
+
+int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
+                                       uint32_t* out_scales, void* stream) {
+    ScaledGeom sg;
+    if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, sg)) return rc;
+    if (x_dtype != BF16) return fail(ERR_UNSUPPORTED, "a dense operand of the block-scaled GEMM must be bfloat16");
+    if (!x || !out_codes || !out_scales) return fail(ERR_INVALID, "null pointer");
+    if (!aligned(x, 16) || !aligned(out_codes, 8) || !aligned(out_scales, 4)) return fail(ERR_INVALID, "x must be 16-byte aligned, out_codes 8-byte, out_scales 4-byte");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t n = rows * K;
+    return dispatch_fmt(exp_bits, frac_bits, 1, RN, [&](auto f) {
+        if constexpr (decltype(f)::kStatic && decltype(f){}.E() != 5) {
+            constexpr int U = MASE_UNROLL_PACKED;
+            hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 2>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
+                               static_cast<const uint4*>(x), reinterpret_cast<uint8_t*>(out_scales), reinterpret_cast<uint2*>(out_codes), nullptr,
+                               n / 8, f, sg);
+            return check_launch("scaled_operand_from_dense");
+        }
+        return fail(ERR_UNSUPPORTED, "element format not supported by the block-scaled GEMM");
+    });
+}
 
 }  // extern "C"

@@ -329,6 +329,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 }
 
 #include "gemm_tall.h"
+#include "gemm_scaled.h"
 #include "gemm_skinny.h"
 #include "gemm_rows16.h"
 #include "gemm_mid.h"

@@ -1,0 +1,380 @@
+// Block-scaled MXFP GEMM for gfx950:  y[M,N] = A[M,K] * W[N,K]^T (+ bias) on v_mfma_scale_f32_16x16x128_f8f6f4.
+//
+// Both operands stay MXFP all the way into the matrix unit: one FP8 (E4M3) code per element and one E8M0 scale per
+// 32 elements along K, which the instruction applies itself.  Nothing is composed to bf16, no operand byte passes
+// through a VGPR on its way to LDS, and an operand row costs one byte per element of LDS and L2 traffic instead of two.
+// The operands come from the prepare kernels (scaled_prepare.hip), which
+//   * re-encode every block that holds the code S.1111.111 one scale step up (the instruction reads that code as NaN,
+//     the reference as +-480) and embed the narrower element formats into E4M3 bytes (exact),
+//   * pad the rows to a multiple of 256 and store the scales transposed: dword [K/128][rows], the four bytes of a dword
+//     being the scales of the four 32-k blocks of one 128-k macro step of one row.
+//
+// What the instruction expects (measured with a one-wavefront probe): lane l = 16 g + r supplies row r of a 16-row
+// operand tile; its first 16 bytes are k 16 g .. 16 g + 15 and its second 16 bytes k 64 + 16 g .. 64 + 16 g + 15 of the
+// 128 k; byte `opsel` of its scale register is the scale of k block g (k 32 g .. 32 g + 31) of that row.  The first
+// operand's rows are the result's rows in lane groups of four (c[4 (l >> 4) + v][l & 15] in element v), so W is fed
+// first and a lane ends up with four consecutive n of one m, as in the bf16 kernels.
+//
+// Tile 256 x 256, four wavefronts 2 x 2, each 128 x 128 (8 x 8 MFMA tiles, 256 accumulator AGPRs), macro steps of 128 k.
+// A macro step is worked off in two periods of four m-tiles (32 MFMAs); the eight W fragments of a macro step live in
+// registers (they are read from LDS during the macro step before).  The data of one period is a "chunk": 128 rows of A
+// (the period's four m-tiles of both wave rows) and 128 rows of W (four n-tiles of the NEXT macro step, both wave
+// columns), 16 KB each, plus 1 KB of scales, all by DMA (global_load_lds).  LDS holds a ring of four chunks:
+//
+//   period c    multiplies chunk c's A rows, reads chunk c's W rows into the registers of the next macro step,
+//               and issues the DMAs of chunk c + 3 (into the slot that chunk c - 1 left), spread over the period
+//   barrier c+1 sits before the last eight MFMAs of period c: every wave has finished reading chunk c, and has waited
+//               until its own DMAs of chunk c + 1 (issued two periods earlier: vmcnt(18)) have landed
+//
+// so a DMA has between two and three periods (2000 - 3000 cycles) to land and the address unit sees an even stream.
+// (included from gemm_impl.h's namespace, after gemm_tall.h whose asm helpers it shares)
+
+constexpr int SM = 256, SN = 256, SMAC = 128;
+constexpr int S_RING = 4;
+constexpr int S_PART_BYTES = 128 * 128;                       // 128 rows of one operand, 128 k
+constexpr int S_A_OFF = 0;                                    // [4 chunks][128 rows][128 B]
+constexpr int S_W_OFF = S_RING * S_PART_BYTES;                // the same for W: both below 64 KB offsets from their base
+constexpr int S_SC_OFF = 2 * S_RING * S_PART_BYTES;           // [4 chunks][4 waves][64 dwords]: 32 A rows, 32 W rows per wave
+constexpr int S_SC_BYTES = 1024;
+constexpr int S_OUT_OFF = S_SC_OFF + S_RING * S_SC_BYTES;     // [4 waves][32 rows][128 B] output staging
+constexpr int S_LDS_BYTES = S_OUT_OFF + 4 * 4096;             // 148 KB
+
+typedef int intx8 __attribute__((ext_vector_type(8)));
+
+// c += w (16 n x 128 k, scales sw) * a (16 m x 128 k, scales sa)^T
+__device__ inline void mfma_scaled(floatx4& c, const intx8& w, const intx8& a, uint32_t sw, uint32_t sa) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]" : "+a"(c) : "v"(w), "v"(a), "v"(sw), "v"(sa));
+}
+__device__ inline void mfma_scaled_first(floatx4& c, const intx8& w, const intx8& a, uint32_t sw, uint32_t sa) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel_hi:[0,0,0]" : "=a"(c) : "v"(w), "v"(a), "v"(sw), "v"(sa));
+}
+// 64 lanes x 4 bytes from per-lane 64-bit addresses to LDS [lds_addr, lds_addr + 256)
+__device__ inline void dma_dwords(uint32_t lds_addr, const void* lane_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(lane_addr) : "memory");
+}
+
+// 16 bytes to a per-lane address (non-temporal: the output is not read again by this kernel); the trailing s_nop keeps a
+// following VALU write of the data registers out of the store's read window
+__device__ inline void store16_nt(void* dst, const u32x4& v) {
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 0" ::"v"(dst), "v"(v) : "memory");
+}
+
+struct ScaledTile {
+    const uint8_t* a;    // codes of the tile's first A row
+    const uint8_t* w;    // codes of the tile's first W row
+    const uint32_t* as;  // scale dword of the tile's first A row, macro step 0
+    const uint32_t* ws;
+    int m0, n0;
+};
+
+template <int DT_OUT>
+__global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_scaled_kernel(
+    const uint8_t* __restrict__ a_codes, const uint32_t* __restrict__ a_scales, const uint8_t* __restrict__ w_codes,
+    const uint32_t* __restrict__ w_scales, const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K,
+    int rows_a, int rows_w, int tiles_m, int tiles_n) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int nmac = K / SMAC;   // even and at least 4 (the launcher checks)
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+    // ---- per-lane constants
+    // data DMA d (0..3) of a wave covers rows 32 wave + 8 d .. + 7 of a chunk part; lane l fills position l & 7 of row
+    // 8 d + (l >> 3), which must hold the row's 16-byte piece (l & 7) ^ (row >> 1 & 7) = (l & 7) ^ ((4 d + (l >> 4)) & 7)
+    const uint32_t dma_voff_even = (uint32_t)(lane >> 3) * (uint32_t)K + (uint32_t)((((lane & 7) ^ (lane >> 4)) & 7) << 4);
+    const uint32_t dma_voff_odd = dma_voff_even ^ 64u;
+    // fragment reads: lane (g = l >> 4, r = l & 15) reads pieces g and g + 4 of row r of its 16-row tile
+    const uint32_t f_off = (uint32_t)(lane & 15) * 128u + (uint32_t)((((lane >> 4) ^ ((lane >> 1) & 7)) & 7) << 4);
+    const uint8_t* const a_frag0 = lds + S_A_OFF + wave_m * (64 * 128) + f_off;
+    const uint8_t* const a_frag1 = lds + S_A_OFF + wave_m * (64 * 128) + (f_off ^ 64u);
+    const uint8_t* const w_frag0 = lds + S_W_OFF + wave_n * (64 * 128) + f_off;
+    const uint8_t* const w_frag1 = lds + S_W_OFF + wave_n * (64 * 128) + (f_off ^ 64u);
+    // scale bytes: the dword of chunk row q sits at (q >> 5) * 256 + (q & 31) * 4 (A) or + 128 (W); a lane wants byte g
+    const uint8_t* const a_sc = lds + S_SC_OFF + wave_m * 512 + (lane & 15) * 4 + (lane >> 4);
+    const uint8_t* const w_sc = lds + S_SC_OFF + wave_n * 512 + 128 + (lane & 15) * 4 + (lane >> 4);
+
+    const int n_tiles = tiles_m * tiles_n;
+    const int per_xcd = (n_tiles + 7) >> 3;
+    const int slots = gridDim.x >> 3;
+    auto has_tile = [&](int local) __attribute__((always_inline)) { return local < per_xcd && (int)(blockIdx.x & 7) * per_xcd + local < n_tiles; };
+    auto tile_at = [&](int local) __attribute__((always_inline)) {
+        const int pos = (blockIdx.x & 7) * per_xcd + local;
+        // groups of 4 tile rows, rows fastest: the 32 tiles an XCD runs at once form a 4 x 8 patch
+        constexpr int GROUP = 4;
+        const int in_group = GROUP * tiles_n;
+        const int first_m = (pos / in_group) * GROUP;
+        const int rows = min(tiles_m - first_m, GROUP);
+        const int rr = pos % in_group;
+        ScaledTile t;
+        t.m0 = (first_m + rr % rows) * SM;
+        t.n0 = (rr / rows) * SN;
+        t.a = a_codes + (size_t)t.m0 * K;
+        t.w = w_codes + (size_t)t.n0 * K;
+        t.as = a_scales + t.m0;
+        t.ws = w_scales + t.n0;
+        return t;
+    };
+
+    int local = blockIdx.x >> 3;
+    if (!has_tile(local)) return;
+    ScaledTile cur = tile_at(local), next = cur;
+
+    // ---- DMAs of the chunk (macro step ma of A, macro step ma + 1 of W, half h) into ring slot `slot`; ma may run past
+    //      the tile's end, into the next tile.  PART 0..2: three of the nine operations each.
+    const int rows_in_part = 32 * wave;   // this wave's first row within a chunk part
+    auto issue_chunk = [&](int ma, int h, int slot, auto part_c) __attribute__((always_inline)) {
+        constexpr int PART = decltype(part_c)::value;
+        const bool a_wrap = ma >= nmac;
+        const int mw = ma + 1;
+        const bool w_wrap = mw >= nmac;
+        const ScaledTile& ta = a_wrap ? next : cur;
+        const ScaledTile& tw = w_wrap ? next : cur;
+        const int ma_t = a_wrap ? ma - nmac : ma, mw_t = w_wrap ? mw - nmac : mw;
+        // the wave's 32 rows of the part are tile rows 128 (wave >> 1) + 64 h + 32 (wave & 1) ..
+        const int row0 = 128 * (wave >> 1) + 64 * h + 32 * (wave & 1);
+        const uint8_t* const a_src = ta.a + (size_t)row0 * K + (size_t)ma_t * SMAC;
+        const uint8_t* const w_src = tw.w + (size_t)row0 * K + (size_t)mw_t * SMAC;
+        const uint32_t lds_a = lds_base + S_A_OFF + slot * S_PART_BYTES + rows_in_part * 128;
+        const uint32_t lds_w = lds_base + S_W_OFF + slot * S_PART_BYTES + rows_in_part * 128;
+        if constexpr (PART == 0) {
+            dma_1kb(lds_a, dma_voff_even, a_src);
+            dma_1kb(lds_a + 1024, dma_voff_odd, a_src + (size_t)8 * K);
+            dma_1kb(lds_a + 2048, dma_voff_even, a_src + (size_t)16 * K);
+        } else if constexpr (PART == 1) {
+            dma_1kb(lds_a + 3072, dma_voff_odd, a_src + (size_t)24 * K);
+            dma_1kb(lds_w, dma_voff_even, w_src);
+            dma_1kb(lds_w + 1024, dma_voff_odd, w_src + (size_t)8 * K);
+        } else {
+            dma_1kb(lds_w + 2048, dma_voff_even, w_src + (size_t)16 * K);
+            dma_1kb(lds_w + 3072, dma_voff_odd, w_src + (size_t)24 * K);
+            // scales: lanes 0..31 the dwords of the wave's 32 A rows, lanes 32..63 those of its 32 W rows
+            const uint32_t* const sp = lane < 32 ? ta.as + (size_t)ma_t * rows_a + row0 + lane : tw.ws + (size_t)mw_t * rows_w + row0 + (lane - 32);
+            dma_dwords(lds_base + S_SC_OFF + slot * S_SC_BYTES + wave * 256, sp);
+        }
+    };
+    // the W half of a chunk alone (the first tile's first macro step of W travels in two chunks of its own)
+    auto issue_w_only = [&](int mw_t, int h, int slot) __attribute__((always_inline)) {
+        const int row0 = 128 * (wave >> 1) + 64 * h + 32 * (wave & 1);
+        const uint8_t* const w_src = cur.w + (size_t)row0 * K + (size_t)mw_t * SMAC;
+        const uint32_t lds_w = lds_base + S_W_OFF + slot * S_PART_BYTES + rows_in_part * 128;
+        dma_1kb(lds_w, dma_voff_even, w_src);
+        dma_1kb(lds_w + 1024, dma_voff_odd, w_src + (size_t)8 * K);
+        dma_1kb(lds_w + 2048, dma_voff_even, w_src + (size_t)16 * K);
+        dma_1kb(lds_w + 3072, dma_voff_odd, w_src + (size_t)24 * K);
+        const uint32_t* const sp = cur.ws + (size_t)mw_t * rows_w + row0 + (lane & 31);   // lanes 0..31 land where nobody looks
+        dma_dwords(lds_base + S_SC_OFF + slot * S_SC_BYTES + wave * 256, sp);
+    };
+
+    floatx4 acc[8][8];        // [n-tile j][m-tile i]
+    intx8 wreg[2][8];         // the W fragments of the macro step in flight and of the next one
+    uint32_t wsc[2][8];       // their scale bytes
+    intx8 areg[2];            // A fragment ring
+    uint32_t asc[2][4];       // scale bytes of the period's four m-tiles, and of the next period's
+
+    // fragment t (0..3) of ring slot `slot`
+    auto read_a = [&](intx8& dst, int slot, int t) __attribute__((always_inline)) {
+        const uint4 lo = *reinterpret_cast<const uint4*>(a_frag0 + slot * S_PART_BYTES + t * 2048);
+        const uint4 hi = *reinterpret_cast<const uint4*>(a_frag1 + slot * S_PART_BYTES + t * 2048);
+        dst = intx8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+    };
+    auto read_w = [&](intx8& dst, uint32_t& sc, int slot, int t) __attribute__((always_inline)) {
+        const uint4 lo = *reinterpret_cast<const uint4*>(w_frag0 + slot * S_PART_BYTES + t * 2048);
+        const uint4 hi = *reinterpret_cast<const uint4*>(w_frag1 + slot * S_PART_BYTES + t * 2048);
+        dst = intx8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        sc = w_sc[slot * S_SC_BYTES + (t >> 1) * 256 + (t & 1) * 64];
+    };
+    auto read_a_scales = [&](uint32_t(&dst)[4], int slot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) dst[t] = a_sc[slot * S_SC_BYTES + (t >> 1) * 256 + (t & 1) * 64];
+    };
+
+    // ---- prologue of the stream: W macro step 0 of the first tile through slots 2 and 3, chunks 0 and 1, then chunk 2
+    issue_w_only(0, 0, 2);
+    issue_w_only(0, 1, 3);
+    issue_chunk(0, 0, 0, IntC<0>{});
+    issue_chunk(0, 0, 0, IntC<1>{});
+    issue_chunk(0, 0, 0, IntC<2>{});
+    issue_chunk(0, 1, 1, IntC<0>{});
+    issue_chunk(0, 1, 1, IntC<1>{});
+    issue_chunk(0, 1, 1, IntC<2>{});
+    asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        read_w(wreg[0][t], wsc[0][t], 2, t);
+        read_w(wreg[0][4 + t], wsc[0][4 + t], 3, t);
+    }
+    lds_barrier();   // slots 2 and 3 are free again
+    issue_chunk(1, 0, 2, IntC<0>{});
+    issue_chunk(1, 0, 2, IntC<1>{});
+    issue_chunk(1, 0, 2, IntC<2>{});
+    asm volatile("s_waitcnt vmcnt(18)" ::: "memory");   // chunk 0 has landed
+    __builtin_amdgcn_s_barrier();
+    read_a(areg[0], 0, 0);
+    read_a_scales(asc[0], 0);
+
+    // One period: H = half of the macro step (m-tiles 4 H .. 4 H + 3), C4 = ring slot of its chunk, WC = register set of
+    // the macro step's W fragments.  ma = macro step (of the current tile).
+    auto period = [&](int ma, auto h_c, auto c4_c, auto wc_c, auto first_c) __attribute__((always_inline)) {
+        constexpr int H = decltype(h_c)::value, C4 = decltype(c4_c)::value, WC = decltype(wc_c)::value;
+        constexpr bool FIRST = decltype(first_c)::value != 0;
+        constexpr int WN = WC ^ 1, NEXT_SLOT = (C4 + 1) & 3, ISSUE_SLOT = (C4 + 3) & 3;
+        constexpr int AS = H, ASN = H ^ 1;   // scale register set of this period, of the next
+        // the chunk issued during this period: three periods ahead
+        const int issue_ma = H == 0 ? ma + 1 : ma + 2;
+        constexpr int issue_h = H ^ 1;
+        auto mm8 = [&](const intx8& a, uint32_t sa, auto i_c) __attribute__((always_inline)) {
+            constexpr int i = decltype(i_c)::value;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (FIRST) mfma_scaled_first(acc[j][i], wreg[WC][j], a, wsc[WC][j], sa);
+                else mfma_scaled(acc[j][i], wreg[WC][j], a, wsc[WC][j], sa);
+            }
+        };
+#define S_SLOT_END() __builtin_amdgcn_sched_barrier(0)
+        // row 0
+        read_a(areg[1], C4, 1);
+        read_w(wreg[WN][4 * H + 0], wsc[WN][4 * H + 0], C4, 0);
+        read_w(wreg[WN][4 * H + 1], wsc[WN][4 * H + 1], C4, 1);
+        issue_chunk(issue_ma, issue_h, ISSUE_SLOT, IntC<0>{});
+        S_SLOT_END();
+        mm8(areg[0], asc[AS][0], IntC<4 * H + 0>{});
+        S_SLOT_END();
+        // row 1
+        read_a(areg[0], C4, 2);
+        read_w(wreg[WN][4 * H + 2], wsc[WN][4 * H + 2], C4, 2);
+        issue_chunk(issue_ma, issue_h, ISSUE_SLOT, IntC<1>{});
+        S_SLOT_END();
+        mm8(areg[1], asc[AS][1], IntC<4 * H + 1>{});
+        S_SLOT_END();
+        // row 2
+        read_a(areg[1], C4, 3);
+        read_w(wreg[WN][4 * H + 3], wsc[WN][4 * H + 3], C4, 3);
+        issue_chunk(issue_ma, issue_h, ISSUE_SLOT, IntC<2>{});
+        S_SLOT_END();
+        mm8(areg[0], asc[AS][2], IntC<4 * H + 2>{});
+        S_SLOT_END();
+        // row 3: the next chunk has landed everywhere, this one is no longer read
+        asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+        lds_barrier();
+        read_a(areg[0], NEXT_SLOT, 0);
+        read_a_scales(asc[ASN], NEXT_SLOT);
+        S_SLOT_END();
+        mm8(areg[1], asc[AS][3], IntC<4 * H + 3>{});
+        S_SLOT_END();
+#undef S_SLOT_END
+    };
+
+    for (;;) {
+        const int next_local = local + slots;
+        const bool more = has_tile(next_local);
+        if (more) next = tile_at(next_local);  // else the look-ahead re-reads this tile's first operands (unused)
+
+        // macro steps in pairs: the register sets of W and the ring slots alternate at compile time
+        period(0, IntC<0>{}, IntC<0>{}, IntC<0>{}, IntC<1>{});
+        period(0, IntC<1>{}, IntC<1>{}, IntC<0>{}, IntC<1>{});
+        period(1, IntC<0>{}, IntC<2>{}, IntC<1>{}, IntC<0>{});
+        period(1, IntC<1>{}, IntC<3>{}, IntC<1>{}, IntC<0>{});
+        for (int ma = 2; ma < nmac; ma += 2) {
+            period(ma, IntC<0>{}, IntC<0>{}, IntC<0>{}, IntC<0>{});
+            period(ma, IntC<1>{}, IntC<1>{}, IntC<0>{}, IntC<0>{});
+            period(ma + 1, IntC<0>{}, IntC<2>{}, IntC<1>{}, IntC<0>{});
+            period(ma + 1, IntC<1>{}, IntC<3>{}, IntC<1>{}, IntC<0>{});
+        }
+
+        // ---- output: lane holds, for tile (j, i), y[m][n .. n+3] with m = m0 + 128 wave_m + 16 i + lane % 16,
+        //      n = n0 + 128 wave_n + 16 j + 4 (lane / 16); staged through LDS so that a store instruction writes whole lines
+        uint8_t* const lds_out = lds + S_OUT_OFF + wave * 4096;
+        const int row_base = cur.m0 + wave_m * 128, col_base = cur.n0 + wave_n * 128;
+        uint32_t ol = (uint32_t)lane;
+        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(ol));  // also: the last MFMA results are readable after this
+        const uint32_t o_row = ol & 15u, o_q = ol >> 4;
+        const uint32_t o_rd_off = (ol >> 3) * 128u + (((ol & 7u) ^ (ol >> 3)) * 16u);
+        auto write_tile = [&](auto has_bias_c) __attribute__((always_inline)) {
+            constexpr bool HAS_BIAS = decltype(has_bias_c)::value != 0;
+            float bv[2] = {0.0f, 0.0f};
+            if (HAS_BIAS) {
+                bv[0] = col_base + (int)ol < N ? load_bias(bias, bias_dtype, col_base + (int)ol) : 0.0f;
+                bv[1] = col_base + 64 + (int)ol < N ? load_bias(bias, bias_dtype, col_base + 64 + (int)ol) : 0.0f;
+            }
+            auto values = [&](auto j_c, auto i_c, float(&r)[4]) {
+                constexpr int j = decltype(j_c)::value, i = decltype(i_c)::value;
+                static_for<4>([&](auto t_c) __attribute__((always_inline)) {
+                    constexpr int t = decltype(t_c)::value;
+                    r[t] = acc_read(acc[j][i][t]);
+                    if (HAS_BIAS) {
+                        const int src = (int)(((uint32_t)(16 * j + t) + 4u * o_q) & 63u);
+                        r[t] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src * 4, __builtin_bit_cast(int, bv[j >> 2])));
+                    }
+                });
+            };
+            constexpr int OB = DT_OUT == F32 ? 4 : 2;           // bytes per output
+            constexpr int PASS_COLS = 128 / OB;                 // columns of a 128-byte staged row: 32 (fp32) or 64
+            constexpr int NPASS_J = 128 / PASS_COLS;            // passes across the wave's 128 columns
+            constexpr int JT = PASS_COLS / 16;                  // n-tiles per pass
+            // store: lane covers 16 bytes (16 / OB columns) of row (ol >> 3) of each 8-row group
+            const int st_col = col_base + (int)(ol & 7u) * (16 / OB);
+            static_for<4>([&](auto ip_c) __attribute__((always_inline)) {
+                static_for<NPASS_J>([&](auto jp_c) __attribute__((always_inline)) {
+                    constexpr int ip = decltype(ip_c)::value, jp = decltype(jp_c)::value;
+                    static_for<2 * JT>([&](auto x_c) __attribute__((always_inline)) {
+                        constexpr int ii = decltype(x_c)::value / JT, jj = decltype(x_c)::value % JT;
+                        float r[4];
+                        values(IntC<JT * jp + jj>{}, IntC<2 * ip + ii>{}, r);
+                        const uint32_t row = 16u * ii + o_row;
+                        if constexpr (DT_OUT == F32) {
+                            const uint32_t chunk = ((uint32_t)(4 * jj) + o_q) ^ (row & 7u);
+                            *reinterpret_cast<uint4*>(lds_out + row * 128u + chunk * 16u) = make_uint4(f32_bits(r[0]), f32_bits(r[1]), f32_bits(r[2]), f32_bits(r[3]));
+                        } else {
+                            const uint2 p = pack_out4<DT_OUT>(r[0], r[1], r[2], r[3]);
+                            const uint32_t chunk = ((uint32_t)(2 * jj) + (o_q >> 1)) ^ (row & 7u);
+                            *reinterpret_cast<uint2*>(lds_out + row * 128u + chunk * 16u + (o_q & 1u) * 8u) = p;
+                        }
+                    });
+                    u32x4 v[4];
+                    static_for<4>([&](auto t_c) __attribute__((always_inline)) {
+                        constexpr int t = decltype(t_c)::value;
+                        v[t] = *reinterpret_cast<const u32x4*>(lds_out + o_rd_off + t * 1024);
+                    });
+                    static_for<4>([&](auto t_c) __attribute__((always_inline)) {
+                        constexpr int t = decltype(t_c)::value;
+                        const int row = row_base + ip * 32 + 8 * t + (int)(ol >> 3);
+                        const int col = st_col + jp * PASS_COLS;
+                        if (row < M && col < N) {
+                            uint8_t* const dst = static_cast<uint8_t*>(y) + ((size_t)row * N + col) * OB;
+                            store16_nt(dst, v[t]);
+                        }
+                    });
+                    __builtin_amdgcn_sched_barrier(0);  // one pass at a time
+                });
+            });
+        };
+        if (bias) write_tile(IntC<1>{});
+        else write_tile(IntC<0>{});
+
+        if (!more) break;
+        cur = next;
+        local = next_local;
+    }
+    // the look-ahead DMAs of the last periods still target LDS: let them finish
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// a_codes [rows_a, K], w_codes [rows_w, K]: rows padded to multiples of 256; scales [K / 128][rows] dwords
+template <int DT_OUT>
+int launch_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
+                       int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
+    const int tiles_m = (M + SM - 1) / SM, tiles_n = (N + SN - 1) / SN;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n;
+    if (tiles >= (1 << 30)) return fail(ERR_UNSUPPORTED, "too many tiles");
+    const int cus = device_cu_count();
+    if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
+    auto kern = mxfp_gemm_scaled_kernel<DT_OUT>;
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), S_LDS_BYTES, lds_allowed)) return rc;
+    const unsigned grid = (unsigned)(tiles < cus ? ((tiles + 7) / 8) * 8 : (cus / 8) * 8);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), S_LDS_BYTES, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N, K,
+                       tiles_m * SM, tiles_n * SN, tiles_m, tiles_n);
+    return check_launch("mxfp_gemm_scaled");
+}

@@ -1,0 +1,22 @@
+// C-ABI entry point of the block-scaled MXFP GEMM; the kernel is in gemm_scaled.h.
+#include "gemm_impl.h"
+
+using namespace mase;
+
+extern "C" int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales,
+                                         const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                         void* stream) {
+    if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
+    if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K >= ((int64_t)1 << 27)) return fail(ERR_INVALID, "M, N must fit in 31 bits and K in 27");
+    if (K % 256 != 0 || K < 512) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM needs K to be a multiple of 256, at least 512");
+    if (!a_codes || !a_scales || !w_codes || !w_scales || !y) return fail(ERR_INVALID, "null pointer");
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (bias) if (int rc = check_dtype(bias_dtype, "bias")) return rc;
+    if (!aligned(a_codes, 16) || !aligned(w_codes, 16) || !aligned(a_scales, 4) || !aligned(w_scales, 4) || !aligned(y, 16))
+        return fail(ERR_INVALID, "codes and y must be 16-byte aligned, scales 4-byte aligned");
+    if (N % (16 / dtype_size(out_dtype)) != 0) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM stores 16 bytes at a time: N must be a multiple of 8 (4 for fp32 output)");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dispatch_dtype(out_dtype, [&](auto dout) {
+        return launch_gemm_scaled<decltype(dout)::value>(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, (int)M, (int)N, (int)K, s);
+    });
+}

@@ -222,3 +222,84 @@ def mxfp_gemm_batched(a: Tensor, w_scales: Tensor, w_elements: Tensor, w_meta: M
                 w_meta.element_exp_bits, w_meta.element_frac_bits, y[first].data_ptr(), _lib.dtype_code(output_dtype),
                 M, N, K, 32, count, a_batch_stride, w_batch_stride, M * N, _lib.stream_ptr(dev)))
     return y
+
+
+# ---- the block-scaled matrix instruction route (FP8 bytes and E8M0 scales straight into the matrix unit)
+_SCALED_FORMATS = {(4, 3), (2, 3), (3, 2), (2, 1)}
+
+
+class ScaledOperand:
+    """An [rows, K] MXFP matrix in the form the block-scaled GEMM reads: ``codes`` uint8 [rows_pad, K] (E4M3 bytes) and
+    ``scales`` int32 [K // 128, rows_pad]; rows past ``rows`` are padding with undefined contents."""
+
+    __slots__ = ("codes", "scales", "rows", "K")
+
+    def __init__(self, codes: Tensor, scales: Tensor, rows: int, K: int):
+        self.codes, self.scales, self.rows, self.K = codes, scales, rows, K
+
+
+def scaled_format_supported(meta: MXFPMeta) -> bool:
+    return (meta.block_size == 32 and meta.element_is_finite and meta.scale_exp_bits == 8
+            and (meta.element_exp_bits, meta.element_frac_bits) in _SCALED_FORMATS)
+
+
+def scaled_shape_supported(N: int, K: int, output_dtype: torch.dtype) -> bool:
+    return K % 256 == 0 and K >= 512 and N % (4 if output_dtype == torch.float32 else 8) == 0
+
+
+def _scaled_buffers(rows: int, K: int, dev) -> tuple[Tensor, Tensor]:
+    rows_pad = (rows + 255) // 256 * 256
+    return (torch.empty((rows_pad, K), dtype=torch.uint8, device=dev),
+            torch.empty((K // 128, rows_pad), dtype=torch.int32, device=dev))
+
+
+def scaled_operand_from_dense(x: Tensor, meta: MXFPMeta) -> ScaledOperand:
+    """Quantise the bfloat16 matrix x [rows, K] (blocks along K) straight into a block-scaled GEMM operand."""
+    assert x.ndim == 2 and x.dtype == torch.bfloat16 and scaled_format_supported(meta) and meta.round_mode == "rn"
+    _lib.require_gpu(x, "activations")
+    x = _lib.dense(x)
+    rows, K = x.shape
+    codes, scales = _scaled_buffers(rows, K, x.device)
+    with _lib.on_device(x.device):
+        _lib.check(_lib.load().mase_hip_scaled_operand_from_dense(
+            x.data_ptr(), _lib.dtype_code(x.dtype), meta.element_exp_bits, meta.element_frac_bits, rows, K,
+            codes.data_ptr(), scales.data_ptr(), _lib.stream_ptr(x.device)))
+    return ScaledOperand(codes, scales, rows, K)
+
+
+def scaled_operand_from_mxfp(scales: Tensor, elements: Tensor, meta: MXFPMeta, rows: int, K: int) -> ScaledOperand:
+    """MXFP components of a row-major [rows, K] matrix, blocked along K -> block-scaled GEMM operand."""
+    assert scaled_format_supported(meta)
+    assert scales.dtype == torch.uint8 and elements.dtype == torch.uint8
+    _lib.require_gpu(elements, "elements")
+    scales, elements = _lib.dense(scales), _lib.dense(elements)
+    assert elements.numel() == rows * K and scales.numel() == rows * K // 32
+    codes, out_scales = _scaled_buffers(rows, K, elements.device)
+    with _lib.on_device(elements.device):
+        _lib.check(_lib.load().mase_hip_scaled_operand_from_mxfp(
+            scales.data_ptr(), elements.data_ptr(), meta.element_exp_bits, meta.element_frac_bits, rows, K,
+            codes.data_ptr(), out_scales.data_ptr(), _lib.stream_ptr(elements.device)))
+    return ScaledOperand(codes, out_scales, rows, K)
+
+
+def mxfp_gemm_scaled(a: ScaledOperand, w: ScaledOperand, bias: Tensor | None, output_dtype: torch.dtype,
+                     out: Tensor | None = None) -> Tensor:
+    """y[M,N] = A @ W^T (+ bias) on the block-scaled matrix instruction, fp32 accumulation."""
+    assert a.K == w.K
+    M, N, K = a.rows, w.rows, a.K
+    dev = w.codes.device
+    b_ptr, b_dt = None, 0
+    if bias is not None:
+        bias = _lib.dense(bias)
+        assert bias.numel() == N
+        b_ptr, b_dt = bias.data_ptr(), _lib.dtype_code(bias.dtype)
+    if out is None:
+        y = torch.empty((M, N), dtype=output_dtype, device=dev)
+    else:
+        assert out.is_contiguous() and out.dtype == output_dtype and out.numel() == M * N and out.device == dev
+        y = out
+    with _lib.on_device(dev):
+        _lib.check(_lib.load().mase_hip_mxfp_gemm_scaled(
+            a.codes.data_ptr(), a.scales.data_ptr(), w.codes.data_ptr(), w.scales.data_ptr(), b_ptr, b_dt, y.data_ptr(),
+            _lib.dtype_code(output_dtype), M, N, K, _lib.stream_ptr(dev)))
+    return y

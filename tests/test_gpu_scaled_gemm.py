@@ -1,0 +1,265 @@
+"""GPU parity tests for the block-scaled route of the MXFP GEMM: operands kept as FP8 bytes and E8M0 scales up to the
+matrix unit (mase_hip_scaled_operand_from_dense / _from_mxfp, mase_hip_mxfp_gemm_scaled).
+
+What is checked, against the CPU checker's components of the same inputs:
+  * the prepared operand holds the reference's values: bit for bit in the formats that are embedded into E4M3 bytes,
+    and for E4M3 itself in every block that does not hold the code S.1111.111; blocks that do are stored one scale
+    step up with halved codes, by a rule restated here on integers, and no element moves by more than 2^-14 of its
+    block's largest;
+  * the product against float64 dequantise-then-matmul of the checker's values: relative Frobenius error <= 1e-3 for
+    16-bit outputs (compared with the reference rounded to that type) and 1e-4 for fp32 outputs (measured 1 - 2e-5:
+    the matrix unit adds a block's 32 products with fewer bits than a chain of fp32 FMAs keeps);
+  * identity times W returns W's dequantised values exactly;
+  * inf / NaN blocks poison exactly the rows (columns) they poison in dequantise-then-matmul.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import PRESETS
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F32_TOL = 1e-4
+SCALED_TAGS = ["MXFP8_E4M3_fn", "OCP_MXFP6_E3M2", "OCP_MXFP6_E2M3", "OCP_MXFP4_E2M1"]
+
+
+def rel_fro(y, y_ref):
+    y, y_ref = y.double().cpu(), y_ref.double().cpu()
+    return ((y - y_ref).norm() / y_ref.norm()).item()
+
+
+@pytest.fixture(scope="module")
+def mh():
+    import mase_hip.mxfp.functional as F
+    import mase_hip.mxfp.kernels as mxk
+    from mase_hip import _lib
+    from mase_hip.mxfp import meta
+    from mase_hip.mxfp.layers import MXFPLinearPTQ
+
+    _lib.load()
+
+    class NS:
+        pass
+
+    ns = NS()
+    ns.F, ns.mxk, ns.meta, ns.MXFPLinearPTQ = F, mxk, meta, MXFPLinearPTQ
+    return ns
+
+
+# ---------------------------------------------------------------- the prepared operand, decoded on the CPU
+def decode_e4m3(codes: np.ndarray) -> np.ndarray:
+    """OCP E4M3 bytes (no NaN code expected) -> float64."""
+    c = codes.astype(np.int64)
+    s, e, m = c >> 7, (c >> 3) & 15, c & 7
+    v = np.where(e == 0, m / 8.0 * 2.0 ** -6, (1 + m / 8.0) * 2.0 ** (e - 7.0))
+    return np.where(s == 1, -v, v)
+
+
+def decode_fmt(codes: np.ndarray, E: int, M: int) -> np.ndarray:
+    """Codes of the reference's finite (E, M) format -> float64 (minifloat/fake.py:97-123)."""
+    c = codes.astype(np.int64)
+    bias = (1 << (E - 1)) - 1
+    s, e, m = (c >> (E + M)) & 1, (c >> M) & ((1 << E) - 1), c & ((1 << M) - 1)
+    v = np.where(e == 0, m / float(1 << M) * 2.0 ** (1 - bias), (1 + m / float(1 << M)) * 2.0 ** (e.astype(np.float64) - bias))
+    return np.where(s == 1, -v, v)
+
+
+def operand_arrays(op):
+    """(codes [rows, K] uint8, scales [rows, K/32] uint8) of a ScaledOperand, padding rows dropped."""
+    codes = op.codes[: op.rows].cpu().numpy()
+    sc = op.scales.cpu().numpy().view(np.uint32)                      # [K/128, rows_pad]
+    by = np.stack([(sc >> (8 * b)) & 0xFF for b in range(4)], axis=-1)  # [K/128, rows_pad, 4]
+    scales = by.transpose(1, 0, 2).reshape(sc.shape[1], -1)[: op.rows].astype(np.uint8)
+    return codes, scales
+
+
+def halved(codes: np.ndarray) -> np.ndarray:
+    """The documented re-encoding of an E4M3 block one scale step up."""
+    c = codes.astype(np.int64)
+    sign, mag = c & 0x80, c & 0x7F
+    small = mag // 2 + ((mag & 1) & ((mag // 2) & 1))   # below 16 the magnitude is linear in the value: halve, ties to even
+    return (sign | np.where(mag >= 16, mag - 8, small)).astype(np.uint8)
+
+
+def mixed_inputs(rows, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, K, generator=g)
+    x[rows // 3] *= torch.exp2(torch.randint(-20, 20, (K,), generator=g).float())   # wide range inside blocks
+    x[rows // 2, : K // 2] = 0.0                                                     # all-zero blocks
+    x[rows // 2 + 1] *= 2.0 ** -130                                                  # flushed inputs
+    x = x.to(torch.bfloat16)
+    x[1, 5] = float("inf")
+    x[2, 40] = float("-inf")
+    x[3, 70] = float("nan")
+    return x
+
+
+def expected_operand(x: torch.Tensor, E: int, M: int):
+    """What the prepared operand must hold, from the checker's components."""
+    rows, K = x.shape
+    sc, el = oracle.extract_mxfp(x, 32, E, M)
+    sc = sc.numpy().reshape(rows, K // 32).astype(np.int64)
+    el = el.numpy().reshape(rows, K // 32, 32)
+    if (E, M) == (4, 3):
+        top = ((el & 0x7F) == 0x7F).any(axis=2) & (sc < 254)
+        codes = np.where(top[..., None], halved(el), el)
+        scales = sc + top
+    else:
+        codes, scales = None, sc
+    return sc, el, codes, scales
+
+
+@pytest.mark.parametrize("tag", SCALED_TAGS)
+def test_operand_from_dense_holds_the_reference_values(mh, tag):
+    E, M = PRESETS[tag]
+    rows, K = 300, 1024
+    x = mixed_inputs(rows, K, seed=E * 10 + M)
+    op = mh.mxk.scaled_operand_from_dense(x.to(DEV), getattr(mh.meta, tag))
+    assert op.codes.shape == (512, K) and op.scales.shape == (K // 128, 512)
+    codes, scales = operand_arrays(op)
+    codes = codes.reshape(rows, K // 32, 32)
+    ref_sc, ref_el, want_codes, want_scales = expected_operand(x, E, M)
+    assert np.array_equal(scales, want_scales), "scale bytes"
+    finite = ref_sc != 255
+    got = decode_e4m3(codes) * 2.0 ** (scales[..., None].astype(np.float64) - 127)
+    ref = decode_fmt(ref_el, E, M) * 2.0 ** (ref_sc[..., None].astype(np.float64) - 127)
+    if (E, M) == (4, 3):
+        assert np.array_equal(codes[finite], want_codes[finite]), "codes"
+        assert not ((codes[finite] & 0x7F) == 0x7F).any(), "the NaN code must not appear"
+        moved = np.abs(got - ref)[finite]
+        assert (moved <= 2.0 ** -14 * np.abs(ref).max(axis=2, keepdims=True)[finite]).all()
+        untouched = finite & (want_scales == ref_sc)
+        assert np.array_equal(got[untouched], ref[untouched])
+        assert (want_scales != ref_sc).sum() > 100, "the test data must hold blocks with the top code"
+    else:
+        assert np.array_equal(got[finite], ref[finite]), "embedded values"
+
+
+@pytest.mark.parametrize("tag", SCALED_TAGS)
+def test_operand_from_components_equals_from_dense(mh, tag):
+    E, M = PRESETS[tag]
+    rows, K = 260, 768
+    x = mixed_inputs(rows, K, seed=3)
+    sc, el = oracle.extract_mxfp(x, 32, E, M)
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), getattr(mh.meta, tag))
+    b = mh.mxk.scaled_operand_from_mxfp(sc.to(DEV), el.to(DEV), getattr(mh.meta, tag), rows, K)
+    ca, sa = operand_arrays(a)
+    cb, sb = operand_arrays(b)
+    assert np.array_equal(sa, sb)
+    assert np.array_equal(ca, cb)
+
+
+# ---------------------------------------------------------------- the product
+def quantised(t: torch.Tensor, tag: str):
+    E, M = PRESETS[tag]
+    sc, el = oracle.extract_mxfp(t, 32, E, M)
+    dq = oracle.compose_mxfp(sc, el, 32, E, M, True, torch.float32).view(t.shape)
+    return sc, el, dq
+
+
+@pytest.mark.parametrize("MNK", [(256, 256, 512), (300, 520, 768), (1024, 768, 1024), (1, 8, 512), (513, 264, 2048)])
+@pytest.mark.parametrize("x_tag,w_tag", [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP6_E3M2"),
+                                         ("OCP_MXFP6_E2M3", "OCP_MXFP4_E2M1"), ("OCP_MXFP4_E2M1", "OCP_MXFP6_E2M3")])
+def test_scaled_gemm_vs_checker(mh, MNK, x_tag, w_tag):
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    _, _, x_dq = quantised(x, x_tag)
+    w_sc, w_el, w_dq = quantised(w, w_tag)
+    y_ref = oracle.matmul_nt(x_dq, w_dq)
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), getattr(mh.meta, x_tag))
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), getattr(mh.meta, w_tag), N, K)
+    y32 = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.float32)
+    assert y32.shape == (M, N)
+    assert rel_fro(y32, y_ref) <= F32_TOL
+    y16 = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.bfloat16)
+    assert rel_fro(y16, y_ref.to(torch.bfloat16)) <= 1e-3
+
+
+def test_scaled_gemm_bias_and_dtypes(mh):
+    M, N, K = 300, 264, 512
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    _, _, x_dq = quantised(x, "MXFP8_E4M3_fn")
+    w_sc, w_el, w_dq = quantised(w, "MXFP8_E4M3_fn")
+    meta = mh.meta.MXFP8_E4M3_fn
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), meta)
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), meta, N, K)
+    for bdt in (torch.float32, torch.bfloat16, torch.float16):
+        b = torch.randn(N, generator=torch.Generator().manual_seed(1)).to(bdt)
+        y_ref = oracle.matmul_nt(x_dq, w_dq) + b.float()
+        for odt, tol in ((torch.float32, F32_TOL), (torch.bfloat16, 1e-3), (torch.float16, 1e-3)):
+            y = mh.mxk.mxfp_gemm_scaled(a, wop, b.to(DEV), odt)
+            assert y.dtype == odt
+            assert rel_fro(y, y_ref.to(odt)) <= tol
+
+
+@pytest.mark.parametrize("w_tag", SCALED_TAGS)
+def test_identity_times_w_is_w(mh, w_tag):
+    """x = identity: every output is one product, so the result must be W's dequantised values (rounded to bf16 the way
+    the reference's compose rounds them); for E4M3 that includes the blocks that were re-encoded, except where a block
+    holds both the top code and an odd code below 16.  Compared as values: a sign-only code composes to -0.0, and a
+    product -0.0 added to the row's other products (+0.0) is +0.0 in any matmul."""
+    E, M = PRESETS[w_tag]
+    K = N = 512
+    g = torch.Generator().manual_seed(9)
+    w = (torch.randn(N, K, generator=g) * torch.exp2(torch.randint(-12, 12, (N, 1), generator=g).float())).to(torch.bfloat16)
+    w_sc, w_el = oracle.extract_mxfp(w, 32, E, M)
+    want = oracle.compose_mxfp(w_sc, w_el, 32, E, M, True, torch.bfloat16).view(N, K)
+    x = torch.eye(K, dtype=torch.bfloat16)
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), mh.meta.MXFP8_E4M3_fn)
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), getattr(mh.meta, w_tag), N, K)
+    y = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.bfloat16).cpu()   # y[k, n] = W[n, k]
+    got = y.t().contiguous()
+    if (E, M) == (4, 3):
+        el = w_el.numpy().reshape(N, K // 32, 32)
+        top = ((el & 0x7F) == 0x7F).any(axis=2)
+        odd_small = (((el & 0x7F) < 16) & ((el & 1) == 1)).any(axis=2)
+        inexact = torch.from_numpy(np.repeat(top & odd_small, 32, axis=1))
+        assert top.sum() > 50
+        assert torch.equal(got[~inexact].float(), want[~inexact].float())
+        assert rel_fro(got, want) <= 1e-5
+    else:
+        assert torch.equal(got.float(), want.float())
+
+
+def test_special_blocks_poison_the_same_outputs(mh):
+    """inf / NaN in x or W: scale byte 255.  Dequantise-then-matmul turns the affected rows / columns into NaN (a zero
+    code times 2^128 is NaN); so must the matrix unit."""
+    M, N, K = 256, 256, 512
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    x[7, 100] = float("inf")
+    x[200, 3] = float("nan")
+    w[5, 40] = float("-inf")
+    w[255, 511] = float("nan")
+    _, _, x_dq = quantised(x, "MXFP8_E4M3_fn")
+    w_sc, w_el, w_dq = quantised(w, "MXFP8_E4M3_fn")
+    y_ref = x_dq.double() @ w_dq.double().t()
+    meta = mh.meta.MXFP8_E4M3_fn
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), meta)
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), meta, N, K)
+    y = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.float32).cpu()
+    assert torch.equal(y.isnan(), y_ref.isnan())
+    assert y.isnan().sum() == 2 * N + 2 * M - 4
+    ok = ~y_ref.isnan()
+    assert rel_fro(y[ok], y_ref[ok]) <= F32_TOL
+
+
+def test_unsupported_shapes_are_refused(mh):
+    meta = mh.meta.MXFP8_E4M3_fn
+    x = torch.randn(64, 384).to(torch.bfloat16).to(DEV)
+    a = mh.mxk.scaled_operand_from_dense(x, meta)   # K % 128 == 0: an operand can be built
+    with pytest.raises(NotImplementedError):
+        mh.mxk.mxfp_gemm_scaled(a, a, None, torch.bfloat16)   # K % 256 != 0
+    with pytest.raises(NotImplementedError):
+        mh.mxk.scaled_operand_from_dense(torch.randn(8, 96).to(torch.bfloat16).to(DEV), meta)
+    x5 = torch.randn(8, 512).to(torch.bfloat16).to(DEV)
+    with pytest.raises((NotImplementedError, AssertionError)):
+        mh.mxk.scaled_operand_from_dense(x5, mh.meta.MXFP8_E5M2_fn)
