@@ -3,12 +3,14 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--skip-hbm]
 
-One step = one mxfp_linear call on the headline shape: x [16384, 4096] bf16 ~N(0,1), W [14336, 4096]
-bf16 ~N(0,0.02) held as MXFP8 E4M3 components (block 32 along K), activations quantised to MXFP8
-E4M3 on the fly, bf16 output, fp32 accumulation: the fused QDQ kernel over x followed by the
-dequant-fused MFMA GEMM.  Inputs are resident in HBM before the timed region.  The same run also
-measures the bandwidth-bound cast kernels on their own configurations (extra "hbm_kernels" list)
-and times the reference's CPU path (tensor-op restatement under oracle/) on a bounded sample.
+One step = one mxfp_linear(..., layer_type="XqWqB", backend="fused") call on the headline shape: x [16384, 4096] bf16
+~N(0,1), W [14336, 4096] bf16 ~N(0,0.02) held as MXFP8 E4M3 components (block 32 along K), activations quantised to
+MXFP8 E4M3 on the fly, bf16 output, fp32 accumulation.  At this shape "fused" is three kernels: x quantised straight
+into FP8 bytes + E8M0 scales, the weight components brought into the same form (inside the call: a functional call
+has nowhere to keep it; a layer builds it once), and the GEMM on the block-scaled FP8 matrix instruction.  Inputs are
+resident in HBM before the timed region.  The same run also times the bf16-MFMA kernel family on the same shape, the
+SwiGLU block of configuration C5, the bandwidth-bound cast kernels on their own configurations ("hbm_kernels") and the
+reference's CPU path (tensor-op restatement under oracle/) on bounded samples.
 
 Prints ONE JSON line.
 """
@@ -27,6 +29,7 @@ for p in (ROOT, os.path.join(ROOT, "mase-triton_amd"), os.path.join(ROOT, "tests
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8, published
 # HBM-side bytes per launch (roofline.traffic) are not measured by this run: they come from the committed summary of two
 # rocprofv3 --pmc runs of `bench.py --counter-probe` (FETCH_SIZE, then WRITE_SIZE), written by
 # `bench.py --summarize-counters`.  Every entry carries a fingerprint of the kernel sources it was taken with; when the
@@ -34,6 +37,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_counters_gemm_c4_casts_c1_c2_c3.md")
 CSRC = os.path.join(ROOT, "mase-triton_amd", "csrc")
 GEMM_SOURCES = ("gemm_tall.h", "gemm_impl.h", "mxfp_compose.h", "mase_device.h")
+SCALED_SOURCES = ("gemm_scaled.h", "gemm_tall.h", "mase_device.h")
 CAST_SOURCES = ("cast_kernels.hip", "mxfp_compose.h", "mase_device.h")
 
 
@@ -78,8 +82,14 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--skip-hbm", action="store_true", help="skip the cast-kernel bandwidth section")
-    ap.add_argument("--only-gemm-kernel", action="store_true",
-                    help="profiling aid: launch only the GEMM kernel in the timed loop")
+    ap.add_argument("--only-gemm-kernel", choices=("scaled", "bf16"), default=None,
+                    help="profiling aid: launch only that GEMM kernel (block-scaled FP8 or bf16 MFMA) on the headline shape, "
+                         "--steps times after --warmup, and print nothing")
+    ap.add_argument("--summarize-sq", metavar="COUNTER_CSV",
+                    help="no GPU needed: per-kernel table (stdout, markdown) from the counter_collection.csv of a rocprofv3 --pmc run with "
+                         "SQ_BUSY_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_LDS SQ_WAIT_ANY SQ_WAVE_CYCLES SQ_WAVES [SQ_LDS_BANK_CONFLICT]")
+    ap.add_argument("--summarize-trace", metavar="KERNEL_TRACE_CSV",
+                    help="no GPU needed: per-kernel durations (stdout, markdown) from the kernel_trace.csv of a rocprofv3 --kernel-trace run")
     ap.add_argument("--counter-probe", action="store_true",
                     help="profiling aid for rocprofv3 --pmc: a plain 256 MiB device copy (calibration), then 3 launches "
                          "each of the GEMM and of the C3 extract / compose kernels; prints nothing to time")
@@ -117,19 +127,48 @@ def settle(torch, fn, group=5, tol=0.01, most=100):
     return {"steps": done, "first_group_ms_per_step": round(first, 4), "settled_ms_per_step": round(ms, 4)}
 
 
+def timed_loop(torch, fn, steps, warmup):
+    """ms per call: `steps` calls between two device synchronisations, after `warmup` uncounted ones."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
 def bench_linear(args, torch, MXFP_F, kernels, fmt):
+    import workloads
+    from mase_hip.mxfp.functional import linear as L
+
     dev = "cuda:0"
-    M, K, N = 16384, 4096, 14336
-    gen = torch.Generator(device=dev).manual_seed(3)
-    x = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
-    w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
+    x_cpu, w_cpu = workloads.make_c4()          # the very tensors of the parity test (CPU generator, seeds 3 and 4)
+    M, K = x_cpu.shape
+    N = w_cpu.shape[0]
+    x, w = x_cpu.to(dev), w_cpu.to(dev)
+    del x_cpu, w_cpu
     w_sc, w_el, w_tm = MXFP_F.extract_mxfp_components(w, block_dim=1, mxfp_meta=fmt)
     del w
     call = dict(x=x, x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
-                b_elements=None, b_tensor_meta=None, layer_type="XqWqB", backend="fused")
+                b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
+    flop = 2.0 * M * N * K
 
     def step(ev=None):
-        # same two kernels as MXFP_F.mxfp_linear(**call), split so that events can bracket the GEMM
+        # the three kernels of MXFP_F.mxfp_linear(**call, backend="fused") at this shape, split so that events can
+        # bracket the GEMM
+        a_op = kernels.scaled_operand_from_dense(x, fmt)
+        w_op = L.scaled_weight_operand(w_sc, w_el, w_tm)
+        if ev is not None:
+            ev[0].record()
+        y = kernels.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
+        if ev is not None:
+            ev[1].record()
+        return y
+
+    def step_bf16(ev=None):
+        # backend="fused_bf16": single-pass QDQ of x to bf16, then the GEMM that composes W to bf16 in registers
         a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
         if ev is not None:
             ev[0].record()
@@ -138,77 +177,55 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
             ev[1].record()
         return y
 
-    y_api = MXFP_F.mxfp_linear(**call)
-    assert torch.equal(step().view(torch.int16), y_api.view(torch.int16)), "bench step differs from mxfp_linear"
+    if args.only_gemm_kernel:
+        a_op, w_op = kernels.scaled_operand_from_dense(x, fmt), L.scaled_weight_operand(w_sc, w_el, w_tm)
+        a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
+        fn = ((lambda: kernels.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)) if args.only_gemm_kernel == "scaled" else
+              (lambda: kernels.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt, None, M, N, K, torch.bfloat16)))
+        timed_loop(torch, fn, args.steps, args.warmup)
+        return None
+
+    y_api = MXFP_F.mxfp_linear(**call, backend="fused")
+    assert torch.equal(step().view(torch.int16), y_api.view(torch.int16)), "bench step differs from mxfp_linear(backend='fused')"
+    assert torch.equal(step_bf16().view(torch.int16), MXFP_F.mxfp_linear(**call, backend="fused_bf16").view(torch.int16))
     del y_api
     # The shader clock settles over the first few dozen launches after idle (the step gets faster), so a short counted
     # warm-up would time the ramp.  Before the counted warm-up: steps in groups of five until two consecutive groups agree
     # within 1 %, at most 100 steps.  Both figures are reported.
     prewarm = settle(torch, step)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    if args.only_gemm_kernel:
-        a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
+
+    def measure(step_fn):
+        for _ in range(args.warmup):
+            step_fn()
         torch.cuda.synchronize()
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
         t0 = time.perf_counter()
         for i in range(args.steps):
-            pairs[i][0].record()
-            kernels.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt, None, M, N, K, torch.bfloat16)
-            pairs[i][1].record()
+            step_fn(pairs[i])
         torch.cuda.synchronize()
-        t1 = time.perf_counter()
-    else:
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step(pairs[i])
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    gemm_ms = sum(event_ms(pairs)) / args.steps
-    flop = 2.0 * M * N * K
-    # context, not the metric: the same step with backend="separate" (fused QDQ of x, compose W to bf16 in HBM, then
-    # the vendor library's dense bf16 GEMM through F.linear), and that dense GEMM alone on the dequantised operands
-    sep = dict(call, backend="separate")
-    for _ in range(max(3, args.warmup // 2)):
-        MXFP_F.mxfp_linear(**sep)
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    for _ in range(args.steps):
-        MXFP_F.mxfp_linear(**sep)
-    torch.cuda.synchronize()
-    sep_ms = (time.perf_counter() - t2) * 1e3 / args.steps
-    # backend="auto": at this many rows the single-pass QDQ of x, one compose of W into HBM and the library GEMM
-    auto = dict(call, backend="auto")
-    for _ in range(max(3, args.warmup // 2)):
-        MXFP_F.mxfp_linear(**auto)
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    for _ in range(args.steps):
-        MXFP_F.mxfp_linear(**auto)
-    torch.cuda.synchronize()
-    auto_ms = (time.perf_counter() - t2) * 1e3 / args.steps
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        return ms, sum(event_ms(pairs)) / args.steps
+
+    ms_per_step, gemm_ms = measure(step)
+    settle(torch, step_bf16)
+    bf16_ms, bf16_gemm_ms = measure(step_bf16)
+    # context, not the metric
+    half = max(3, args.warmup // 2)
+    w_op = L.scaled_weight_operand(w_sc, w_el, w_tm)      # what a layer keeps
+    prepared_ms = timed_loop(torch, lambda: MXFP_F.mxfp_linear(**call, backend="fused", w_operand=w_op), args.steps, half)
+    del w_op
+    # backend="separate": extract x, compose x, compose W to bf16 in HBM, the vendor library's dense bf16 GEMM
+    sep_ms = timed_loop(torch, lambda: MXFP_F.mxfp_linear(**call, backend="separate"), args.steps, half)
     a_dq = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
     w_dq = kernels.compose_mxfp_tensor(w_sc, w_el, fmt, torch.bfloat16).view(N, K)
-    for _ in range(5):
-        torch.nn.functional.linear(a_dq, w_dq)
-    torch.cuda.synchronize()
-    t3 = time.perf_counter()
-    for _ in range(args.steps):
-        torch.nn.functional.linear(a_dq, w_dq)
-    torch.cuda.synchronize()
-    dense_ms = (time.perf_counter() - t3) * 1e3 / args.steps
+    dense_ms = timed_loop(torch, lambda: torch.nn.functional.linear(a_dq, w_dq), args.steps, 5)
     del a_dq, w_dq
+    tf = lambda ms: flop / (ms * 1e-3) / 1e12
     return {
-        "prewarm": prewarm,
-        "separate_ms": sep_ms, "dense_ms": dense_ms, "auto_ms": auto_ms,
-        "ms_per_step": ms_per_step,
-        "tflops_step": flop / (ms_per_step * 1e-3) / 1e12,
-        "gemm_ms": gemm_ms,
-        "tflops_gemm": flop / (gemm_ms * 1e-3) / 1e12,
-        "shape": (M, N, K),
+        "prewarm": prewarm, "shape": (M, N, K), "flop": flop,
+        "ms_per_step": ms_per_step, "tflops_step": tf(ms_per_step), "gemm_ms": gemm_ms, "tflops_gemm": tf(gemm_ms),
+        "bf16_ms_per_step": bf16_ms, "bf16_tflops_step": tf(bf16_ms), "bf16_gemm_ms": bf16_gemm_ms, "bf16_tflops_gemm": tf(bf16_gemm_ms),
+        "prepared_ms": prepared_ms, "separate_ms": sep_ms, "dense_ms": dense_ms,
     }
 
 
@@ -276,18 +293,18 @@ def cpu_cast_baselines(torch):
         x = full(rows, 4096).reshape(-1)
         n = x.numel()
         sc, el = torch_fake.mxfp_split(x, 32, e, m)
-        sample = f"{rows} rows x 4096 of {tag}'s distribution"
+        sample = f"{rows} rows of {tag}"
         t_ext = timed(lambda: torch_fake.mxfp_split(x, 32, e, m))
         t_cmp = timed(lambda: torch_fake.mxfp_join(sc, el, e, m, True, torch.bfloat16))
         out[("extract_mxfp", tag)] = entry(n * (3 + 1 / 32), t_ext, sample)
         out[("compose_mxfp", tag)] = entry(n * (3 + 1 / 32), t_cmp, sample)
         out[("extract+compose_mxfp", tag)] = entry(n * (6 + 1 / 16), t_ext + t_cmp, sample)
-        out[("qdq_mxfp_fused", tag)] = entry(n * 4.0, t_ext + t_cmp, sample + " (the reference has no fused pass: extract then compose)")
+        out[("qdq_mxfp_fused", tag)] = entry(n * 4.0, t_ext + t_cmp, sample + " (extract then compose)")
     x = workloads.make_c2(1 << 22)
     n = x.numel()
     for e, m in ((4, 3), (5, 2)):
         codes = torch_fake.minifloat_encode(x, e, m)
-        sample = "2^22 of C2's 2^24 elements"
+        sample = "2^22 of C2"
         t_ext = timed(lambda: torch_fake.minifloat_encode(x, e, m))
         t_cmp = timed(lambda: torch_fake.minifloat_decode(codes, e, m, True, torch.float32))
         tag = f"C2/E{e}M{m}"
@@ -372,7 +389,7 @@ def bench_hbm(torch, with_cpu):
         def qdq(i):
             _lib.check(lib.mase_hip_qdq_mxfp(xs[i].data_ptr(), 2, y_o[i].data_ptr(), 2, n, 32, e, m, 1, 0, sp_of()))
 
-        wl = f"{tag}: {rows}x{cols} bf16, E{e}M{m}, block 32, the configuration's value distribution"
+        wl = f"{tag}: {rows}x{cols} bf16, E{e}M{m}, block 32"
         for name, fn, nbytes in (("extract_mxfp", ext, ext_bytes), ("compose_mxfp", cmp, cmp_bytes),
                                  ("extract+compose_mxfp", both, ext_bytes + cmp_bytes), ("qdq_mxfp_fused", qdq, n * 4.0)):
             avg, best = time_kernel(torch, fn, copies)
@@ -399,7 +416,7 @@ def bench_hbm(torch, with_cpu):
         def cmp(i):
             _lib.check(lib.mase_hip_compose_minifloat(cs[i].data_ptr(), ys[i].data_ptr(), 0, n, e, m, 1, sp_of()))
 
-        wl = f"C2: 2^24 fp32 with outliers, zeros and subnormals, FP8 E{e}M{m}"
+        wl = f"C2: 2^24 fp32, FP8 E{e}M{m}"
         for i in range(len(xs)):
             ext(i)                # codes for the compose rows
         for name, fn, nbytes in (("qdq_minifloat_fused", qdq, n * 8.0), ("extract_minifloat", ext, n * 6.0),
@@ -459,21 +476,28 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
         return (time.perf_counter() - t0) * 1e6 / steps
 
     def linear_rows(n_out, k_in, Ms):
+        from mase_hip.mxfp.functional import linear as L
+
         wt = (0.02 * torch.randn(n_out, k_in, generator=gen, device=dev)).to(torch.bfloat16)
         sc, el, tm = MXFP_F.extract_mxfp_components(wt, block_dim=1, mxfp_meta=fmt)
+        w_op = L.scaled_weight_operand(sc, el, tm)
         out = []
         for M in Ms:
             x = torch.randn(M, k_in, generator=gen, device=dev).to(torch.bfloat16)
             call = dict(x=x, x_meta=fmt, w=None, w_scales=sc, w_elements=el, w_tensor_meta=tm, b=None, b_scales=None,
                         b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
+            b_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="fused_bf16"))
+            s_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="fused_scaled"))
+            p_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="fused_scaled", w_operand=w_op))
             f_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="fused"))
-            s_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="separate"))
-            out.append({"M": M, "fused_us": round(f_us, 1), "separate_us": round(s_us, 1),
+            sep_us = timed(lambda: MXFP_F.mxfp_linear(**call, backend="separate"))
+            out.append({"M": M, "fused_us": round(f_us, 1), "fused_bf16_us": round(b_us, 1), "fused_scaled_us": round(s_us, 1),
+                        "fused_scaled_kept_weight_us": round(p_us, 1), "separate_us": round(sep_us, 1),
                         "fused_TFLOPs": round(2.0 * M * n_out * k_in / f_us / 1e6, 1)})
         return out
 
-    rows = linear_rows(N, K, (16, 64, 128, 256, 384, 512, 1024, 2048, 4096))
-    rows_down = linear_rows(K, N, (16, 64, 256, 1024, 4096))  # the transposed layer shape: few W rows, long K
+    rows = linear_rows(N, K, (16, 64, 128, 256, 384, 512, 768, 1024, 2048, 4096, 8192))
+    rows_down = linear_rows(K, N, (16, 64, 256, 512, 1024, 2048, 4096))  # the transposed layer shape: few W rows, long K
     w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
     n = w.numel()
     cast = {
@@ -492,6 +516,7 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
     """Three launches of each kernel next to a copy of known size, for hardware-counter runs (see --summarize-counters)."""
     import workloads
     from mase_hip import _lib
+    from mase_hip.mxfp.functional import linear as L
 
     dev = "cuda:0"
     lib = _lib.load()
@@ -502,45 +527,64 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
     for _ in range(3):                                      # calibration: reads 256 MiB, writes 256 MiB
         assert blib.mase_bench_stream_copy(src.data_ptr(), dst.data_ptr(), src.numel(), 1, sp) == 0
     del src, dst
-    M, K, N = 16384, 4096, 14336
-    gen = torch.Generator(device=dev).manual_seed(3)
-    x = torch.randn(M, K, generator=gen, device=dev).to(torch.bfloat16)
-    w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
-    w_sc, w_el, _ = MXFP_F.extract_mxfp_components(w, block_dim=1, mxfp_meta=fmt8)
+    x_cpu, w_cpu = workloads.make_c4()
+    M, K = x_cpu.shape
+    N = w_cpu.shape[0]
+    x, w = x_cpu.to(dev), w_cpu.to(dev)
+    w_sc, w_el, w_tm = MXFP_F.extract_mxfp_components(w, block_dim=1, mxfp_meta=fmt8)
     a = mxk.quantize_dequantize(x.view(-1), fmt8, torch.bfloat16).view(M, K)
     for _ in range(3):
         mxk.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt8, None, M, N, K, torch.bfloat16)
-    del x, w, w_sc, w_el, a
+    for _ in range(3):
+        a_op = mxk.scaled_operand_from_dense(x, fmt8)
+        w_op = L.scaled_weight_operand(w_sc, w_el, w_tm)
+        mxk.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
+    del x, w, w_sc, w_el, a, a_op, w_op
     for make, fmt in ((workloads.make_c1, fmt8), (workloads.make_c3, fmt4)):
         t = make().reshape(-1).to(dev)
         for _ in range(3):
             sc, el = mxk.extract_mxfp_components(t, fmt)
             mxk.compose_mxfp_tensor(sc, el, fmt, torch.bfloat16)
+            mxk.quantize_dequantize(t, fmt, torch.bfloat16)
         del t
     x2 = workloads.make_c2().to(dev)
     y2 = torch.empty_like(x2)
     c2 = torch.empty(x2.numel(), dtype=torch.uint16, device=dev)
-    for _ in range(3):
-        _lib.check(lib.mase_hip_qdq_minifloat(x2.data_ptr(), 0, y2.data_ptr(), 0, x2.numel(), 4, 3, 1, 0, sp))
-        _lib.check(lib.mase_hip_extract_minifloat(x2.data_ptr(), 0, c2.data_ptr(), x2.numel(), 4, 3, 1, 0, sp))
-        _lib.check(lib.mase_hip_compose_minifloat(c2.data_ptr(), y2.data_ptr(), 0, x2.numel(), 4, 3, 1, sp))
+    for e, m in ((4, 3), (5, 2)):
+        for _ in range(3):
+            _lib.check(lib.mase_hip_qdq_minifloat(x2.data_ptr(), 0, y2.data_ptr(), 0, x2.numel(), e, m, 1, 0, sp))
+            _lib.check(lib.mase_hip_extract_minifloat(x2.data_ptr(), 0, c2.data_ptr(), x2.numel(), e, m, 1, 0, sp))
+            _lib.check(lib.mase_hip_compose_minifloat(c2.data_ptr(), y2.data_ptr(), 0, x2.numel(), e, m, 1, sp))
     torch.cuda.synchronize()
 
 
-# kernel-name fragments of the counter probe's launches ('a|b': both must occur; extract is MODE 0 of a kernel whose MODE 1 is
-# the fused QDQ) -> (key in the summary, algorithmic bytes read, written, sources)
+# kernel-name fragments of the counter probe's launches ('a|b': all must occur; the last template argument of
+# mxfp_bf16_b32_kernel is its mode: 0 extract, 1 fused QDQ, 2 block-scaled operand) -> (key in the summary, algorithmic bytes
+# read, written, sources).  A key is "<kernel row of hbm_kernels> <config>" for the cast rows.
 _N1, _N3, _N2 = 4096 * 4096, 14336 * 4096, 1 << 24
+_M4, _N4, _K4 = 16384, 14336, 4096
 COUNTER_ROWS = (
     ("stream_copy_kernel", "calibration copy (256 MiB read, 256 MiB written)", 256 << 20, 256 << 20, None),
-    ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", 16384 * 4096 * 2 + 14336 * 4096 + 14336 * 128, 16384 * 14336 * 2, GEMM_SOURCES),
+    ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C4", (_M4 + _N4) * _K4 * 33 // 32, _M4 * _N4 * 2, SCALED_SOURCES),
+    ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", _M4 * _K4 * 2 + _N4 * _K4 * 33 // 32, _M4 * _N4 * 2, GEMM_SOURCES),
+    ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 2>(", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
+    ("scaled_operand_kernel", "scaled_operand_from_mxfp C4 W", _N4 * _K4 * 33 // 32, _N4 * _K4 * 33 // 32, CAST_SOURCES),
     ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 0>(", "extract_mxfp C1", _N1 * 2, _N1 + _N1 // 32, CAST_SOURCES),
     ("compose_mxfp_bf16_kernel<mase::SFmt<4, 3", "compose_mxfp C1", _N1 + _N1 // 32, _N1 * 2, CAST_SOURCES),
+    ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 1>(", "qdq_mxfp_fused C1", _N1 * 2, _N1 * 2, CAST_SOURCES),
     ("mxfp_bf16_b32_kernel<mase::SFmt<2, 1|, 0>(", "extract_mxfp C3", _N3 * 2, _N3 + _N3 // 32, CAST_SOURCES),
     ("compose_mxfp_bf16_kernel<mase::SFmt<2, 1", "compose_mxfp C3", _N3 + _N3 // 32, _N3 * 2, CAST_SOURCES),
-    ("minifloat_f32_kernel<2", "qdq_minifloat_fused C2/E4M3", _N2 * 4, _N2 * 4, CAST_SOURCES),
-    ("minifloat_f32_kernel<0", "extract_minifloat C2/E4M3", _N2 * 4, _N2 * 2, CAST_SOURCES),
-    ("minifloat_f32_kernel<1", "compose_minifloat C2/E4M3", _N2 * 2, _N2 * 4, CAST_SOURCES),
+    ("mxfp_bf16_b32_kernel<mase::SFmt<2, 1|, 1>(", "qdq_mxfp_fused C3", _N3 * 2, _N3 * 2, CAST_SOURCES),
+    ("minifloat_f32_kernel<2, mase::SFmt<4, 3", "qdq_minifloat_fused C2/E4M3", _N2 * 4, _N2 * 4, CAST_SOURCES),
+    ("minifloat_f32_kernel<0, mase::SFmt<4, 3", "extract_minifloat C2/E4M3", _N2 * 4, _N2 * 2, CAST_SOURCES),
+    ("minifloat_f32_kernel<1, mase::SFmt<4, 3", "compose_minifloat C2/E4M3", _N2 * 2, _N2 * 4, CAST_SOURCES),
+    ("minifloat_f32_kernel<2, mase::SFmt<5, 2", "qdq_minifloat_fused C2/E5M2", _N2 * 4, _N2 * 4, CAST_SOURCES),
+    ("minifloat_f32_kernel<0, mase::SFmt<5, 2", "extract_minifloat C2/E5M2", _N2 * 4, _N2 * 2, CAST_SOURCES),
+    ("minifloat_f32_kernel<1, mase::SFmt<5, 2", "compose_minifloat C2/E5M2", _N2 * 2, _N2 * 4, CAST_SOURCES),
 )
+# launches of one kernel name at several sizes (the probe also quantises the headline's x and W): the size that is meant, in threads
+_COUNTER_THREADS = {"extract_mxfp C1": _N1 // 16, "extract_mxfp C3": _N3 // 16, "qdq_mxfp_fused C1": _N1 // 16, "qdq_mxfp_fused C3": _N3 // 16,
+                    "scaled_operand_from_dense C4 x": _M4 * _K4 // 16}
 
 
 def summarize_counters(fetch_dir, write_dir):
@@ -572,7 +616,7 @@ def summarize_counters(fetch_dir, write_dir):
 
     rows = []
     for frag, key, rd, wr, sources in COUNTER_ROWS:
-        threads = {"extract_mxfp C1": _N1 // 16, "extract_mxfp C3": _N3 // 16}.get(key)   # one lane per 2 x 8 elements
+        threads = _COUNTER_THREADS.get(key)   # one lane per 2 x 8 elements
         (name, f_kib), (_, w_kib) = pick(fetch, frag, threads), pick(write, frag, threads)
         rows.append((key, name, f_kib, w_kib, rd, wr, sources))
     cal = rows[0]
@@ -598,49 +642,160 @@ def summarize_counters(fetch_dir, write_dir):
     print("```")
 
 
-def bench_c5(torch, steps=20, warmup=8):
-    """Context, not the metric: a Llama-3-8B SwiGLU MLP block of MXFPLinearPTQ layers, down(silu(gate(x)) * up(x)),
-    weights gate / up [14336, 4096] and down [4096, 14336] ~N(0, 0.02) stored as MXFP6 E3M2, MXFP8 E4M3 activations,
-    block 32, x [4 x 2048, 4096] bf16 ~N(0, 1): three quantise kernels, three GEMMs and the activation per step."""
+def bench_c5(torch, with_cpu, steps=20, warmup=8):
+    """Configuration C5: a Llama-3-8B SwiGLU MLP block of MXFPLinearPTQ layers, down(silu(gate(x)) * up(x)), weights
+    gate / up [14336, 4096] and down [4096, 14336] ~N(0, 0.02) stored as MXFP6 E3M2, MXFP8 E4M3 activations, block 32,
+    x [4 x 2048, 4096] bf16 ~N(0, 1) (tests/workloads.py: make_c5).  Gate and up are stacked into one [28672, 4096] layer
+    (MXFP blocks run along in_features, so stacking rows changes no value): x is quantised once and one GEMM serves both.
+    Per block: two quantise kernels, two GEMMs, SiLU and the product in torch."""
+    import workloads
+    from mase_hip.mxfp import kernels
     from mase_hip.mxfp.layers import MXFPLinearPTQ
     from mase_hip.mxfp.meta import MXFP8_E4M3_fn, MXFPMeta
 
     dev = "cuda:0"
-    gen = torch.Generator(device=dev).manual_seed(11)
-    x = torch.randn(4, 2048, 4096, generator=gen, device=dev).to(torch.bfloat16)
+    x_cpu, wg, wu, wd = workloads.make_c5()
+    x = x_cpu.to(dev)
     wfmt = MXFPMeta(32, 8, 3, 2, True, "rn")
-    out = {}
-    for backend in ("fused", "separate"):
+    inter = wg.shape[0]
+    flop = 3 * 2.0 * x.shape[0] * x.shape[1] * wg.shape[0] * wg.shape[1]
+    ms = {}
+    for backend in ("fused", "fused_bf16", "separate"):
         ls = []
-        for n_out, n_in in ((14336, 4096), (14336, 4096), (4096, 14336)):
-            lin = torch.nn.Linear(n_in, n_out, bias=False, dtype=torch.bfloat16, device=dev)
-            lin.weight.data.copy_((0.02 * torch.randn(n_out, n_in, generator=gen, device=dev)).to(torch.bfloat16))
+        for w in (torch.cat([wg, wu]), wd):
+            lin = torch.nn.Linear(w.shape[1], w.shape[0], bias=False, dtype=torch.bfloat16, device=dev)
+            lin.weight.data.copy_(w)
             ls.append(MXFPLinearPTQ.from_linear(lin, MXFP8_E4M3_fn, wfmt, None, "XqWqB", backend))
             del lin
-        g, u, d = ls
+        gu, d = ls
 
         def mlp():
-            return d(torch.nn.functional.silu(g(x)) * u(x))
+            t = gu(x)
+            return d(torch.nn.functional.silu(t[..., :inter]) * t[..., inter:])
 
-        for _ in range(warmup):
-            mlp()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            mlp()
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) * 1e3 / steps
-        out[f"{backend}_ms"] = round(ms, 4)
-        out[f"{backend}_TFLOPs"] = round(3 * 2.0 * 8192 * 4096 * 14336 / (ms * 1e-3) / 1e12, 1)
-        del ls, g, u, d
-    out["note"] = "whole block per step (x quantised three times, SiLU and the product in torch); flop = the three GEMMs"
+        ms[backend] = timed_loop(torch, mlp, steps, warmup)
+        if backend == "fused":
+            # the two GEMM kernels of the block on their own, bracketed by events on the launch stream
+            rows = x.shape[0] * x.shape[1]
+            a1 = kernels.scaled_operand_from_dense(x.view(rows, -1), MXFP8_E4M3_fn)
+            h = torch.nn.functional.silu(gu(x)[..., :inter]) * gu(x)[..., inter:]
+            a2 = kernels.scaled_operand_from_dense(h.view(rows, -1), MXFP8_E4M3_fn)
+            w1, w2 = gu._weight_operand(x), d._weight_operand(h)
+            assert w1 is not None and w2 is not None, "the C5 layers did not take the block-scaled route"
+            gemm_ms = []
+            for a_op, w_op in ((a1, w1), (a2, w2)):
+                for _ in range(5):
+                    kernels.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
+                pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+                for e0, e1 in pairs:
+                    e0.record()
+                    kernels.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
+                    e1.record()
+                torch.cuda.synchronize()
+                gemm_ms.append(sum(event_ms(pairs)) / steps)
+            del a1, a2, h, w1, w2
+        del ls, gu, d
+    tf = lambda t: flop / (t * 1e-3) / 1e12
+    kern_tf = tf(sum(gemm_ms))
+    out = {
+        "workload": "C5 SwiGLU block: x[4x2048,4096] bf16, gate+up stacked [28672,4096], down [4096,14336], W MXFP6 E3M2, X MXFP8 E4M3",
+        "ms_per_block": {k: round(v, 4) for k, v in ms.items()},
+        "TFLOPs": {k: round(tf(v), 1) for k, v in ms.items()},
+        "roofline": {"bound": "mfma", "achieved": round(kern_tf, 1), "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(kern_tf / MFMA_FP8_PEAK_TFLOPS, 4), "frac_of_bf16_peak": round(kern_tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "kernel": "mxfp_gemm_scaled_kernel", "avg_kernel_ms": {"gate_up": round(gemm_ms[0], 4), "down": round(gemm_ms[1], 4)},
+                     "traffic": None},
+        "note": "flop = the three GEMMs; ms_per_block = whole block (quantise kernels, GEMMs, SiLU and product)",
+    }
+    if with_cpu:
+        from oracle import torch_fake
+
+        comps = [torch_fake.mxfp_split(w, 32, 3, 2) for w in (wg, wu, wd)]
+        x2 = x_cpu.view(-1, x_cpu.shape[-1])
+
+        def chain(rows):
+            t0 = time.perf_counter()
+            xs = x2[:rows]
+            g = torch_fake.mxfp_linear_xq_wq(xs, *comps[0], tuple(wg.shape), torch.bfloat16, (4, 3), (3, 2))
+            u = torch_fake.mxfp_linear_xq_wq(xs, *comps[1], tuple(wu.shape), torch.bfloat16, (4, 3), (3, 2))
+            y = torch_fake.mxfp_linear_xq_wq(torch.nn.functional.silu(g) * u, *comps[2], tuple(wd.shape), torch.bfloat16, (4, 3), (3, 2))
+            assert y.shape == (rows, wd.shape[0])
+            return time.perf_counter() - t0
+
+        t_probe = chain(256)
+        rows = int(min(x2.shape[0], max(256, 256 * (10.0 / max(t_probe, 1e-3)))) // 256 * 256)
+        dt = chain(rows)
+        out["cpu_baseline"] = {"value": round(flop * rows / x2.shape[0] / dt / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"{rows} of {x2.shape[0]} rows through the three layers, {dt:.1f} s"}
     return out
+
+
+def summarize_sq(counter_csv):
+    """Markdown table (stdout) of the library's kernels in a rocprofv3 --pmc run: cycles per launch, MFMA pipe busy,
+    VALU / LDS instructions per wavefront, share of wavefront time in waits."""
+    import collections
+    import csv
+    import re
+
+    csv.field_size_limit(1 << 30)
+    d = collections.OrderedDict()
+    for r in csv.DictReader(open(counter_csv)):
+        m = re.search(r"mase::(\w+)", r["Kernel_Name"])
+        if not m:
+            continue
+        key = (m.group(1), int(r["Grid_Size"]) // max(1, int(r["Workgroup_Size"])), int(r["Workgroup_Size"]))
+        d.setdefault(key, collections.defaultdict(list))[r["Counter_Name"]].append(float(r["Counter_Value"]))
+    print("| kernel | workgroups x threads | launches | cycles per launch | MFMA pipe busy | VALU / wavefront | LDS / wavefront | LDS bank conflict | wavefront time in waits |")
+    print("|---|---|---|---|---|---|---|---|---|")
+    for k, c in d.items():
+        mean = {n: sum(v) / len(v) for n, v in c.items()}
+        if "SQ_BUSY_CYCLES" not in mean or "SQ_WAVES" not in mean:
+            continue
+        cyc = mean["SQ_BUSY_CYCLES"] / 32            # summed over 32 shader engines
+        waves = mean["SQ_WAVES"]
+        busy = f"{mean['SQ_VALU_MFMA_BUSY_CYCLES'] / 1024 / cyc * 100:.1f} %" if "SQ_VALU_MFMA_BUSY_CYCLES" in mean else "-"   # 1024 SIMDs
+        valu = f"{mean['SQ_INSTS_VALU'] / waves:.0f}" if "SQ_INSTS_VALU" in mean else "-"
+        lds = f"{mean['SQ_INSTS_LDS'] / waves:.0f}" if "SQ_INSTS_LDS" in mean else "-"
+        conf = f"{mean['SQ_LDS_BANK_CONFLICT'] / 256 / cyc * 100:.1f} % of cycles" if "SQ_LDS_BANK_CONFLICT" in mean else "-"   # 256 CUs
+        wait = f"{mean['SQ_WAIT_ANY'] / mean['SQ_WAVE_CYCLES'] * 100:.1f} %" if "SQ_WAIT_ANY" in mean and "SQ_WAVE_CYCLES" in mean else "-"
+        print(f"| `{k[0]}` | {k[1]} x {k[2]} | {len(next(iter(c.values())))} | {cyc:.4g} | {busy} | {valu} | {lds} | {conf} | {wait} |")
+
+
+def summarize_trace(trace_csv):
+    """Markdown table (stdout) of per-kernel durations in a rocprofv3 --kernel-trace run."""
+    import collections
+    import csv
+    import re
+
+    csv.field_size_limit(1 << 30)
+    d = collections.OrderedDict()
+    meta = {}
+    for r in csv.DictReader(open(trace_csv)):
+        n = re.sub(r"^void ", "", r["Kernel_Name"])
+        n = re.sub(r"\(.*$", "", n)
+        if "mase::" not in n and "Cijk" not in n:
+            continue
+        key = (n[:120], int(r["Grid_Size_X"]) // max(1, int(r["Workgroup_Size_X"])), int(r["Workgroup_Size_X"]))
+        d.setdefault(key, []).append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1000.0)
+        meta[key] = (r.get("LDS_Block_Size", "-"), r.get("VGPR_Count", "-"), r.get("Accum_VGPR_Count", "-"), r.get("Scratch_Size", "-"))
+    print("| kernel | workgroups x threads | launches | mean us | median us | min us | LDS | VGPR | AGPR | scratch |")
+    print("|---|---|---|---|---|---|---|---|---|---|")
+    for k, v in d.items():
+        v = sorted(v)
+        m = meta[k]
+        print(f"| `{k[0]}` | {k[1]} x {k[2]} | {len(v)} | {sum(v) / len(v):.2f} | {v[len(v) // 2]:.2f} | {v[0]:.2f} | {m[0]} | {m[1]} | {m[2]} | {m[3]} |")
 
 
 def main():
     args = parse_args()
     if args.summarize_counters:
         summarize_counters(*args.summarize_counters)
+        return
+    if args.summarize_sq:
+        summarize_sq(args.summarize_sq)
+        return
+    if args.summarize_trace:
+        summarize_trace(args.summarize_trace)
         return
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this pool has a single MI355X and the path has no "
@@ -651,10 +806,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the product has no CPU path)", file=sys.stderr)
         sys.exit(2)
-    import mase_hip.minifloat.kernels as mfk
     import mase_hip.mxfp.functional as MXFP_F
     import mase_hip.mxfp.kernels as mxk
-    from mase_hip.minifloat.meta import MinifloatMeta
     from mase_hip.mxfp.meta import MXFP8_E4M3_fn, MXFPMeta
 
     torch.cuda.set_device(0)
@@ -665,7 +818,12 @@ def main():
         print(json.dumps({"shape_sweep": shape_sweep(torch, MXFP_F, mxk, MXFP8_E4M3_fn)}))
         return
     lin = bench_linear(args, torch, MXFP_F, mxk, MXFP8_E4M3_fn)
+    if lin is None:
+        return
     M, N, K = lin["shape"]
+    tf = lambda ms: round(lin["flop"] / (ms * 1e-3) / 1e12, 2)
+    # key order: the driver's record keeps the standard keys and the tail of the line, so the long per-kernel list goes in
+    # the middle and the comparisons last
     result = {
         "metric": "mxfp_linear TFLOP/s at 16384x4096x14336 (MXFP8 E4M3 x MXFP8 E4M3, block 32)",
         "value": round(lin["tflops_step"], 2),
@@ -677,36 +835,36 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "fp8 (E4M3 codes x E8M0 block scales in the matrix unit, fp32 accumulate; MXFP values are exact in it)",
         "data": "synthetic",
-        "config": {"workload": "C4 mxfp_linear: x[16384,4096] bf16 ~N(0,1) quantised on the fly to MXFP8 E4M3, "
-                               "W[14336,4096] ~N(0,0.02) stored as MXFP8 E4M3, block 32 along K, no bias, bf16 out, "
-                               "fp32 accumulate; step = fused QDQ kernel + dequant-fused GEMM kernel",
-                   "M": M, "N": N, "K": K},
-        "roofline": {"bound": "mfma", "achieved": round(lin["tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": traffic_bytes("mxfp_gemm_tall_kernel C4", GEMM_SOURCES),
-                     "kernel": "mxfp_gemm_tall_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4)},
-        "prewarm": dict(lin["prewarm"], note="uncounted steps before the counted warm-up, in groups of five until two groups agree "
-                                             "within 1 % (the shader clock settles over the first launches after idle)"),
-        "context": {
-            "separate_backend_ms_per_step": round(lin["separate_ms"], 4),
-            "separate_backend_TFLOPs": round(2.0 * M * N * K / (lin["separate_ms"] * 1e-3) / 1e12, 2),
-            "auto_backend_ms_per_step": round(lin["auto_ms"], 4),
-            "auto_backend_TFLOPs": round(2.0 * M * N * K / (lin["auto_ms"] * 1e-3) / 1e12, 2),
-            "vendor_dense_bf16_gemm_ms": round(lin["dense_ms"], 4),
-            "vendor_dense_bf16_gemm_TFLOPs": round(2.0 * M * N * K / (lin["dense_ms"] * 1e-3) / 1e12, 2),
-            "note": "same shape on the same GPU: backend='separate' = extract x + compose x + compose W to bf16 in HBM + library GEMM "
-                    "(weights held dequantised during the call); backend='auto' (an extension, not the metric) = single-pass QDQ of x + "
-                    "one compose of W + library GEMM from 3072 rows of x on, the fused kernel below; dense = the library's bf16 GEMM alone",
-        },
+        "config": {"workload": "C4 mxfp_linear XqWqB fused: x[16384,4096] bf16 -> MXFP8 E4M3, W[14336,4096] MXFP8 E4M3, bf16 out",
+                   "M": M, "N": N, "K": K, "inputs": "tests/workloads.py make_c4 (seeds 3, 4)",
+                   "step": "quantise x to FP8 operand + weight components to FP8 operand + block-scaled GEMM"},
+        "roofline": {"bound": "mfma", "achieved": round(lin["tflops_gemm"], 2), "peak": MFMA_FP8_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(lin["tflops_gemm"] / MFMA_FP8_PEAK_TFLOPS, 4),
+                     "traffic": traffic_bytes("mxfp_gemm_scaled_kernel C4", SCALED_SOURCES),
+                     "kernel": "mxfp_gemm_scaled_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4),
+                     "frac_of_bf16_peak": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "bf16_kernel": {"kernel": "mxfp_gemm_tall_kernel", "achieved": round(lin["bf16_tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
+                                     "frac": round(lin["bf16_tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "avg_kernel_ms": round(lin["bf16_gemm_ms"], 4),
+                                     "traffic": traffic_bytes("mxfp_gemm_tall_kernel C4", GEMM_SOURCES)}},
     }
+    result["cpu_baseline"] = None if args.no_cpu else cpu_baseline(torch)
     if not args.skip_hbm:
-        result["context"]["c5_swiglu_mlp_block"] = bench_c5(torch)
         result["hbm_kernels"] = bench_hbm(torch, with_cpu=not args.no_cpu)
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(torch)
-    else:
-        result["cpu_baseline"] = None
+        result["c5"] = bench_c5(torch, with_cpu=not args.no_cpu)
+    result["prewarm"] = lin["prewarm"]
+    result["context"] = {
+        "same_shape_ms_per_step": {
+            "fused (value)": round(lin["ms_per_step"], 4), "fused, weight operand kept by a layer": round(lin["prepared_ms"], 4),
+            "fused_bf16": round(lin["bf16_ms_per_step"], 4), "separate": round(lin["separate_ms"], 4),
+            "vendor dense bf16 GEMM alone": round(lin["dense_ms"], 4)},
+        "same_shape_TFLOPs": {
+            "fused (value)": tf(lin["ms_per_step"]), "fused, weight operand kept by a layer": tf(lin["prepared_ms"]),
+            "fused_bf16": tf(lin["bf16_ms_per_step"]), "separate": tf(lin["separate_ms"]), "vendor dense bf16 GEMM alone": tf(lin["dense_ms"])},
+        "note": "fused_bf16 = QDQ of x to bf16 + GEMM composing W to bf16 in registers (bf16 MFMA); separate = extract x + compose x + "
+                "compose W to bf16 in HBM + library GEMM; prewarm = uncounted steps until two groups of five agree within 1 %",
+    }
     print(json.dumps(result))
 
 

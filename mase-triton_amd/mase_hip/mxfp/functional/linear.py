@@ -6,16 +6,20 @@ B or Bq (bias).
 
 backend="separate" follows the reference literally: dequantise every operand to a dense tensor,
 then ``torch.nn.functional.linear``.
-backend="fused" (NotImplementedError in the reference, :31-32) never builds the dense weight:
-activations go through the single-pass QDQ kernel and the GEMM composes the MXFP weight tiles
-to bf16 in registers on their way to the MFMA units (fp32 accumulation).  Every MXFP value has
-at most four significant bits, so bf16 operands are exact and the result differs from
-"separate" only by the summation order.
-backend="auto" (not in the reference) is "fused" up to ``AUTO_DENSE_FROM_ROWS`` rows of x and, from there on, the
-single-pass QDQ of x, ONE compose of W to bf16 in HBM and the library's dense GEMM: the fused kernel composes every W
-element once per 512 rows of x, and on this power-limited chip that in-loop work costs more than writing W out once when
-there are thousands of rows (measured cross-over between 2048 and 4096 rows for N x K = 14336 x 4096 and 4096 x 14336).
-It needs N * K * 2 bytes of temporary memory per call.
+backend="fused" (NotImplementedError in the reference, :31-32) never builds the dense weight.  It has two kernel
+families and picks between them by format and shape:
+
+* the block-scaled route (``fused_scaled`` forces it): x is quantised straight into FP8 bytes and E8M0 scales, the
+  weight components are turned into the same form (once per layer when a layer calls, see ``w_operand``), and the GEMM
+  feeds both to the block-scaled matrix instruction, which applies the scales itself.  Taken for quantised x and W in
+  the element formats E4M3 / E3M2 / E2M3 / E2M1, bfloat16 x, K a multiple of 256, from ``SCALED_FROM_ROWS`` rows of x;
+* the bf16 route (``fused_bf16`` forces it): activations go through the single-pass QDQ kernel and the GEMM composes
+  the MXFP weight tiles to bf16 in registers on their way to the bf16 matrix instruction.  Every MXFP value has at most
+  four significant bits, so bf16 operands are exact.
+
+Both accumulate in fp32 and differ from "separate" only by the summation order (and, on the block-scaled route, by
+the re-encoding of E4M3 blocks that hold the code the matrix unit reads as NaN: at most 2^-14 of a block's largest
+element, see include/mase_hip.h).
 """
 from __future__ import annotations
 
@@ -30,7 +34,11 @@ from .cast import compose_mxfp_tensor, extract_mxfp_components, quantize_dequant
 
 _LAYER_TYPES = ("XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq")
 _GEMM_DTYPES = (torch.bfloat16, torch.float32)
-AUTO_DENSE_FROM_ROWS = 3072
+_BACKENDS = ("separate", "fused", "fused_bf16", "fused_scaled")
+# rows of x from which "fused" takes the block-scaled route: with fewer the weight-streaming bf16 kernels win (the
+# block-scaled kernel works on 256 x 256 tiles and the weight has to be brought into its form first)
+SCALED_FROM_ROWS = 256
+SCALED_FROM_ROWS_UNPREPARED = 1024   # ... when the weight operand has to be built inside the call
 
 
 def parse_mxfp_linear_type(x_meta: MXFPMeta | None, w_tensor_meta: MXFPTensorMeta | None,
@@ -64,6 +72,27 @@ def _gemm_eligible(x: Tensor, quantised_x: bool, w_tensor_meta: MXFPTensorMeta, 
     return b is None or b.dtype in (torch.bfloat16, torch.float16, torch.float32)
 
 
+def _scaled_eligible(x: Tensor, x_meta: MXFPMeta | None, w_tensor_meta: MXFPTensorMeta, b: Tensor | None) -> bool:
+    """Can the block-scaled matrix instruction take this product?"""
+    if x_meta is None or x.device.type != "cuda" or x.dtype != torch.bfloat16 or len(w_tensor_meta.shape) != 2:
+        return False
+    if not (kernels.scaled_format_supported(x_meta) and kernels.scaled_format_supported(w_tensor_meta.meta)):
+        return False
+    if x_meta.round_mode != "rn" or w_tensor_meta.block_dim % 2 != 1 or getattr(torch, w_tensor_meta.dtype) != x.dtype:
+        return False
+    out_features, in_features = w_tensor_meta.shape
+    if not kernels.scaled_shape_supported(out_features, in_features, x.dtype) or x.numel() == 0:
+        return False
+    return b is None or b.dtype in (torch.bfloat16, torch.float16, torch.float32)
+
+
+def scaled_weight_operand(w_scales: Tensor, w_elements: Tensor, w_tensor_meta: MXFPTensorMeta) -> "kernels.ScaledOperand":
+    """The weight components in the block-scaled GEMM's form (a copy: N * K bytes of codes and N * K / 32 of scales).
+    A layer builds it once and passes it to ``mxfp_linear(..., w_operand=...)``."""
+    out_features, in_features = w_tensor_meta.shape
+    return kernels.scaled_operand_from_mxfp(w_scales, w_elements, w_tensor_meta.meta, out_features, in_features)
+
+
 def mxfp_linear(
     x: Tensor,
     x_meta: MXFPMeta | None,
@@ -76,11 +105,15 @@ def mxfp_linear(
     b_elements: Tensor | None,
     b_tensor_meta: MXFPTensorMeta | None,
     layer_type: Literal["XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq"],
-    backend: Literal["separate", "fused", "auto"],
+    backend: Literal["separate", "fused", "fused_bf16", "fused_scaled"],
+    *,
+    w_operand: "kernels.ScaledOperand | None" = None,
 ) -> Tensor:
+    """``w_operand`` (not in the reference): the weight already in the block-scaled GEMM's form, from
+    ``scaled_weight_operand``; without it the fused block-scaled route builds it inside the call."""
     if layer_type not in _LAYER_TYPES:
         raise NotImplementedError(f"Layer type {layer_type} not implemented")
-    if backend not in ("separate", "fused", "auto"):
+    if backend not in _BACKENDS:
         raise NotImplementedError(f"backend {backend!r} not implemented")
     quantised_x = layer_type.startswith("Xq")
     quantised_w = "Wq" in layer_type
@@ -94,10 +127,22 @@ def mxfp_linear(
             w = compose_mxfp_tensor(w_scales, w_elements, w_tensor_meta)
         return torch.nn.functional.linear(x, w, bias)
 
-    # ---- fused (auto: only while the rows of x are few enough for the in-loop compose to pay)
+    # ---- fused
     rows = x.numel() // x.shape[-1] if x.numel() else 0
-    through_kernel = backend == "fused" or rows < AUTO_DENSE_FROM_ROWS
-    if through_kernel and quantised_w and _gemm_eligible(x, quantised_x, w_tensor_meta, bias):
+    if quantised_x and quantised_w and backend != "fused_bf16" and _scaled_eligible(x, x_meta, w_tensor_meta, bias):
+        if backend == "fused_scaled" or rows >= (SCALED_FROM_ROWS if w_operand is not None else SCALED_FROM_ROWS_UNPREPARED):
+            out_features, in_features = w_tensor_meta.shape
+            assert x.shape[-1] == in_features
+            a_op = kernels.scaled_operand_from_dense(x.reshape(-1, in_features), x_meta)
+            if w_operand is None:
+                w_operand = scaled_weight_operand(w_scales, w_elements, w_tensor_meta)
+            assert w_operand.rows == out_features and w_operand.K == in_features
+            y = kernels.mxfp_gemm_scaled(a_op, w_operand, bias, x.dtype)
+            return y.view(*x.shape[:-1], out_features)
+    elif backend == "fused_scaled":
+        raise NotImplementedError("backend 'fused_scaled' needs quantised bfloat16 x and W in E4M3 / E3M2 / E2M3 / E2M1 with in_features a "
+                                  "multiple of 256 and out_features a multiple of 8")
+    if quantised_w and _gemm_eligible(x, quantised_x, w_tensor_meta, bias):
         out_features, in_features = w_tensor_meta.shape
         assert x.shape[-1] == in_features
         lead = x.shape[:-1]

@@ -21,7 +21,9 @@ class MXFPLinearPTQ(nn.Module):
     ``w_elements`` [N*K/B, B], blocked along in_features; likewise ``b_scales``/``b_elements``.
     Their dtype may never change (``.to(dtype=...)`` raises ``ChangeDtypeError``); moving the
     module between devices refreshes the device recorded in the tensor metas.  Unlike the
-    reference, ``backend="fused"`` (the default) works: it runs the dequant-fused MFMA GEMM.
+    reference, ``backend="fused"`` (the default) works: it runs the fused MFMA GEMMs.  Where the block-scaled route
+    applies, the layer keeps the weight a second time in that kernel's form (``N * K * 33 / 32`` bytes, built on the
+    first such forward and rebuilt when the components change or move; not part of ``state_dict``).
     """
 
     in_features: int
@@ -36,7 +38,7 @@ class MXFPLinearPTQ(nn.Module):
         w_mxfp_meta: MXFPMeta | None,
         b_mxfp_meta: MXFPMeta | None,
         layer_type: LayerType,
-        backend: Literal["separate", "fused", "auto"] = "fused",
+        backend: Literal["separate", "fused", "fused_bf16", "fused_scaled"] = "fused",
         dtype: torch.dtype | None = None,
         device: torch.device | None = None,
         w_scales: Tensor | None = None,
@@ -66,6 +68,7 @@ class MXFPLinearPTQ(nn.Module):
         self.backend = backend
         self.dtype, self.device = dtype, device
 
+        self._scaled_w = self._scaled_w_key = None   # the weight in the block-scaled GEMM's form, and what it was built from
         self.weight = self.bias = None
         self.w_scales = self.w_elements = self.w_tensor_meta = None
         self.b_scales = self.b_elements = self.b_tensor_meta = None
@@ -105,12 +108,37 @@ class MXFPLinearPTQ(nn.Module):
             self.b_tensor_meta = self.b_tensor_meta.create(device=self.b_scales.device)
         return result
 
+    def invalidate_weight_operand(self) -> None:
+        """Drop the cached block-scaled form of the weight.  Writes to ``w_scales`` / ``w_elements`` that torch records
+        (``copy_`` under ``no_grad``, ``load_state_dict``, moving the module) are noticed without this call; writes
+        through ``.data`` are not."""
+        self._scaled_w = self._scaled_w_key = None
+
+    def _weight_operand(self, input: Tensor):
+        """The weight in the block-scaled GEMM's form when this call can take that route, else None."""
+        from .functional import linear as L
+
+        if self.backend not in ("fused", "fused_scaled") or not self.layer_type.startswith("XqWq"):
+            return None
+        rows = input.numel() // input.shape[-1] if input.numel() else 0
+        if self.backend == "fused" and rows < L.SCALED_FROM_ROWS:
+            return None
+        bias = self.bias if not self.layer_type.endswith("Bq") else None
+        if not L._scaled_eligible(input, self.x_mxfp_meta, self.w_tensor_meta, bias):
+            return None
+        key = (self.w_elements.data_ptr(), self.w_elements._version, self.w_scales.data_ptr(), self.w_scales._version)
+        if self._scaled_w is None or self._scaled_w_key != key:
+            self._scaled_w = L.scaled_weight_operand(self.w_scales, self.w_elements, self.w_tensor_meta)
+            self._scaled_w_key = key
+        return self._scaled_w
+
     @torch.no_grad()
     def forward(self, input: Tensor) -> Tensor:
         return MXFP_F.mxfp_linear(
             x=input, x_meta=self.x_mxfp_meta, w=self.weight, w_scales=self.w_scales, w_elements=self.w_elements,
             w_tensor_meta=self.w_tensor_meta, b=self.bias, b_scales=self.b_scales, b_elements=self.b_elements,
-            b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend)
+            b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend,
+            w_operand=self._weight_operand(input))
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
@@ -119,7 +147,7 @@ class MXFPLinearPTQ(nn.Module):
 
     @classmethod
     def from_linear(cls, layer: nn.Linear, x_mxfp_meta: MXFPMeta | None, w_mxfp_meta: MXFPMeta | None,
-                    b_mxfp_meta: MXFPMeta | None, layer_type: LayerType, backend: Literal["separate", "fused", "auto"]):
+                    b_mxfp_meta: MXFPMeta | None, layer_type: LayerType, backend: Literal["separate", "fused", "fused_bf16", "fused_scaled"]):
         """Quantise a trained ``nn.Linear``."""
         assert isinstance(layer, nn.Linear), "layer must be an instance of nn.Linear"
         with torch.no_grad():
@@ -144,7 +172,7 @@ class MXFPLinearPTQ(nn.Module):
         return d
 
     @classmethod
-    def from_exported(cls, d: dict, backend: Literal["separate", "fused", "auto"] = "fused", device=None):
+    def from_exported(cls, d: dict, backend: Literal["separate", "fused", "fused_bf16", "fused_scaled"] = "fused", device=None):
         """Inverse of :meth:`export_quantized`."""
         from . import packing
 
@@ -167,7 +195,7 @@ class MXFPLinearPTQ(nn.Module):
                        bias: Tensor | None, b_scales: Tensor | None, b_elements: Tensor | None,
                        b_tensor_meta: MXFPTensorMeta | None, x_mxfp_meta: MXFPMeta | None,
                        layer_type: Literal["XWqB", "XWqBq", "XqWqB", "XqWqBq"],
-                       backend: Literal["separate", "fused", "auto"]):
+                       backend: Literal["separate", "fused", "fused_bf16", "fused_scaled"]):
         """Re-hydrate from stored components (tensor metas are not part of ``state_dict``)."""
         assert w_scales is not None and w_elements is not None and w_tensor_meta is not None
         return cls(weight=None, bias=bias, x_mxfp_meta=x_mxfp_meta, w_mxfp_meta=None, b_mxfp_meta=None,

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(lib):
     from mase_hip import _lib
 
     names = declared_symbols()
-    assert len(names) == 17
+    assert len(names) == 21
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mase_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of step with the header"
@@ -58,6 +58,15 @@ def test_argument_errors_without_a_gpu(lib):
     assert b"aligned" in lib.mase_hip_last_error()
     assert lib.mase_hip_compose_minifloat(p, p, 3, 16, 4, 3, 1, None) == -1
     assert lib.mase_hip_qdq_minifloat(p, 0, p, 2, 16, 4, 3, 1, 0, None) == -1  # in place with different sizes
+    # the block-scaled route: shapes and formats it does not take are refused before any launch
+    assert lib.mase_hip_scaled_padded_rows(1) == 256 and lib.mase_hip_scaled_padded_rows(257) == 512
+    assert lib.mase_hip_scaled_operand_from_dense(p, 2, 4, 3, 8, 96, p, p, None) == -2     # K % 128
+    assert lib.mase_hip_scaled_operand_from_dense(p, 2, 5, 2, 8, 128, p, p, None) == -2    # E5M2
+    assert lib.mase_hip_scaled_operand_from_dense(p, 0, 4, 3, 8, 128, p, p, None) == -2    # fp32 input
+    assert lib.mase_hip_scaled_operand_from_mxfp(p, p + 4, 4, 3, 8, 128, p, p, None) == -1  # alignment
+    assert lib.mase_hip_mxfp_gemm_scaled(p, p, p, p, None, 0, p, 2, 8, 8, 384, None) == -2  # K % 256
+    assert lib.mase_hip_mxfp_gemm_scaled(p, p, p, p, None, 0, p, 2, 8, 12, 512, None) == -2  # N % 8
+    assert lib.mase_hip_mxfp_gemm_scaled(p, None, p, p, None, 0, p, 2, 8, 8, 512, None) == -1
     assert lib.mase_hip_mxfp_gemm(p, 2, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, 16, 16, 48, 32, None) == -1
     assert lib.mase_hip_mxfp_gemm(p, 2, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, 16, 16, 64, 16, None) == -2
     assert lib.mase_hip_mxfp_gemm(p, 0, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, 16, 16, 64, 32, None) == -2
