@@ -471,19 +471,49 @@ __device__ inline size_t scaled_scale_offset(uint32_t row0, uint32_t kb0, uint32
     return ((size_t)((uint32_t)r >> 2) * g.rows_pad + row0 + q) * 4 + ((uint32_t)r & 3u);
 }
 
-// MODE 0: extract (scales + elements); MODE 1: fused quantise-dequantise to bf16; MODE 2: extract as an operand of the
-// block-scaled GEMM (E4M3 bytes without the NaN code, scales transposed)
+// The arithmetic of one 128-bit step of the bf16 kernels below: 8 elements of a lane whose three quad neighbours hold the
+// rest of the block.  QDQ false: o[j] = two codes in the low bytes of the halves; true: two quantised bf16 values.
+// Every lane of a quad must call it (DPP).
+template <class F, bool QDQ>
+__device__ inline void bf16_block_step(const uint4& raw, const F& f, uint32_t (&o)[4], uint32_t& scale) {
+    const uint32_t h[4] = {raw.x, raw.y, raw.z, raw.w};
+    // block maximum of |x| bits: packed max over the lane's four registers, then the two halves,
+    // then the four lanes of the block (DPP quad permutes)
+    u16x2 m2 = __builtin_elementwise_max(__builtin_elementwise_max(as_u16x2(h[0] & 0x7FFF7FFFu), as_u16x2(h[1] & 0x7FFF7FFFu)),
+                                         __builtin_elementwise_max(as_u16x2(h[2] & 0x7FFF7FFFu), as_u16x2(h[3] & 0x7FFF7FFFu)));
+    uint32_t amax = max((uint32_t)m2[0], (uint32_t)m2[1]);
+    amax = max(amax, (uint32_t)__builtin_amdgcn_mov_dpp((int)amax, 0xB1, 0xF, 0xF, true));  // lane ^ 1
+    amax = max(amax, (uint32_t)__builtin_amdgcn_mov_dpp((int)amax, 0x4E, 0xF, 0xF, true));  // lane ^ 2
+    const int ef_max = (int)(amax >> 7);
+    const int scale_n = max(ef_max - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
+    // (scale_n < bias: the packed arithmetic subtracts (scale_n - bias) << 7 with unsigned saturation)
+    const bool hard = amax >= 0x7F80u || scale_n >= 151 || (amax != 0u && scale_n < fmt_bias(f) + (QDQ ? 1 : 0));
+    scale = (uint32_t)scale_n;
+    if (__builtin_amdgcn_ballot_w64(hard) == 0) {
+        const uint32_t ssb = (uint32_t)((scale_n - fmt_bias(f)) << 7) & 0xFFFFu;
+        const uint32_t ssb2 = ssb | (ssb << 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = QDQ ? PackedBf16<F>::qdq(h[j], ssb2) : PackedBf16<F>::codes(h[j], ssb2);
+    } else {
+        // exact per-element routine (the block's lanes agree on amax, so they agree on the result)
+        const uint32_t amax32 = amax << 16;
+        const int se = shared_exponent<F, true>(amax32, f);
+        scale = amax32 < 0x00800000u ? 0u : (uint32_t)(se + 127);
+        const float sc = scale_f32(scale);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t c0 = encode_mxfp_element(h[j] << 16, se, f), c1 = encode_mxfp_element(h[j] & 0xFFFF0000u, se, f);
+            o[j] = QDQ ? pack_bf16(mxfp_value(c0, sc, f), mxfp_value(c1, sc, f)) : (c0 | (c1 << 16));
+        }
+    }
+}
+
+// MODE 0: extract (scales + elements); MODE 1: fused quantise-dequantise to bf16
 template <class F, int UNROLL, int MODE>
 __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __restrict__ x, uint8_t* __restrict__ scales,
                                                                   uint2* __restrict__ elements, uint4* __restrict__ out,
-                                                                  int64_t n_chunks, F f, ScaledGeom sg) {
+                                                                  int64_t n_chunks, F f) {
     const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
-    uint32_t sg_row0 = 0, sg_kb0 = 0;
-    if constexpr (MODE == 2) {   // (row, k block) of the workgroup's first block
-        const uint32_t b0 = blockIdx.x * (uint32_t)(UNROLL * kThreads / 4);
-        sg_row0 = b0 / sg.kblocks;
-        sg_kb0 = b0 - sg_row0 * sg.kblocks;
-    }
     uint4 raw[UNROLL];
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
@@ -493,65 +523,66 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
         const int64_t c = chunk0 + (int64_t)r * kThreads;
-        const uint32_t h[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
-        // block maximum of |x| bits: packed max over the lane's four registers, then the two halves,
-        // then the four lanes of the block (DPP quad permutes)
-        u16x2 m2 = __builtin_elementwise_max(__builtin_elementwise_max(as_u16x2(h[0] & 0x7FFF7FFFu), as_u16x2(h[1] & 0x7FFF7FFFu)),
-                                             __builtin_elementwise_max(as_u16x2(h[2] & 0x7FFF7FFFu), as_u16x2(h[3] & 0x7FFF7FFFu)));
-        uint32_t amax = max((uint32_t)m2[0], (uint32_t)m2[1]);
-        amax = max(amax, (uint32_t)__builtin_amdgcn_mov_dpp((int)amax, 0xB1, 0xF, 0xF, true));  // lane ^ 1
-        amax = max(amax, (uint32_t)__builtin_amdgcn_mov_dpp((int)amax, 0x4E, 0xF, 0xF, true));  // lane ^ 2
-        const int ef_max = (int)(amax >> 7);
-        const int scale_n = max(ef_max - fmt_emax_unb(f), 0);  // amax == 0 gives 0: the all-flushed rule
-        // (scale_n < bias: the packed arithmetic subtracts (scale_n - bias) << 7 with unsigned saturation)
-        const bool hard = amax >= 0x7F80u || scale_n >= 151 || (amax != 0u && scale_n < fmt_bias(f) + (MODE == 1 ? 1 : 0));
-        uint32_t o[4];
-        uint32_t scale = (uint32_t)scale_n;
-        if (__builtin_amdgcn_ballot_w64(hard) == 0) {
-            const uint32_t ssb = (uint32_t)((scale_n - fmt_bias(f)) << 7) & 0xFFFFu;
-            const uint32_t ssb2 = ssb | (ssb << 16);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) o[j] = MODE != 1 ? PackedBf16<F>::codes(h[j], ssb2) : PackedBf16<F>::qdq(h[j], ssb2);
-        } else {
-            // exact per-element routine (the block's lanes agree on amax, so they agree on the result)
-            const uint32_t amax32 = amax << 16;
-            const int se = shared_exponent<F, true>(amax32, f);
-            scale = amax32 < 0x00800000u ? 0u : (uint32_t)(se + 127);
-            const float sc = scale_f32(scale);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t c0 = encode_mxfp_element(h[j] << 16, se, f), c1 = encode_mxfp_element(h[j] & 0xFFFF0000u, se, f);
-                o[j] = MODE != 1 ? (c0 | (c1 << 16)) : pack_bf16(mxfp_value(c0, sc, f), mxfp_value(c1, sc, f));
-            }
-        }
+        uint32_t o[4], scale;
+        bf16_block_step<F, MODE == 1>(raw[r], f, o, scale);
         if (c < n_chunks) {
             if (MODE == 0) {
                 // o[j] holds two codes in the low bytes of its halves: gather the 8 code bytes
                 st64(elements + c, make_uint2(__builtin_amdgcn_perm(o[1], o[0], 0x06040200u), __builtin_amdgcn_perm(o[3], o[2], 0x06040200u)));
                 if ((c & 3) == 0) scales[c >> 2] = (uint8_t)scale;
-            } else if (MODE == 1) {
+            } else {
                 st128(out + c, make_uint4(o[0], o[1], o[2], o[3]));
             }
         }
-        if constexpr (MODE == 2) {
-            uint32_t w0 = __builtin_amdgcn_perm(o[1], o[0], 0x06040200u), w1 = __builtin_amdgcn_perm(o[3], o[2], 0x06040200u);
-            if constexpr (F{}.E() == 4 && F{}.M() == 3) {
-                uint32_t top = e4m3_top_bits(w0) | e4m3_top_bits(w1);
-                top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xF, 0xF, true);
-                top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0x4E, 0xF, 0xF, true);
-                if (top != 0u && scale < 254u) {   // (a block of scale 255 holds inf / NaN: its row of the product is NaN either way)
-                    w0 = e4m3_halve4(w0);
-                    w1 = e4m3_halve4(w1);
-                    scale += 1u;
-                }
-            } else {
-                w0 = embed_e4m3_x4(w0, f);
-                w1 = embed_e4m3_x4(w1, f);
+    }
+}
+
+// bf16 matrix x [rows, K] -> operand of the block-scaled GEMM in one pass (extract, then the re-encoding / embedding
+// above).  A workgroup owns 32 rows x 128 k, the unit whose scale dwords fill one 128-byte line of the transposed scale
+// array: 16 lanes read the 256 bytes of one row (8 elements each, four lanes to a block), a wavefront four rows per
+// step, two steps.  The four scale bytes of a row are gathered into one lane and stored as a dword.
+template <class F>
+__global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes,
+                                                                      uint32_t* __restrict__ scales, int rows, int K, int nmac,
+                                                                      uint32_t rows_pad, F f) {
+    const uint32_t ms = blockIdx.x % (uint32_t)nmac, row_base = (blockIdx.x / (uint32_t)nmac) * 32u;
+    const int t = threadIdx.x;
+    uint4 raw[2];
+    size_t off[2];
+    bool live[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const uint32_t row = row_base + 16u * r + (uint32_t)(t >> 4);
+        live[r] = row < (uint32_t)rows;
+        off[r] = (size_t)row * K + ms * 128u + (uint32_t)(t & 15) * 8u;
+        raw[r] = live[r] ? ld128(x + off[r]) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        uint32_t o[4], scale;
+        bf16_block_step<F, false>(raw[r], f, o, scale);
+        uint32_t w0 = __builtin_amdgcn_perm(o[1], o[0], 0x06040200u), w1 = __builtin_amdgcn_perm(o[3], o[2], 0x06040200u);
+        if constexpr (F{}.E() == 4 && F{}.M() == 3) {
+            uint32_t top = e4m3_top_bits(w0) | e4m3_top_bits(w1);
+            top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xF, 0xF, true);
+            top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0x4E, 0xF, 0xF, true);
+            if (top != 0u && scale < 254u) {   // (a block of scale 255 holds inf / NaN: its row of the product is NaN either way)
+                w0 = e4m3_halve4(w0);
+                w1 = e4m3_halve4(w1);
+                scale += 1u;
             }
-            if (c < n_chunks) {
-                st64(elements + c, make_uint2(w0, w1));
-                if ((c & 3) == 0) scales[scaled_scale_offset(sg_row0, sg_kb0, (uint32_t)((threadIdx.x + r * kThreads) >> 2), sg)] = (uint8_t)scale;
-            }
+        } else {
+            w0 = embed_e4m3_x4(w0, f);
+            w1 = embed_e4m3_x4(w1, f);
+        }
+        // the row's four scale bytes (lanes 0, 4, 8, 12 of its 16) into its first lane: row_shl 4, 8, 12
+        uint32_t dw = scale;
+        dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x104, 0xF, 0xF, true) << 8;
+        dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x108, 0xF, 0xF, true) << 16;
+        dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x10C, 0xF, 0xF, true) << 24;
+        if (live[r]) {
+            st64(codes + off[r], make_uint2(w0, w1));
+            if ((t & 15) == 0) scales[(size_t)ms * rows_pad + row_base + 16u * r + (uint32_t)(t >> 4)] = dw;
         }
     }
 }
@@ -1115,7 +1146,7 @@ int mase_hip_extract_mxfp(const void* x, int x_dtype, uint8_t* scales, uint8_t* 
             if (x_dtype == BF16 && B == 32 && vec) {
                 constexpr int U = MASE_UNROLL_PACKED;
                 hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 0>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
-                                   static_cast<const uint4*>(x), scales, reinterpret_cast<uint2*>(elements), nullptr, n / 8, f, ScaledGeom{});
+                                   static_cast<const uint4*>(x), scales, reinterpret_cast<uint2*>(elements), nullptr, n / 8, f);
                 return check_launch("extract_mxfp");
             }
         }
@@ -1183,7 +1214,7 @@ int mase_hip_qdq_mxfp(const void* x, int x_dtype, void* out, int out_dtype, int6
             if (x_dtype == BF16 && out_dtype == BF16 && B == 32 && vec) {
                 constexpr int U = MASE_UNROLL_PACKED;
                 hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 1>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
-                                   static_cast<const uint4*>(x), nullptr, nullptr, static_cast<uint4*>(out), n / 8, f, ScaledGeom{});
+                                   static_cast<const uint4*>(x), nullptr, nullptr, static_cast<uint4*>(out), n / 8, f);
                 return check_launch("qdq_mxfp");
             }
         }
@@ -1345,13 +1376,13 @@ int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits,
     if (!x || !out_codes || !out_scales) return fail(ERR_INVALID, "null pointer");
     if (!aligned(x, 16) || !aligned(out_codes, 8) || !aligned(out_scales, 4)) return fail(ERR_INVALID, "x must be 16-byte aligned, out_codes 8-byte, out_scales 4-byte");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int64_t n = rows * K;
     return dispatch_fmt(exp_bits, frac_bits, 1, RN, [&](auto f) {
         if constexpr (decltype(f)::kStatic && decltype(f){}.E() != 5) {
-            constexpr int U = MASE_UNROLL_PACKED;
-            hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 2>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
-                               static_cast<const uint4*>(x), reinterpret_cast<uint8_t*>(out_scales), reinterpret_cast<uint2*>(out_codes), nullptr,
-                               n / 8, f, sg);
+            const int nmac = (int)(K / 128);
+            const int64_t blocks = (rows + 31) / 32 * nmac;
+            if (blocks > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "operand too large for one launch");
+            hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f)>), dim3((unsigned)blocks), dim3(kThreads), 0, s, static_cast<const uint16_t*>(x),
+                               out_codes, out_scales, (int)rows, (int)K, nmac, sg.rows_pad, f);
             return check_launch("scaled_operand_from_dense");
         }
         return fail(ERR_UNSUPPORTED, "element format not supported by the block-scaled GEMM");

@@ -24,7 +24,7 @@
 //   period c    multiplies chunk c's A rows, reads chunk c's W rows into the registers of the next macro step,
 //               and issues the DMAs of chunk c + 3 (into the slot that chunk c - 1 left), spread over the period
 //   barrier c+1 sits before the last eight MFMAs of period c: every wave has finished reading chunk c, and has waited
-//               until its own DMAs of chunk c + 1 (issued two periods earlier: vmcnt(18)) have landed
+//               until its own DMAs of chunk c + 1 (issued two periods earlier: vmcnt(20)) have landed
 //
 // so a DMA has between two and three periods (2000 - 3000 cycles) to land and the address unit sees an even stream.
 // (included from gemm_impl.h's namespace, after gemm_tall.h whose asm helpers it shares)
@@ -40,6 +40,7 @@ constexpr int S_OUT_OFF = S_SC_OFF + S_RING * S_SC_BYTES;     // [4 waves][32 ro
 constexpr int S_LDS_BYTES = S_OUT_OFF + 4 * 4096;             // 148 KB
 
 typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
 
 // c += w (16 n x 128 k, scales sw) * a (16 m x 128 k, scales sa)^T
 __device__ inline void mfma_scaled(floatx4& c, const intx8& w, const intx8& a, uint32_t sw, uint32_t sa) {
@@ -48,9 +49,12 @@ __device__ inline void mfma_scaled(floatx4& c, const intx8& w, const intx8& a, u
 __device__ inline void mfma_scaled_first(floatx4& c, const intx8& w, const intx8& a, uint32_t sw, uint32_t sa) {
     asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel_hi:[0,0,0]" : "=a"(c) : "v"(w), "v"(a), "v"(sw), "v"(sa));
 }
-// 64 lanes x 4 bytes from per-lane 64-bit addresses to LDS [lds_addr, lds_addr + 256)
-__device__ inline void dma_dwords(uint32_t lds_addr, const void* lane_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(lane_addr) : "memory");
+// for the lanes in `mask`: 4 bytes from (sbase + voff) to LDS lds_addr + 4 * lane.  (The mask is applied here and not by
+// a branch around the call: the LDS address has to stay in a scalar register.)
+__device__ inline void dma_dwords_masked(uint32_t lds_addr, uint32_t voff, const void* sbase, uint64_t mask) {
+    uint64_t saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved) : "s"(lds_addr), "v"(voff), "s"(sbase), "s"(mask) : "memory");
 }
 
 // 16 bytes to a per-lane address (non-temporal: the output is not read again by this kernel); the trailing s_nop keeps a
@@ -60,10 +64,6 @@ __device__ inline void store16_nt(void* dst, const u32x4& v) {
 }
 
 struct ScaledTile {
-    const uint8_t* a;    // codes of the tile's first A row
-    const uint8_t* w;    // codes of the tile's first W row
-    const uint32_t* as;  // scale dword of the tile's first A row, macro step 0
-    const uint32_t* ws;
     int m0, n0;
 };
 
@@ -82,8 +82,10 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     // ---- per-lane constants
     // data DMA d (0..3) of a wave covers rows 32 wave + 8 d .. + 7 of a chunk part; lane l fills position l & 7 of row
     // 8 d + (l >> 3), which must hold the row's 16-byte piece (l & 7) ^ (row >> 1 & 7) = (l & 7) ^ ((4 d + (l >> 4)) & 7)
-    const uint32_t dma_voff_even = (uint32_t)(lane >> 3) * (uint32_t)K + (uint32_t)((((lane & 7) ^ (lane >> 4)) & 7) << 4);
-    const uint32_t dma_voff_odd = dma_voff_even ^ 64u;
+    uint32_t dma_voff[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+        dma_voff[d] = (uint32_t)(8 * d + (lane >> 3)) * (uint32_t)K + (uint32_t)((((lane & 7) ^ ((4 * d + (lane >> 4)) & 7))) << 4);
     // fragment reads: lane (g = l >> 4, r = l & 15) reads pieces g and g + 4 of row r of its 16-row tile
     const uint32_t f_off = (uint32_t)(lane & 15) * 128u + (uint32_t)((((lane >> 4) ^ ((lane >> 1) & 7)) & 7) << 4);
     const uint8_t* const a_frag0 = lds + S_A_OFF + wave_m * (64 * 128) + f_off;
@@ -109,10 +111,6 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         ScaledTile t;
         t.m0 = (first_m + rr % rows) * SM;
         t.n0 = (rr / rows) * SN;
-        t.a = a_codes + (size_t)t.m0 * K;
-        t.w = w_codes + (size_t)t.n0 * K;
-        t.as = a_scales + t.m0;
-        t.ws = w_scales + t.n0;
         return t;
     };
 
@@ -120,51 +118,37 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     if (!has_tile(local)) return;
     ScaledTile cur = tile_at(local), next = cur;
 
-    // ---- DMAs of the chunk (macro step ma of A, macro step ma + 1 of W, half h) into ring slot `slot`; ma may run past
-    //      the tile's end, into the next tile.  PART 0..2: three of the nine operations each.
-    const int rows_in_part = 32 * wave;   // this wave's first row within a chunk part
-    auto issue_chunk = [&](int ma, int h, int slot, auto part_c) __attribute__((always_inline)) {
-        constexpr int PART = decltype(part_c)::value;
-        const bool a_wrap = ma >= nmac;
-        const int mw = ma + 1;
-        const bool w_wrap = mw >= nmac;
-        const ScaledTile& ta = a_wrap ? next : cur;
-        const ScaledTile& tw = w_wrap ? next : cur;
-        const int ma_t = a_wrap ? ma - nmac : ma, mw_t = w_wrap ? mw - nmac : mw;
-        // the wave's 32 rows of the part are tile rows 128 (wave >> 1) + 64 h + 32 (wave & 1) ..
-        const int row0 = 128 * (wave >> 1) + 64 * h + 32 * (wave & 1);
-        const uint8_t* const a_src = ta.a + (size_t)row0 * K + (size_t)ma_t * SMAC;
-        const uint8_t* const w_src = tw.w + (size_t)row0 * K + (size_t)mw_t * SMAC;
-        const uint32_t lds_a = lds_base + S_A_OFF + slot * S_PART_BYTES + rows_in_part * 128;
-        const uint32_t lds_w = lds_base + S_W_OFF + slot * S_PART_BYTES + rows_in_part * 128;
-        if constexpr (PART == 0) {
-            dma_1kb(lds_a, dma_voff_even, a_src);
-            dma_1kb(lds_a + 1024, dma_voff_odd, a_src + (size_t)8 * K);
-            dma_1kb(lds_a + 2048, dma_voff_even, a_src + (size_t)16 * K);
-        } else if constexpr (PART == 1) {
-            dma_1kb(lds_a + 3072, dma_voff_odd, a_src + (size_t)24 * K);
-            dma_1kb(lds_w, dma_voff_even, w_src);
-            dma_1kb(lds_w + 1024, dma_voff_odd, w_src + (size_t)8 * K);
-        } else {
-            dma_1kb(lds_w + 2048, dma_voff_even, w_src + (size_t)16 * K);
-            dma_1kb(lds_w + 3072, dma_voff_odd, w_src + (size_t)24 * K);
-            // scales: lanes 0..31 the dwords of the wave's 32 A rows, lanes 32..63 those of its 32 W rows
-            const uint32_t* const sp = lane < 32 ? ta.as + (size_t)ma_t * rows_a + row0 + lane : tw.ws + (size_t)mw_t * rows_w + row0 + (lane - 32);
-            dma_dwords(lds_base + S_SC_OFF + slot * S_SC_BYTES + wave * 256, sp);
-        }
+    // ---- The DMA streams.  A chunk = (macro step ma of A, macro step ma + 1 of W, half h): ten operations per wave, its
+    //      32 rows of A and of W (four of 8 rows each) and the scale dwords of those rows (lanes 0..31 those of A, lanes
+    //      32..63 those of W).  Each half of each operand is a stream of its own that moves one macro step along K per
+    //      chunk and jumps to the next tile when it passes the end of this one (the W streams one macro step before the
+    //      A streams).
+    const int row0_w = 128 * (wave >> 1) + 32 * (wave & 1);   // this wave's first row of a part, as a row of the tile, for half 0
+    const uint32_t wave_lds = lds_base + (uint32_t)wave * 4096u;   // ... and its place within a chunk part
+    const uint32_t wave_lds_sc = lds_base + (uint32_t)wave * 256u;
+    const uint32_t sc_voff = (uint32_t)(lane & 31) * 4u;
+    const uint8_t *pa[2], *pw[2];      // where the next chunk of half h reads its codes ...
+    const uint32_t *pas[2], *pws[2];   // ... and its scales
+    auto a_stream_to = [&](const ScaledTile& t, int h) __attribute__((always_inline)) {
+        const int row = t.m0 + row0_w + 64 * h;
+        pa[h] = a_codes + (size_t)row * K;
+        pas[h] = a_scales + row;
     };
-    // the W half of a chunk alone (the first tile's first macro step of W travels in two chunks of its own)
-    auto issue_w_only = [&](int mw_t, int h, int slot) __attribute__((always_inline)) {
-        const int row0 = 128 * (wave >> 1) + 64 * h + 32 * (wave & 1);
-        const uint8_t* const w_src = cur.w + (size_t)row0 * K + (size_t)mw_t * SMAC;
-        const uint32_t lds_w = lds_base + S_W_OFF + slot * S_PART_BYTES + rows_in_part * 128;
-        dma_1kb(lds_w, dma_voff_even, w_src);
-        dma_1kb(lds_w + 1024, dma_voff_odd, w_src + (size_t)8 * K);
-        dma_1kb(lds_w + 2048, dma_voff_even, w_src + (size_t)16 * K);
-        dma_1kb(lds_w + 3072, dma_voff_odd, w_src + (size_t)24 * K);
-        const uint32_t* const sp = cur.ws + (size_t)mw_t * rows_w + row0 + (lane & 31);   // lanes 0..31 land where nobody looks
-        dma_dwords(lds_base + S_SC_OFF + slot * S_SC_BYTES + wave * 256, sp);
+    auto w_stream_to = [&](const ScaledTile& t, int h) __attribute__((always_inline)) {
+        const int row = t.n0 + row0_w + 64 * h;
+        pw[h] = w_codes + (size_t)row * K;
+        pws[h] = w_scales + row;
     };
+    // operation q (0..9) of the next chunk of half H into ring slot SLOT
+    auto chunk_dma = [&](auto h_c, auto slot_c, auto q_c) __attribute__((always_inline)) {
+        constexpr int H = decltype(h_c)::value, SLOT = decltype(slot_c)::value, q = decltype(q_c)::value;
+        if constexpr (q < 4) dma_1kb(wave_lds + (S_A_OFF + SLOT * S_PART_BYTES + q * 1024), dma_voff[q], pa[H]);
+        else if constexpr (q < 8) dma_1kb(wave_lds + (S_W_OFF + SLOT * S_PART_BYTES + (q - 4) * 1024), dma_voff[q - 4], pw[H]);
+        else if constexpr (q == 8) dma_dwords_masked(wave_lds_sc + (S_SC_OFF + SLOT * S_SC_BYTES), sc_voff, pas[H], 0x00000000FFFFFFFFull);
+        else dma_dwords_masked(wave_lds_sc + (S_SC_OFF + SLOT * S_SC_BYTES), sc_voff, pws[H], 0xFFFFFFFF00000000ull);
+    };
+    auto a_advance = [&](int h) __attribute__((always_inline)) { pa[h] += SMAC; pas[h] += rows_a; };
+    auto w_advance = [&](int h) __attribute__((always_inline)) { pw[h] += SMAC; pws[h] += rows_w; };
 
     floatx4 acc[8][8];        // [n-tile j][m-tile i]
     intx8 wreg[2][8];         // the W fragments of the macro step in flight and of the next one
@@ -172,97 +156,111 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     intx8 areg[2];            // A fragment ring
     uint32_t asc[2][4];       // scale bytes of the period's four m-tiles, and of the next period's
 
-    // fragment t (0..3) of ring slot `slot`
-    auto read_a = [&](intx8& dst, int slot, int t) __attribute__((always_inline)) {
-        const uint4 lo = *reinterpret_cast<const uint4*>(a_frag0 + slot * S_PART_BYTES + t * 2048);
-        const uint4 hi = *reinterpret_cast<const uint4*>(a_frag1 + slot * S_PART_BYTES + t * 2048);
-        dst = intx8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-    };
-    auto read_w = [&](intx8& dst, uint32_t& sc, int slot, int t) __attribute__((always_inline)) {
-        const uint4 lo = *reinterpret_cast<const uint4*>(w_frag0 + slot * S_PART_BYTES + t * 2048);
-        const uint4 hi = *reinterpret_cast<const uint4*>(w_frag1 + slot * S_PART_BYTES + t * 2048);
-        dst = intx8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        sc = w_sc[slot * S_SC_BYTES + (t >> 1) * 256 + (t & 1) * 64];
-    };
-    auto read_a_scales = [&](uint32_t(&dst)[4], int slot) __attribute__((always_inline)) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) dst[t] = a_sc[slot * S_SC_BYTES + (t >> 1) * 256 + (t & 1) * 64];
-    };
+    // halves of fragment t (0..3) of ring slot `slot`
+    auto read_a_lo = [&](intx8& dst, int slot, int t) __attribute__((always_inline)) { dst.lo = *reinterpret_cast<const intx4*>(a_frag0 + slot * S_PART_BYTES + t * 2048); };
+    auto read_a_hi = [&](intx8& dst, int slot, int t) __attribute__((always_inline)) { dst.hi = *reinterpret_cast<const intx4*>(a_frag1 + slot * S_PART_BYTES + t * 2048); };
+    auto read_w_lo = [&](intx8& dst, int slot, int t) __attribute__((always_inline)) { dst.lo = *reinterpret_cast<const intx4*>(w_frag0 + slot * S_PART_BYTES + t * 2048); };
+    auto read_w_hi = [&](intx8& dst, int slot, int t) __attribute__((always_inline)) { dst.hi = *reinterpret_cast<const intx4*>(w_frag1 + slot * S_PART_BYTES + t * 2048); };
+    auto read_w_sc = [&](uint32_t& sc, int slot, int t) __attribute__((always_inline)) { sc = w_sc[slot * S_SC_BYTES + (t >> 1) * 256 + (t & 1) * 64]; };
+    auto read_a_sc = [&](uint32_t& sc, int slot, int t) __attribute__((always_inline)) { sc = a_sc[slot * S_SC_BYTES + (t >> 1) * 256 + (t & 1) * 64]; };
 
-    // ---- prologue of the stream: W macro step 0 of the first tile through slots 2 and 3, chunks 0 and 1, then chunk 2
-    issue_w_only(0, 0, 2);
-    issue_w_only(0, 1, 3);
-    issue_chunk(0, 0, 0, IntC<0>{});
-    issue_chunk(0, 0, 0, IntC<1>{});
-    issue_chunk(0, 0, 0, IntC<2>{});
-    issue_chunk(0, 1, 1, IntC<0>{});
-    issue_chunk(0, 1, 1, IntC<1>{});
-    issue_chunk(0, 1, 1, IntC<2>{});
-    asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+    // ---- prologue of the stream: W macro step 0 of the first tile travels alone through slots 2 and 3 (as the W halves
+    //      of chunks "-2" and "-1"); then chunks 0, 1, 2.  The waits here are total: only the steady state counts.
+    a_stream_to(cur, 0); a_stream_to(cur, 1); w_stream_to(cur, 0); w_stream_to(cur, 1);
+    auto issue_w_half = [&](auto h_c, auto slot_c) __attribute__((always_inline)) {
+        chunk_dma(h_c, slot_c, IntC<4>{}); chunk_dma(h_c, slot_c, IntC<5>{}); chunk_dma(h_c, slot_c, IntC<6>{});
+        chunk_dma(h_c, slot_c, IntC<7>{}); chunk_dma(h_c, slot_c, IntC<9>{});
+        w_advance(decltype(h_c)::value);
+    };
+    auto issue_a_half = [&](auto h_c, auto slot_c) __attribute__((always_inline)) {
+        chunk_dma(h_c, slot_c, IntC<0>{}); chunk_dma(h_c, slot_c, IntC<1>{}); chunk_dma(h_c, slot_c, IntC<2>{});
+        chunk_dma(h_c, slot_c, IntC<3>{}); chunk_dma(h_c, slot_c, IntC<8>{});
+        a_advance(decltype(h_c)::value);
+    };
+    issue_w_half(IntC<0>{}, IntC<2>{});
+    issue_w_half(IntC<1>{}, IntC<3>{});
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        read_w(wreg[0][t], wsc[0][t], 2, t);
-        read_w(wreg[0][4 + t], wsc[0][4 + t], 3, t);
+        read_w_lo(wreg[0][t], 2, t); read_w_hi(wreg[0][t], 2, t); read_w_sc(wsc[0][t], 2, t);
+        read_w_lo(wreg[0][4 + t], 3, t); read_w_hi(wreg[0][4 + t], 3, t); read_w_sc(wsc[0][4 + t], 3, t);
     }
     lds_barrier();   // slots 2 and 3 are free again
-    issue_chunk(1, 0, 2, IntC<0>{});
-    issue_chunk(1, 0, 2, IntC<1>{});
-    issue_chunk(1, 0, 2, IntC<2>{});
-    asm volatile("s_waitcnt vmcnt(18)" ::: "memory");   // chunk 0 has landed
+    issue_a_half(IntC<0>{}, IntC<0>{}); issue_w_half(IntC<0>{}, IntC<0>{});
+    issue_a_half(IntC<1>{}, IntC<1>{}); issue_w_half(IntC<1>{}, IntC<1>{});
+    issue_a_half(IntC<0>{}, IntC<2>{}); issue_w_half(IntC<0>{}, IntC<2>{});
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
-    read_a(areg[0], 0, 0);
-    read_a_scales(asc[0], 0);
+    read_a_lo(areg[0], 0, 0); read_a_hi(areg[0], 0, 0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) read_a_sc(asc[0][t], 0, t);
 
     // One period: H = half of the macro step (m-tiles 4 H .. 4 H + 3), C4 = ring slot of its chunk, WC = register set of
-    // the macro step's W fragments.  ma = macro step (of the current tile).
+    // the macro step's W fragments.  ma = macro step (of the current tile).  Every MFMA is followed by at most a few
+    // other instructions (a wave can issue about six under one 32-cycle MFMA), in this order, pinned by scheduling
+    // barriers: the period's ten DMAs, the reads of the next A fragment and of the next macro step's W fragments.
     auto period = [&](int ma, auto h_c, auto c4_c, auto wc_c, auto first_c) __attribute__((always_inline)) {
         constexpr int H = decltype(h_c)::value, C4 = decltype(c4_c)::value, WC = decltype(wc_c)::value;
         constexpr bool FIRST = decltype(first_c)::value != 0;
         constexpr int WN = WC ^ 1, NEXT_SLOT = (C4 + 1) & 3, ISSUE_SLOT = (C4 + 3) & 3;
         constexpr int AS = H, ASN = H ^ 1;   // scale register set of this period, of the next
-        // the chunk issued during this period: three periods ahead
-        const int issue_ma = H == 0 ? ma + 1 : ma + 2;
-        constexpr int issue_h = H ^ 1;
-        auto mm8 = [&](const intx8& a, uint32_t sa, auto i_c) __attribute__((always_inline)) {
-            constexpr int i = decltype(i_c)::value;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                if (FIRST) mfma_scaled_first(acc[j][i], wreg[WC][j], a, wsc[WC][j], sa);
-                else mfma_scaled(acc[j][i], wreg[WC][j], a, wsc[WC][j], sa);
-            }
+        // the chunk issued during this period: three periods ahead, the other half; its streams may have to move on to
+        // the next tile first
+        constexpr int IH = H ^ 1;
+        {
+            const int issue_ma = H == 0 ? ma + 1 : ma + 2;
+            if (issue_ma == nmac) a_stream_to(next, IH);
+            if (issue_ma == nmac - 1) w_stream_to(next, IH);
+        }
+        auto dma = [&](auto q_c) __attribute__((always_inline)) { chunk_dma(IntC<IH>{}, IntC<ISSUE_SLOT>{}, q_c); };
+        auto mm = [&](const intx8& a, uint32_t sa, auto i_c, auto j_c) __attribute__((always_inline)) {
+            constexpr int i = decltype(i_c)::value, j = decltype(j_c)::value;
+            if (FIRST) mfma_scaled_first(acc[j][i], wreg[WC][j], a, wsc[WC][j], sa);
+            else mfma_scaled(acc[j][i], wreg[WC][j], a, wsc[WC][j], sa);
         };
 #define S_SLOT_END() __builtin_amdgcn_sched_barrier(0)
-        // row 0
-        read_a(areg[1], C4, 1);
-        read_w(wreg[WN][4 * H + 0], wsc[WN][4 * H + 0], C4, 0);
-        read_w(wreg[WN][4 * H + 1], wsc[WN][4 * H + 1], C4, 1);
-        issue_chunk(issue_ma, issue_h, ISSUE_SLOT, IntC<0>{});
-        S_SLOT_END();
-        mm8(areg[0], asc[AS][0], IntC<4 * H + 0>{});
-        S_SLOT_END();
-        // row 1
-        read_a(areg[0], C4, 2);
-        read_w(wreg[WN][4 * H + 2], wsc[WN][4 * H + 2], C4, 2);
-        issue_chunk(issue_ma, issue_h, ISSUE_SLOT, IntC<1>{});
-        S_SLOT_END();
-        mm8(areg[1], asc[AS][1], IntC<4 * H + 1>{});
-        S_SLOT_END();
-        // row 2
-        read_a(areg[1], C4, 3);
-        read_w(wreg[WN][4 * H + 3], wsc[WN][4 * H + 3], C4, 3);
-        issue_chunk(issue_ma, issue_h, ISSUE_SLOT, IntC<2>{});
-        S_SLOT_END();
-        mm8(areg[0], asc[AS][2], IntC<4 * H + 2>{});
-        S_SLOT_END();
-        // row 3: the next chunk has landed everywhere, this one is no longer read
-        asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
-        lds_barrier();
-        read_a(areg[0], NEXT_SLOT, 0);
-        read_a_scales(asc[ASN], NEXT_SLOT);
-        S_SLOT_END();
-        mm8(areg[1], asc[AS][3], IntC<4 * H + 3>{});
-        S_SLOT_END();
+        // rows 0..2: m-tile 4 H + r against the eight n-tiles; beside them the A fragment of row r + 1, W fragment(s) of the
+        // next macro step, three or four DMAs
+        static_for<3>([&](auto r_c) __attribute__((always_inline)) {
+            constexpr int r = decltype(r_c)::value;
+            constexpr int i = 4 * H + r;
+            intx8& a_now = areg[r & 1];
+            intx8& a_nxt = areg[(r + 1) & 1];
+            const uint32_t sa = asc[AS][r];
+            constexpr int wt = r == 0 ? 0 : r + 1;          // W fragment read in this row (row 0 reads two: 0 and 1)
+            mm(a_now, sa, IntC<i>{}, IntC<0>{}); read_a_lo(a_nxt, C4, r + 1); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<1>{}); read_a_hi(a_nxt, C4, r + 1); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<2>{}); dma(IntC<r == 0 ? 0 : r == 1 ? 3 : 7>{}); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<3>{}); read_w_lo(wreg[WN][4 * H + wt], C4, wt); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<4>{}); read_w_hi(wreg[WN][4 * H + wt], C4, wt); read_w_sc(wsc[WN][4 * H + wt], C4, wt); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<5>{}); dma(IntC<r == 0 ? 1 : r == 1 ? 4 : 8>{}); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<6>{});
+            if constexpr (r == 0) { read_w_lo(wreg[WN][4 * H + 1], C4, 1); read_w_hi(wreg[WN][4 * H + 1], C4, 1); read_w_sc(wsc[WN][4 * H + 1], C4, 1); }
+            else dma(IntC<r == 1 ? 5 : 9>{});
+            S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<7>{});
+            if constexpr (r < 2) dma(IntC<r == 0 ? 2 : 6>{});
+            if constexpr (r == 2) { a_advance(IH); w_advance(IH); }
+            S_SLOT_END();
+        });
+        // row 3: the next chunk has landed everywhere (this wave's part of it was issued two periods ago: 20 younger
+        // operations), this one is no longer read
+        {
+            constexpr int i = 4 * H + 3;
+            intx8& a_now = areg[1];
+            const uint32_t sa = asc[AS][3];
+            asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+            lds_barrier();
+            mm(a_now, sa, IntC<i>{}, IntC<0>{}); read_a_lo(areg[0], NEXT_SLOT, 0); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<1>{}); read_a_hi(areg[0], NEXT_SLOT, 0); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<2>{}); read_a_sc(asc[ASN][0], NEXT_SLOT, 0); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<3>{}); read_a_sc(asc[ASN][1], NEXT_SLOT, 1); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<4>{}); read_a_sc(asc[ASN][2], NEXT_SLOT, 2); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<5>{}); read_a_sc(asc[ASN][3], NEXT_SLOT, 3); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<6>{}); S_SLOT_END();
+            mm(a_now, sa, IntC<i>{}, IntC<7>{}); S_SLOT_END();
+        }
 #undef S_SLOT_END
     };
 
