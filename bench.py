@@ -82,9 +82,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--skip-hbm", action="store_true", help="skip the cast-kernel bandwidth section")
-    ap.add_argument("--only-gemm-kernel", choices=("scaled", "bf16"), default=None,
-                    help="profiling aid: launch only that GEMM kernel (block-scaled FP8 or bf16 MFMA) on the headline shape, "
-                         "--steps times after --warmup, and print nothing")
+    ap.add_argument("--only-gemm-kernel", choices=("scaled", "bf16", "bf16-components"), default=None,
+                    help="profiling aid: launch only that GEMM kernel (block-scaled FP8; bf16 MFMA on the prepared weight; bf16 MFMA on "
+                         "the weight components) on the headline shape, --steps times after --warmup, and print nothing")
     ap.add_argument("--summarize-sq", metavar="COUNTER_CSV",
                     help="no GPU needed: per-kernel table (stdout, markdown) from the counter_collection.csv of a rocprofv3 --pmc run with "
                          "SQ_BUSY_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_LDS SQ_WAIT_ANY SQ_WAVE_CYCLES SQ_WAVES [SQ_LDS_BANK_CONFLICT]")
@@ -177,10 +177,22 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
             ev[1].record()
         return y
 
-    if args.only_gemm_kernel:
-        a_op, w_op = kernels.scaled_operand_from_dense(x, fmt), L.scaled_weight_operand(w_sc, w_el, w_tm)
+    def step_bf16_kept(ev=None):
+        # the same with the weight operand a layer keeps: the 512 x 128 kernel reads the prepared form
         a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
-        fn = ((lambda: kernels.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)) if args.only_gemm_kernel == "scaled" else
+        if ev is not None:
+            ev[0].record()
+        y = kernels.mxfp_gemm_prepared_w(a, w_kept, None, torch.bfloat16)
+        if ev is not None:
+            ev[1].record()
+        return y
+
+    w_kept = L.scaled_weight_operand(w_sc, w_el, w_tm)      # what a layer keeps
+    if args.only_gemm_kernel:
+        a_op = kernels.scaled_operand_from_dense(x, fmt)
+        a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
+        fn = ((lambda: kernels.mxfp_gemm_scaled(a_op, w_kept, None, torch.bfloat16)) if args.only_gemm_kernel == "scaled" else
+              (lambda: kernels.mxfp_gemm_prepared_w(a, w_kept, None, torch.bfloat16)) if args.only_gemm_kernel == "bf16" else
               (lambda: kernels.mxfp_gemm(a, None, None, None, w_sc, w_el, fmt, None, M, N, K, torch.bfloat16)))
         timed_loop(torch, fn, args.steps, args.warmup)
         return None
@@ -188,6 +200,7 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
     y_api = MXFP_F.mxfp_linear(**call, backend="fused")
     assert torch.equal(step().view(torch.int16), y_api.view(torch.int16)), "bench step differs from mxfp_linear(backend='fused')"
     assert torch.equal(step_bf16().view(torch.int16), MXFP_F.mxfp_linear(**call, backend="fused_bf16").view(torch.int16))
+    assert torch.equal(step_bf16_kept().view(torch.int16), MXFP_F.mxfp_linear(**call, backend="fused_bf16", w_operand=w_kept).view(torch.int16))
     del y_api
     # The shader clock settles over the first few dozen launches after idle (the step gets faster), so a short counted
     # warm-up would time the ramp.  Before the counted warm-up: steps in groups of five until two consecutive groups agree
@@ -207,13 +220,12 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
         return ms, sum(event_ms(pairs)) / args.steps
 
     ms_per_step, gemm_ms = measure(step)
-    settle(torch, step_bf16)
-    bf16_ms, bf16_gemm_ms = measure(step_bf16)
+    settle(torch, step_bf16_kept)
+    bf16_ms, bf16_gemm_ms = measure(step_bf16_kept)
+    bf16c_ms, bf16c_gemm_ms = measure(step_bf16)
     # context, not the metric
     half = max(3, args.warmup // 2)
-    w_op = L.scaled_weight_operand(w_sc, w_el, w_tm)      # what a layer keeps
-    prepared_ms = timed_loop(torch, lambda: MXFP_F.mxfp_linear(**call, backend="fused", w_operand=w_op), args.steps, half)
-    del w_op
+    prepared_ms = timed_loop(torch, lambda: MXFP_F.mxfp_linear(**call, backend="fused", w_operand=w_kept), args.steps, half)
     # backend="separate": extract x, compose x, compose W to bf16 in HBM, the vendor library's dense bf16 GEMM
     sep_ms = timed_loop(torch, lambda: MXFP_F.mxfp_linear(**call, backend="separate"), args.steps, half)
     a_dq = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
@@ -225,6 +237,7 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
         "prewarm": prewarm, "shape": (M, N, K), "flop": flop,
         "ms_per_step": ms_per_step, "tflops_step": tf(ms_per_step), "gemm_ms": gemm_ms, "tflops_gemm": tf(gemm_ms),
         "bf16_ms_per_step": bf16_ms, "bf16_tflops_step": tf(bf16_ms), "bf16_gemm_ms": bf16_gemm_ms, "bf16_tflops_gemm": tf(bf16_gemm_ms),
+        "bf16c_ms_per_step": bf16c_ms, "bf16c_gemm_ms": bf16c_gemm_ms, "bf16c_tflops_gemm": tf(bf16c_gemm_ms),
         "prepared_ms": prepared_ms, "separate_ms": sep_ms, "dense_ms": dense_ms,
     }
 
@@ -559,7 +572,7 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
 
 
 # kernel-name fragments of the counter probe's launches ('a|b': all must occur; the last template argument of
-# mxfp_bf16_b32_kernel is its mode: 0 extract, 1 fused QDQ, 2 block-scaled operand) -> (key in the summary, algorithmic bytes
+# mxfp_bf16_b32_kernel is its mode: 0 extract, 1 fused QDQ) -> (key in the summary, algorithmic bytes
 # read, written, sources).  A key is "<kernel row of hbm_kernels> <config>" for the cast rows.
 _N1, _N3, _N2 = 4096 * 4096, 14336 * 4096, 1 << 24
 _M4, _N4, _K4 = 16384, 14336, 4096
@@ -567,7 +580,7 @@ COUNTER_ROWS = (
     ("stream_copy_kernel", "calibration copy (256 MiB read, 256 MiB written)", 256 << 20, 256 << 20, None),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C4", (_M4 + _N4) * _K4 * 33 // 32, _M4 * _N4 * 2, SCALED_SOURCES),
     ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", _M4 * _K4 * 2 + _N4 * _K4 * 33 // 32, _M4 * _N4 * 2, GEMM_SOURCES),
-    ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 2>(", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
+    ("scaled_from_dense_kernel", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
     ("scaled_operand_kernel", "scaled_operand_from_mxfp C4 W", _N4 * _K4 * 33 // 32, _N4 * _K4 * 33 // 32, CAST_SOURCES),
     ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 0>(", "extract_mxfp C1", _N1 * 2, _N1 + _N1 // 32, CAST_SOURCES),
     ("compose_mxfp_bf16_kernel<mase::SFmt<4, 3", "compose_mxfp C1", _N1 + _N1 // 32, _N1 * 2, CAST_SOURCES),
@@ -583,8 +596,7 @@ COUNTER_ROWS = (
     ("minifloat_f32_kernel<1, mase::SFmt<5, 2", "compose_minifloat C2/E5M2", _N2 * 2, _N2 * 4, CAST_SOURCES),
 )
 # launches of one kernel name at several sizes (the probe also quantises the headline's x and W): the size that is meant, in threads
-_COUNTER_THREADS = {"extract_mxfp C1": _N1 // 16, "extract_mxfp C3": _N3 // 16, "qdq_mxfp_fused C1": _N1 // 16, "qdq_mxfp_fused C3": _N3 // 16,
-                    "scaled_operand_from_dense C4 x": _M4 * _K4 // 16}
+_COUNTER_THREADS = {"extract_mxfp C1": _N1 // 16, "extract_mxfp C3": _N3 // 16, "qdq_mxfp_fused C1": _N1 // 16, "qdq_mxfp_fused C3": _N3 // 16}
 
 
 def summarize_counters(fetch_dir, write_dir):
@@ -845,9 +857,11 @@ def main():
                      "traffic": traffic_bytes("mxfp_gemm_scaled_kernel C4", SCALED_SOURCES),
                      "kernel": "mxfp_gemm_scaled_kernel", "avg_kernel_ms": round(lin["gemm_ms"], 4),
                      "frac_of_bf16_peak": round(lin["tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "bf16_kernel": {"kernel": "mxfp_gemm_tall_kernel", "achieved": round(lin["bf16_tflops_gemm"], 2), "peak": MFMA_BF16_PEAK_TFLOPS,
-                                     "frac": round(lin["bf16_tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4), "avg_kernel_ms": round(lin["bf16_gemm_ms"], 4),
-                                     "traffic": traffic_bytes("mxfp_gemm_tall_kernel C4", GEMM_SOURCES)}},
+                     "bf16_kernel": {"kernel": "mxfp_gemm_tall_kernel on the weight operand a layer keeps", "achieved": round(lin["bf16_tflops_gemm"], 2),
+                                     "peak": MFMA_BF16_PEAK_TFLOPS, "frac": round(lin["bf16_tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4),
+                                     "avg_kernel_ms": round(lin["bf16_gemm_ms"], 4), "traffic": traffic_bytes("mxfp_gemm_tall_kernel C4", GEMM_SOURCES),
+                                     "on_weight_components": {"achieved": round(lin["bf16c_tflops_gemm"], 2), "avg_kernel_ms": round(lin["bf16c_gemm_ms"], 4),
+                                                              "frac": round(lin["bf16c_tflops_gemm"] / MFMA_BF16_PEAK_TFLOPS, 4)}}},
     }
     result["cpu_baseline"] = None if args.no_cpu else cpu_baseline(torch)
     if not args.skip_hbm:
@@ -857,11 +871,13 @@ def main():
     result["context"] = {
         "same_shape_ms_per_step": {
             "fused (value)": round(lin["ms_per_step"], 4), "fused, weight operand kept by a layer": round(lin["prepared_ms"], 4),
-            "fused_bf16": round(lin["bf16_ms_per_step"], 4), "separate": round(lin["separate_ms"], 4),
+            "fused_bf16, weight operand kept by a layer": round(lin["bf16_ms_per_step"], 4), "fused_bf16": round(lin["bf16c_ms_per_step"], 4),
+            "separate": round(lin["separate_ms"], 4),
             "vendor dense bf16 GEMM alone": round(lin["dense_ms"], 4)},
         "same_shape_TFLOPs": {
             "fused (value)": tf(lin["ms_per_step"]), "fused, weight operand kept by a layer": tf(lin["prepared_ms"]),
-            "fused_bf16": tf(lin["bf16_ms_per_step"]), "separate": tf(lin["separate_ms"]), "vendor dense bf16 GEMM alone": tf(lin["dense_ms"])},
+            "fused_bf16, weight operand kept by a layer": tf(lin["bf16_ms_per_step"]), "fused_bf16": tf(lin["bf16c_ms_per_step"]),
+            "separate": tf(lin["separate_ms"]), "vendor dense bf16 GEMM alone": tf(lin["dense_ms"])},
         "note": "fused_bf16 = QDQ of x to bf16 + GEMM composing W to bf16 in registers (bf16 MFMA); separate = extract x + compose x + "
                 "compose W to bf16 in HBM + library GEMM; prewarm = uncounted steps until two groups of five agree within 1 %",
     }

@@ -296,6 +296,20 @@ int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, 
                               const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
                               int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
 
+/*
+ * y[M,N] = A[M,K] * W[N,K]^T (+ bias) with a DENSE bfloat16 A (used as is, like a_dense of mase_hip_mxfp_gemm) and W in
+ * the prepared form above (mase_hip_scaled_operand_from_mxfp with rows = N), on the bf16 matrix instruction: the
+ * 512 x 128 tile kernel of mase_hip_mxfp_gemm composing W to bfloat16 in registers, with what the prepared form saves it
+ * (one convert per pair of codes, because no byte holds the code the convert reads as NaN; the scales of a 128-k step
+ * of 128 rows as 512 contiguous bytes).  For layers that keep the prepared weight anyway and whose activations are not
+ * quantised (layer types XWq*) or are quantised to a format the block-scaled GEMM does not take.
+ * M >= 512, N % 128 == 0, K % 128 == 0, else -2 (use mase_hip_mxfp_gemm with the components).
+ * Replaces the body of mxfp_linear_XWq with backend="fused"  src/mase_triton/mxfp/functional/linear.py:10-33.
+ */
+int mase_hip_mxfp_gemm_prepared_w(const void* a_dense, int a_dtype, const uint8_t* w_codes,
+                                  const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
+                                  int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

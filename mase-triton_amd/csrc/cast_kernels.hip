@@ -457,20 +457,6 @@ __device__ inline uint32_t embed_e4m3_x4(uint32_t w, const F& f) {
     return embed_e4m3(w & 0xFFu, f) | (embed_e4m3((w >> 8) & 0xFFu, f) << 8) | (embed_e4m3((w >> 16) & 0xFFu, f) << 16) |
            (embed_e4m3(w >> 24, f) << 24);
 }
-// where the scale byte of block `b0 + i` goes: b0 = (row0, kb0) is uniform, i small; kblocks = K / 32
-struct ScaledGeom {
-    uint32_t kblocks, rows_pad;
-    float inv_kblocks;
-};
-__device__ inline size_t scaled_scale_offset(uint32_t row0, uint32_t kb0, uint32_t i, const ScaledGeom& g) {
-    const uint32_t x = kb0 + i;   // below 2^23: exact in fp32
-    uint32_t q = (uint32_t)((float)x * g.inv_kblocks);
-    int32_t r = (int32_t)(x - q * g.kblocks);
-    if (r < 0) { r += (int32_t)g.kblocks; --q; }
-    else if (r >= (int32_t)g.kblocks) { r -= (int32_t)g.kblocks; ++q; }
-    return ((size_t)((uint32_t)r >> 2) * g.rows_pad + row0 + q) * 4 + ((uint32_t)r & 3u);
-}
-
 // The arithmetic of one 128-bit step of the bf16 kernels below: 8 elements of a lane whose three quad neighbours hold the
 // rest of the block.  QDQ false: o[j] = two codes in the low bytes of the halves; true: two quantised bf16 values.
 // Every lane of a quad must call it (DPP).
@@ -980,17 +966,19 @@ __global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_lines_kernel(const
 }
 
 // MXFP components (reference layout: one code byte per element, scales [rows, K / 32]) -> operand of the block-scaled
-// GEMM.  A lane owns 16 codes, two adjacent lanes a block.
+// GEMM.  A workgroup owns 32 rows x 128 k (one line of the transposed scale array): a lane 16 codes, two lanes a block,
+// eight lanes the 128 bytes of a row.  The four scale bytes of a row are one dword on either side.
 template <class F>
-__global__ __launch_bounds__(kThreads) void scaled_operand_kernel(const uint8_t* __restrict__ scales, const uint4* __restrict__ elements,
-                                                                   uint4* __restrict__ out_codes, uint8_t* __restrict__ out_scales,
-                                                                   int64_t n_chunks, F f, ScaledGeom sg) {
-    const uint32_t b0 = blockIdx.x * (uint32_t)(kThreads / 2);
-    const uint32_t row0 = b0 / sg.kblocks, kb0 = b0 - row0 * sg.kblocks;
-    const int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    const bool live = c < n_chunks;
-    uint4 w = live ? ld128(elements + c) : make_uint4(0, 0, 0, 0);
-    uint32_t scale = live ? (uint32_t)scales[c >> 1] : 0u;
+__global__ __launch_bounds__(kThreads) void scaled_operand_kernel(const uint8_t* __restrict__ scales, const uint8_t* __restrict__ elements,
+                                                                   uint8_t* __restrict__ out_codes, uint32_t* __restrict__ out_scales,
+                                                                   int rows, int K, int nmac, uint32_t rows_pad, F f) {
+    const uint32_t ms = blockIdx.x % (uint32_t)nmac, row = (blockIdx.x / (uint32_t)nmac) * 32u + (threadIdx.x >> 3);
+    const int piece = threadIdx.x & 7;                  // 16 codes of the row's 128
+    const bool live = row < (uint32_t)rows;
+    const size_t off = (size_t)row * K + ms * 128u + (uint32_t)piece * 16u;
+    uint4 w = live ? ld128(elements + off) : make_uint4(0, 0, 0, 0);
+    const uint32_t sc4 = live ? *reinterpret_cast<const uint32_t*>(scales + ((size_t)row * (K / 32) + ms * 4u)) : 0u;
+    uint32_t scale = (sc4 >> (8 * (piece >> 1))) & 0xFFu;
     if constexpr (F{}.E() == 4 && F{}.M() == 3) {
         uint32_t top = e4m3_top_bits(w.x) | e4m3_top_bits(w.y) | e4m3_top_bits(w.z) | e4m3_top_bits(w.w);
         top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xF, 0xF, true);  // lane ^ 1
@@ -1001,9 +989,14 @@ __global__ __launch_bounds__(kThreads) void scaled_operand_kernel(const uint8_t*
     } else {
         w = make_uint4(embed_e4m3_x4(w.x, f), embed_e4m3_x4(w.y, f), embed_e4m3_x4(w.z, f), embed_e4m3_x4(w.w, f));
     }
+    // the row's four scale bytes (lanes 0, 2, 4, 6 of its 8) into its first lane: row_shl 2, 4, 6
+    uint32_t dw = scale;
+    dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x102, 0xF, 0xF, true) << 8;
+    dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x104, 0xF, 0xF, true) << 16;
+    dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x106, 0xF, 0xF, true) << 24;
     if (live) {
-        st128(out_codes + c, w);
-        if ((c & 1) == 0) out_scales[scaled_scale_offset(row0, kb0, threadIdx.x >> 1, sg)] = (uint8_t)scale;
+        st128(out_codes + off, w);
+        if (piece == 0) out_scales[(size_t)ms * rows_pad + row] = dw;
     }
 }
 
@@ -1336,32 +1329,32 @@ int mase_hip_qdq_mxfp_strided(const void* x, int x_dtype, void* out, int out_dty
 // ---- operands of the block-scaled GEMM (mase_hip_mxfp_gemm_scaled)
 int64_t mase_hip_scaled_padded_rows(int64_t rows) { return rows <= 0 ? 0 : (rows + 255) / 256 * 256; }
 
-static int scaled_operand_args(int64_t rows, int64_t K, int exp_bits, int frac_bits, ScaledGeom& sg) {
+static int scaled_operand_args(int64_t rows, int64_t K, int exp_bits, int frac_bits, uint32_t& rows_pad) {
     if (rows < 1 || K < 1) return fail(ERR_INVALID, "rows and K must be positive");
     if (K % 128 != 0) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM needs K to be a multiple of 128");
     if (K >= ((int64_t)1 << 27) || rows * (K / 32) >= ((int64_t)1 << 31)) return fail(ERR_UNSUPPORTED, "operand too large for the block-scaled GEMM");
     const bool ok = (exp_bits == 4 && frac_bits == 3) || (exp_bits == 2 && frac_bits == 3) || (exp_bits == 3 && frac_bits == 2) ||
                     (exp_bits == 2 && frac_bits == 1);
     if (!ok) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM takes element formats (4,3) (2,3) (3,2) (2,1)");
-    sg.kblocks = (uint32_t)(K / 32);
-    sg.rows_pad = (uint32_t)mase_hip_scaled_padded_rows(rows);
-    sg.inv_kblocks = 1.0f / (float)sg.kblocks;
+    rows_pad = (uint32_t)mase_hip_scaled_padded_rows(rows);
     return OK;
 }
 
 int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elements, int exp_bits, int frac_bits, int64_t rows, int64_t K,
                                       uint8_t* out_codes, uint32_t* out_scales, void* stream) {
-    ScaledGeom sg;
-    if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, sg)) return rc;
+    uint32_t rows_pad;
+    if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, rows_pad)) return rc;
     if (!scales || !elements || !out_codes || !out_scales) return fail(ERR_INVALID, "null pointer");
-    if (!aligned(elements, 16) || !aligned(out_codes, 16) || !aligned(out_scales, 4)) return fail(ERR_INVALID, "elements and out_codes must be 16-byte aligned, out_scales 4-byte aligned");
+    if (!aligned(elements, 16) || !aligned(out_codes, 16) || !aligned(out_scales, 4) || !aligned(scales, 4))
+        return fail(ERR_INVALID, "elements and out_codes must be 16-byte aligned, scales and out_scales 4-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int64_t n_chunks = rows * K / 16;
     return dispatch_fmt(exp_bits, frac_bits, 1, RN, [&](auto f) {
         if constexpr (decltype(f)::kStatic && decltype(f){}.E() != 5) {
-            hipLaunchKernelGGL((scaled_operand_kernel<decltype(f)>), dim3(grid_for(n_chunks, kThreads)), dim3(kThreads), 0, s, scales,
-                               reinterpret_cast<const uint4*>(elements), reinterpret_cast<uint4*>(out_codes), reinterpret_cast<uint8_t*>(out_scales),
-                               n_chunks, f, sg);
+            const int nmac = (int)(K / 128);
+            const int64_t blocks = (rows + 31) / 32 * nmac;
+            if (blocks > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "operand too large for one launch");
+            hipLaunchKernelGGL((scaled_operand_kernel<decltype(f)>), dim3((unsigned)blocks), dim3(kThreads), 0, s, scales, elements, out_codes,
+                               out_scales, (int)rows, (int)K, nmac, rows_pad, f);
             return check_launch("scaled_operand_from_mxfp");
         }
         return fail(ERR_UNSUPPORTED, "element format not supported by the block-scaled GEMM");
@@ -1370,8 +1363,8 @@ int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elem
 
 int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
                                        uint32_t* out_scales, void* stream) {
-    ScaledGeom sg;
-    if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, sg)) return rc;
+    uint32_t rows_pad;
+    if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, rows_pad)) return rc;
     if (x_dtype != BF16) return fail(ERR_UNSUPPORTED, "a dense operand of the block-scaled GEMM must be bfloat16");
     if (!x || !out_codes || !out_scales) return fail(ERR_INVALID, "null pointer");
     if (!aligned(x, 16) || !aligned(out_codes, 8) || !aligned(out_scales, 4)) return fail(ERR_INVALID, "x must be 16-byte aligned, out_codes 8-byte, out_scales 4-byte");
@@ -1382,7 +1375,7 @@ int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits,
             const int64_t blocks = (rows + 31) / 32 * nmac;
             if (blocks > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "operand too large for one launch");
             hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f)>), dim3((unsigned)blocks), dim3(kThreads), 0, s, static_cast<const uint16_t*>(x),
-                               out_codes, out_scales, (int)rows, (int)K, nmac, sg.rows_pad, f);
+                               out_codes, out_scales, (int)rows, (int)K, nmac, rows_pad, f);
             return check_launch("scaled_operand_from_dense");
         }
         return fail(ERR_UNSUPPORTED, "element format not supported by the block-scaled GEMM");

@@ -109,9 +109,11 @@ extern "C" int mase_hip_mxfp_gemm_static_ws(const void* a_dense, int a_dtype, co
         return fail(ERR_UNSUPPORTED, "this shape splits K into " + std::to_string(need) + " bytes of partial sums, more than the " +
                                          std::to_string((long long)MASE_HIP_STATIC_WORKSPACE_BYTES) +
                                          " bytes of the static workspace: pass a workspace to mase_hip_mxfp_gemm_ws, or call mase_hip_mxfp_gemm (no split, no workspace)");
+    // looked up on every call (one atomic load after the first): the first call on a device, whatever its shape, is the one
+    // that may load the code object, so a caller who warms up outside a capture has done it
     void* ws = nullptr;
-    if (need > 0)
-        if (int rc = static_workspace(&ws)) return rc;
+    if (int rc = static_workspace(&ws)) return rc;
+    if (need == 0) ws = nullptr;
     // every split writes all of its [M, N] array before the second kernel reads it: nothing has to start at zero
     return gemm_entry(a_dense, a_dtype, a_scales, a_elements, a_exp_bits, a_frac_bits, w_scales, w_elements, w_exp_bits, w_frac_bits,
                       bias, bias_dtype, y, out_dtype, M, N, K, block_size, ws, ws ? (int64_t)MASE_HIP_STATIC_WORKSPACE_BYTES : 0, stream);

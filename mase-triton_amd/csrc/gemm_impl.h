@@ -516,7 +516,7 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
             // one persistent workgroup per CU (a multiple of the 8 XCDs), never more than tiles
             const unsigned grid = (unsigned)(tall_tiles < cus ? ((tall_tiles + 7) / 8) * 8 : (cus / 8) * 8);
             hipLaunchKernelGGL(kern, dim3(grid, 1u, (unsigned)batches), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense),
-                               w_scales, w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN, 1, (int64_t)0, gb);
+                               w_scales, w_elements, bias, bias_dtype, y, M, N, K, tall_tiles_m, N / UN, 1, (int64_t)0, gb, 0);
             return check_launch("mxfp_gemm");
         }
     }
@@ -543,6 +543,30 @@ int launch_gemm(const void* a_dense, const uint8_t* a_scales, const uint8_t* a_e
     return check_launch("mxfp_gemm");
 }
 
+
+// Dense bf16 A against a weight in prepared form (the operand of the block-scaled GEMM: E4M3 bytes [rows_pad, K] without the
+// NaN code, scales dword [K / 128][rows_pad]) on the 512 x 128 bf16 kernel: the compose is one convert per pair of
+// codes and the scales of a macro step come as whole lines.
+inline bool tall_prepared_shape_ok(int64_t M, int64_t N, int64_t K) {
+    return M >= UM && N % UN == 0 && K % UMAC == 0 && K <= (1 << 23) && N <= (1 << 26) && ((M + UM - 1) / UM) * (N / UN) < (1 << 30);
+}
+template <int DT_OUT>
+int launch_gemm_tall_prepared(const void* a_dense, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
+                              int M, int N, int K, hipStream_t s) {
+    if (!tall_prepared_shape_ok(M, N, K)) return fail(ERR_UNSUPPORTED, "the prepared-weight bf16 GEMM takes M >= 512, N % 128 == 0, K % 128 == 0");
+    const int cus = device_cu_count();
+    if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
+    const int tiles_m = (M + UM - 1) / UM;
+    const int64_t tiles = (int64_t)tiles_m * (N / UN);
+    auto kern = mxfp_gemm_tall_kernel<PreparedE4M3, DT_OUT, false>;
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), U_LDS_BYTES, lds_allowed)) return rc;
+    const unsigned grid = (unsigned)(tiles < cus ? ((tiles + 7) / 8) * 8 : (cus / 8) * 8);
+    const int rows_pad = (N + SN - 1) / SN * SN;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), U_LDS_BYTES, s, static_cast<const uint16_t*>(a_dense), reinterpret_cast<const uint8_t*>(w_scales),
+                       w_codes, bias, bias_dtype, y, M, N, K, tiles_m, N / UN, 1, (int64_t)0, GemmBatch{0, 0, 0, 0}, rows_pad);
+    return check_launch("mxfp_gemm_prepared_w");
+}
 
 // One entry per weight format; each lives in its own translation unit (gemm_w_*.hip) so that the
 // formats compile in parallel.  a_exp_bits == 0 selects the dense-A kernel.

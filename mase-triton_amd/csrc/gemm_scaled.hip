@@ -20,3 +20,19 @@ extern "C" int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t*
         return launch_gemm_scaled<decltype(dout)::value>(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, (int)M, (int)N, (int)K, s);
     });
 }
+
+extern "C" int mase_hip_mxfp_gemm_prepared_w(const void* a_dense, int a_dtype, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
+                                             int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+    if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
+    if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(ERR_INVALID, "M, N, K must fit in 31 bits");
+    if (!a_dense || !w_codes || !w_scales || !y) return fail(ERR_INVALID, "null pointer");
+    if (a_dtype != BF16) return fail(ERR_UNSUPPORTED, "a dense A operand must be bfloat16");
+    if (int rc = check_dtype(out_dtype, "output")) return rc;
+    if (bias) if (int rc = check_dtype(bias_dtype, "bias")) return rc;
+    if (!aligned(a_dense, 16) || !aligned(w_codes, 16) || !aligned(w_scales, 4) || !aligned(y, 16))
+        return fail(ERR_INVALID, "A, codes and y must be 16-byte aligned, scales 4-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dispatch_dtype(out_dtype, [&](auto dout) {
+        return launch_gemm_tall_prepared<decltype(dout)::value>(a_dense, w_codes, w_scales, bias, bias_dtype, y, (int)M, (int)N, (int)K, s);
+    });
+}

@@ -119,7 +119,7 @@ int launch_gemm_split_k(const void* a_dense, const uint8_t* w_scales, const uint
         const int walks = tiles_m * (N / UN) * plan.splits;          // at most one per CU (the plan splits only then)
         hipLaunchKernelGGL(kern, dim3((unsigned)((walks + 7) / 8 * 8)), dim3(kGemmThreads), U_LDS_BYTES, s,
                            static_cast<const uint16_t*>(a_dense), w_scales, w_elements, static_cast<const void*>(nullptr), 0, workspace,
-                           M, N, K, tiles_m, N / UN, plan.splits, mn * 4, GemmBatch{0, 0, 0, 0});
+                           M, N, K, tiles_m, N / UN, plan.splits, mn * 4, GemmBatch{0, 0, 0, 0}, 0);
     }
     if (int rc = check_launch("mxfp_gemm")) return rc;
     hipLaunchKernelGGL(split_k_reduce_kernel<DT_OUT>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s,

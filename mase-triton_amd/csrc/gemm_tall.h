@@ -139,7 +139,11 @@ template <class FW, int DT_OUT, bool SC4>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_tall_kernel(
     const uint16_t* __restrict__ a_dense0, const uint8_t* __restrict__ w_scales0, const uint8_t* __restrict__ w_elements0,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ y0, int M, int N, int K, int tiles_m, int tiles_n, int splits, int64_t y_split_bytes,
-    GemmBatch gb) {
+    GemmBatch gb, int w_rows_pad) {
+    // WT: the weight is a prepared operand (see scaled_operand_kernel): E4M3 bytes without the NaN code and its scales
+    // transposed, dword [k / 128][row of w_rows_pad]: the 128 rows' scales of a macro step are 512 contiguous bytes
+    constexpr bool WT = has_no_top_code<FW>::value;
+    static_assert(!(WT && SC4), "transposed scales come one dword per row and macro step");
     // batched launches: workgroups of grid plane z work on product z (offsets are zero for a single product)
     const uint16_t* __restrict__ const a_dense = a_dense0 + (int64_t)blockIdx.z * gb.a;
     const uint8_t* __restrict__ const w_scales = w_scales0 + (int64_t)blockIdx.z * gb.ws;
@@ -175,7 +179,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     // W staging: thread t owns codes [16 h, 16 h + 16) of row t >> 1 in every K step, h = t & 1
     const int w_row = tid >> 1, w_half = tid & 1;
     const uint32_t w_voff = (uint32_t)w_row * (uint32_t)K + (uint32_t)w_half * 16u;
-    const uint32_t ws_voff = (uint32_t)w_row * (uint32_t)kblocks;
+    const uint32_t ws_voff = WT ? (uint32_t)w_row * 4u : (uint32_t)w_row * (uint32_t)kblocks;
+    const size_t ws_mac_stride = WT ? (size_t)w_rows_pad * 4u : (size_t)(UMAC / 32);   // bytes between a row's scales of consecutive macro steps
     // its 16 bf16 of K step p (0 / 1 within the 64-k stage) are chunks 4p + 2h and 4p + 2h + 1 of the row
     uint32_t w_lds_off[2][2];
 #pragma unroll
@@ -205,7 +210,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         const size_t k0 = (size_t)z * k_len;
         t.a = reinterpret_cast<const uint8_t*>(a_dense) + ((size_t)(t.m0 + wave * 128) * K + k0) * 2;
         t.w = w_elements + (size_t)t.n0 * K + k0;
-        t.ws = w_scales + (size_t)t.n0 * kblocks + k0 / 32;
+        t.ws = WT ? w_scales + (size_t)t.n0 * 4u + (k0 / UMAC) * ws_mac_stride : w_scales + (size_t)t.n0 * kblocks + k0 / 32;
         t.y_off = (size_t)z * (size_t)y_split_bytes;
         return t;
     };
@@ -447,7 +452,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
             ws_voff_now = sc_fresh ? ws_voff : 0u;
             ws_nxt = (wrap ? next.ws : cur.ws) + (mn >> 2) * 16;
         } else {
-            ws_nxt = (wrap ? next.ws : cur.ws) + mn * (UMAC / 32);
+            ws_nxt = (wrap ? next.ws : cur.ws) + mn * ws_mac_stride;
         }
         step(IntC<0>{}, first_c);
         step(IntC<1>{}, IntC<0>{});

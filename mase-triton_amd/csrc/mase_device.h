@@ -8,6 +8,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace mase {
 
 enum DType : int { F32 = 0, F16 = 1, BF16 = 2 };
@@ -25,6 +27,14 @@ struct SFmt {
     __host__ __device__ constexpr bool finite() const { return FIN_; }
     __host__ __device__ constexpr int rmode() const { return RM_; }
 };
+
+// E4M3 bytes as the operand-prepare kernels of the block-scaled GEMM leave them: every element format embedded into
+// E4M3 with the same value, and no byte with the magnitude 0x7F (the one E4M3 code the hardware converts read as NaN)
+struct PreparedE4M3 : SFmt<4, 3> {
+    static constexpr bool kNoTopCode = true;
+};
+template <class F, class = void> struct has_no_top_code { static constexpr bool value = false; };
+template <class F> struct has_no_top_code<F, std::enable_if_t<F::kNoTopCode>> { static constexpr bool value = true; };
 
 struct DFmt {
     static constexpr bool kStatic = false;

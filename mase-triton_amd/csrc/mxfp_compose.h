@@ -44,7 +44,8 @@ struct Composer {
     static constexpr int E = F{}.E(), M = F{}.M();
     static constexpr int BIAS = (1 << (E - 1)) - 1;
     static constexpr bool HW = E <= 4;                       // hardware convert route
-    static constexpr bool TOP_IS_NAN = E == 4 && M == 3;     // magnitude 0x7F: NaN to the hardware, 480 to the reference
+    // magnitude 0x7F: NaN to the hardware, 480 to the reference (prepared operands never hold it)
+    static constexpr bool TOP_IS_NAN = E == 4 && M == 3 && !has_no_top_code<F>::value;
     static constexpr int SCALE_UP = 7 - BIAS;
     // first scale byte that needs the slow route (none for E5M2, whose only route handles every scale)
     static constexpr uint32_t SLOW_FROM = !HW ? 256u : TOP_IS_NAN ? 247u : (uint32_t)(255 - SCALE_UP);

@@ -150,6 +150,10 @@ def mxfp_linear(
         if quantised_x:
             # MXFP values are exact in bf16 whatever x.dtype is
             a = kernels.quantize_dequantize(a.flatten(), x_meta, torch.bfloat16).view(-1, in_features)
+        if (w_operand is not None and a.dtype == torch.bfloat16 and w_operand.rows == out_features and w_operand.K == in_features
+                and kernels.prepared_w_shape_supported(a.shape[0], out_features, in_features)):
+            # a layer's kept weight operand: the large-tile bf16 kernel reads it with a cheaper compose and scale fetch
+            return kernels.mxfp_gemm_prepared_w(a, w_operand, bias, x.dtype).view(*lead, out_features)
         y = kernels.mxfp_gemm(a, None, None, None, w_scales, w_elements, w_tensor_meta.meta, bias,
                               a.shape[0], out_features, in_features, x.dtype)
         return y.view(*lead, out_features)

@@ -303,3 +303,32 @@ def mxfp_gemm_scaled(a: ScaledOperand, w: ScaledOperand, bias: Tensor | None, ou
             a.codes.data_ptr(), a.scales.data_ptr(), w.codes.data_ptr(), w.scales.data_ptr(), b_ptr, b_dt, y.data_ptr(),
             _lib.dtype_code(output_dtype), M, N, K, _lib.stream_ptr(dev)))
     return y
+
+
+def prepared_w_shape_supported(M: int, N: int, K: int) -> bool:
+    return M >= 512 and N % 128 == 0 and K % 128 == 0 and K <= (1 << 23)
+
+
+def mxfp_gemm_prepared_w(a: Tensor, w: ScaledOperand, bias: Tensor | None, output_dtype: torch.dtype, out: Tensor | None = None) -> Tensor:
+    """y[M,N] = a @ W^T (+ bias): dense bfloat16 ``a`` [M, K] (used as is) against a weight in the block-scaled GEMM's form, on
+    the bf16 matrix instruction (W composed to bf16 in registers)."""
+    assert a.ndim == 2 and a.dtype == torch.bfloat16 and a.shape[1] == w.K
+    _lib.require_gpu(a, "activations")
+    a = _lib.dense(a)
+    M, N, K = a.shape[0], w.rows, w.K
+    dev = w.codes.device
+    b_ptr, b_dt = None, 0
+    if bias is not None:
+        bias = _lib.dense(bias)
+        assert bias.numel() == N
+        b_ptr, b_dt = bias.data_ptr(), _lib.dtype_code(bias.dtype)
+    if out is None:
+        y = torch.empty((M, N), dtype=output_dtype, device=dev)
+    else:
+        assert out.is_contiguous() and out.dtype == output_dtype and out.numel() == M * N and out.device == dev
+        y = out
+    with _lib.on_device(dev):
+        _lib.check(_lib.load().mase_hip_mxfp_gemm_prepared_w(
+            a.data_ptr(), _lib.dtype_code(a.dtype), w.codes.data_ptr(), w.scales.data_ptr(), b_ptr, b_dt, y.data_ptr(),
+            _lib.dtype_code(output_dtype), M, N, K, _lib.stream_ptr(dev)))
+    return y

@@ -115,17 +115,24 @@ class MXFPLinearPTQ(nn.Module):
         self._scaled_w = self._scaled_w_key = None
 
     def _weight_operand(self, input: Tensor):
-        """The weight in the block-scaled GEMM's form when this call can take that route, else None."""
+        """The weight in the block-scaled GEMM's form when this call has a kernel that reads it (the block-scaled GEMM for
+        quantised bfloat16 activations, the large-tile bf16 kernel from 512 rows on), else None."""
+        from . import kernels
         from .functional import linear as L
 
-        if self.backend not in ("fused", "fused_scaled") or not self.layer_type.startswith("XqWq"):
+        if self.backend == "separate" or "Wq" not in self.layer_type or input.device.type != "cuda":
             return None
         rows = input.numel() // input.shape[-1] if input.numel() else 0
-        if self.backend == "fused" and rows < L.SCALED_FROM_ROWS:
-            return None
         bias = self.bias if not self.layer_type.endswith("Bq") else None
-        if not L._scaled_eligible(input, self.x_mxfp_meta, self.w_tensor_meta, bias):
-            return None
+        scaled = (self.backend != "fused_bf16" and self.layer_type.startswith("XqWq") and (self.backend == "fused_scaled" or rows >= L.SCALED_FROM_ROWS)
+                  and L._scaled_eligible(input, self.x_mxfp_meta, self.w_tensor_meta, bias))
+        if not scaled:
+            tm = self.w_tensor_meta
+            bf16 = (self.backend != "fused_scaled" and len(tm.shape) == 2 and kernels.scaled_format_supported(tm.meta) and tm.block_dim % 2 == 1
+                    and input.dtype == torch.bfloat16 and getattr(torch, tm.dtype) == input.dtype
+                    and kernels.prepared_w_shape_supported(rows, tm.shape[0], tm.shape[1]))
+            if not bf16:
+                return None
         key = (self.w_elements.data_ptr(), self.w_elements._version, self.w_scales.data_ptr(), self.w_scales._version)
         if self._scaled_w is None or self._scaled_w_key != key:
             self._scaled_w = L.scaled_weight_operand(self.w_scales, self.w_elements, self.w_tensor_meta)

@@ -252,6 +252,63 @@ def test_special_blocks_poison_the_same_outputs(mh):
     assert rel_fro(y[ok], y_ref[ok]) <= F32_TOL
 
 
+# ---------------------------------------------------------------- the prepared weight on the bf16 kernel
+@pytest.mark.parametrize("MNK", [(512, 256, 512), (1100, 384, 1024), (640, 128, 128)])
+@pytest.mark.parametrize("w_tag", SCALED_TAGS)
+def test_prepared_weight_on_the_bf16_kernel(mh, MNK, w_tag):
+    """Dense bf16 A against the weight in prepared form (mase_hip_mxfp_gemm_prepared_w): against the float64 checker, and
+    against mase_hip_mxfp_gemm on the components (which may pick another tile shape, i.e. another order of additions)."""
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(M + N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    _, _, x_dq = quantised(x, "MXFP8_E4M3_fn")
+    w_sc, w_el, w_dq = quantised(w, w_tag)
+    meta = getattr(mh.meta, w_tag)
+    a = x_dq.to(torch.bfloat16).to(DEV)
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), meta, N, K)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    y_ref = oracle.matmul_nt(x_dq, w_dq) + b.float()
+    for odt, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-3)):
+        y = mh.mxk.mxfp_gemm_prepared_w(a, wop, b.to(DEV), odt)
+        assert y.shape == (M, N) and y.dtype == odt
+        assert rel_fro(y, y_ref.to(odt)) <= tol
+        y_comp = mh.mxk.mxfp_gemm(a, None, None, None, w_sc.to(DEV), w_el.to(DEV), meta, b.to(DEV), M, N, K, odt, split_k=False)
+        assert rel_fro(y, y_comp) <= 2 * tol
+
+
+def test_prepared_weight_special_blocks_and_refusals(mh):
+    M, N, K = 512, 128, 256
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    w[5, 40] = float("inf")
+    w[77, 255] = float("nan")
+    w_sc, w_el, w_dq = quantised(w, "OCP_MXFP6_E3M2")
+    meta = mh.meta.OCP_MXFP6_E3M2
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), meta, N, K)
+    y = mh.mxk.mxfp_gemm_prepared_w(x.to(DEV), wop, None, torch.float32).cpu()
+    y_ref = x.double() @ w_dq.double().t()
+    assert torch.equal(y.isnan(), y_ref.isnan()) and y.isnan().sum() == 2 * M
+    with pytest.raises(NotImplementedError):
+        mh.mxk.mxfp_gemm_prepared_w(x[:256].to(DEV), wop, None, torch.float32)   # fewer than 512 rows
+
+
+def test_weight_only_layer_keeps_the_prepared_weight(mh):
+    """XWqB (dense bfloat16 activations): from 512 rows on the layer runs the bf16 kernel on its kept prepared weight."""
+    lin = torch.nn.Linear(512, 256, bias=True, dtype=torch.bfloat16, device=DEV)
+    wfmt = mh.meta.OCP_MXFP4_E2M1
+    fused = mh.MXFPLinearPTQ.from_linear(lin, None, wfmt, None, "XWqB", "fused")
+    sep = mh.MXFPLinearPTQ.from_linear(lin, None, wfmt, None, "XWqB", "separate")
+    g = torch.Generator().manual_seed(3)
+    small = torch.randn(64, 512, generator=g).to(torch.bfloat16).to(DEV)
+    big = torch.randn(2, 300, 512, generator=g).to(torch.bfloat16).to(DEV)
+    assert rel_fro(fused(small), sep(small)) <= 1e-3 and fused._scaled_w is None
+    y = fused(big)
+    assert fused._scaled_w is not None and y.shape == (2, 300, 256)
+    assert rel_fro(y, sep(big)) <= 1e-3
+
+
 def test_unsupported_shapes_are_refused(mh):
     meta = mh.meta.MXFP8_E4M3_fn
     x = torch.randn(64, 384).to(torch.bfloat16).to(DEV)

@@ -19,7 +19,10 @@ def _operands(mxk, meta, M, N, K, seed):
     return a, w_sc, w_el, bias
 
 
-def test_static_workspace_matches_caller_workspace():
+def both(M, N, K, seed, out_code, out_dtype):
+    """The product through mase_hip_mxfp_gemm_static_ws and through mase_hip_mxfp_gemm_ws with a workspace from torch; also the
+    free device memory before and after the former.  The split plan depends on the device's compute-unit count: a shape
+    that is not split there, or asks for more than the static array holds, skips the test."""
     import mase_hip.mxfp.kernels as mxk
     from mase_hip import _lib
     from mase_hip.mxfp.meta import MXFP8_E4M3_fn as meta
@@ -27,25 +30,33 @@ def test_static_workspace_matches_caller_workspace():
     lib = _lib.load()
     stream = _lib.stream_ptr(torch.device(DEV))
     limit = 32 * 1024 * 1024
+    a, w_sc, w_el, bias = _operands(mxk, meta, M, N, K, seed)
+    need = lib.mase_hip_mxfp_gemm_workspace_bytes(1, M, N, K)
+    if not 0 < need <= limit:
+        pytest.skip(f"({M}, {N}, {K}) asks for {need} bytes of partial sums on this device: not a split shape that fits the static workspace")
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    y_ref = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+    rc = lib.mase_hip_mxfp_gemm_ws(a.data_ptr(), 2, None, None, 0, 0, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, bias.data_ptr(), 2,
+                                   y_ref.data_ptr(), out_code, M, N, K, 32, ws.data_ptr(), need, stream)
+    assert rc == 0, lib.mase_hip_last_error()
+    y = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    rc = lib.mase_hip_mxfp_gemm_static_ws(a.data_ptr(), 2, None, None, 0, 0, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, bias.data_ptr(), 2,
+                                          y.data_ptr(), out_code, M, N, K, 32, stream)
+    assert rc == 0, lib.mase_hip_last_error()
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    # the split really ran: the unsplit kernels add in another order
+    y_unsplit = torch.empty_like(y)
+    assert lib.mase_hip_mxfp_gemm(a.data_ptr(), 2, None, None, 0, 0, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, bias.data_ptr(), 2,
+                                  y_unsplit.data_ptr(), out_code, M, N, K, 32, stream) == 0
+    torch.cuda.synchronize()
+    assert not torch.equal(y.view(torch.uint8), y_unsplit.view(torch.uint8)), "the split path left no trace in the result"
+    return y, y_ref, free_before, free_after
 
-    def both(M, N, K, seed, out_code, out_dtype):
-        a, w_sc, w_el, bias = _operands(mxk, meta, M, N, K, seed)
-        need = lib.mase_hip_mxfp_gemm_workspace_bytes(1, M, N, K)
-        assert 0 < need <= limit, f"({M}, {N}, {K}) should be a split shape that fits the static workspace, asks for {need}"
-        ws = torch.empty(need, dtype=torch.uint8, device=DEV)
-        y_ref = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-        rc = lib.mase_hip_mxfp_gemm_ws(a.data_ptr(), 2, None, None, 0, 0, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, bias.data_ptr(), 2,
-                                       y_ref.data_ptr(), out_code, M, N, K, 32, ws.data_ptr(), need, stream)
-        assert rc == 0, lib.mase_hip_last_error()
-        y = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-        torch.cuda.synchronize()
-        free_before = torch.cuda.mem_get_info()[0]
-        rc = lib.mase_hip_mxfp_gemm_static_ws(a.data_ptr(), 2, None, None, 0, 0, w_sc.data_ptr(), w_el.data_ptr(), 4, 3, bias.data_ptr(), 2,
-                                              y.data_ptr(), out_code, M, N, K, 32, stream)
-        assert rc == 0, lib.mase_hip_last_error()
-        torch.cuda.synchronize()
-        return y, y_ref, free_before, torch.cuda.mem_get_info()[0]
 
+def test_static_workspace_matches_caller_workspace():
     # the first call on the device looks up the array (and may load the code object): not part of the memory comparison
     y, y_ref, _, _ = both(256, 2048, 14336, 1, 2, torch.bfloat16)
     assert torch.isfinite(y.float()).all() and torch.equal(y.view(torch.int16), y_ref.view(torch.int16))
@@ -104,3 +115,6 @@ def test_static_workspace_unsplit_shape_runs_without_the_array():
                                             M, N, K, 32, stream) == 0
     torch.cuda.synchronize()
     assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
+    # an unsplit call first and a split call after it (the order of a caller who warms up on a small shape)
+    y, y_ref, _, _ = both(256, 2048, 14336, 5, 2, torch.bfloat16)
+    assert torch.equal(y.view(torch.int16), y_ref.view(torch.int16))
