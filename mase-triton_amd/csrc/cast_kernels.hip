@@ -25,6 +25,9 @@ constexpr int kThreads = 256;
 #ifndef MASE_UNROLL_MXFP
 #define MASE_UNROLL_MXFP 1
 #endif
+#ifndef MASE_UNROLL_EXTRACT
+#define MASE_UNROLL_EXTRACT 2
+#endif
 #ifndef MASE_UNROLL_PACKED
 #define MASE_UNROLL_PACKED 2
 #endif
@@ -457,11 +460,58 @@ __device__ inline uint32_t embed_e4m3_x4(uint32_t w, const F& f) {
     return embed_e4m3(w & 0xFFu, f) | (embed_e4m3((w >> 8) & 0xFFu, f) << 8) | (embed_e4m3((w >> 16) & 0xFFu, f) << 16) |
            (embed_e4m3(w >> 24, f) << 24);
 }
+// ---- code tables of the bf16 kernels
+// With t as above ((ye << 7) | f7: the element's exponent field in the target format above the 7 mantissa bits of its
+// bf16 magnitude), the code magnitude is a function of t alone: 2^(E + 7) entries, built at compile time by the same steps
+// as PackedBf16::magnitude (round half to even on the M-bit mantissa, the reference's OR that loses a carry into an odd
+// exponent field, the one reachable subnormal binade).  A workgroup copies its format's table into LDS and looks every
+// element up there: half the vector instructions of the arithmetic.
+template <int E, int M>
+struct CodeLut {
+    static constexpr int N = 1 << (E + 7);
+    uint8_t code[N];
+    constexpr CodeLut() : code{} {
+        constexpr int SH = 7 - M;
+        for (int t = 0; t < N; ++t) {
+            const int ye = t >> 7, f7 = t & 127;
+            const int q = f7 >> SH, r = f7 & ((1 << SH) - 1), half = 1 << (SH - 1);
+            const int yf = q + ((r > half || (r == half && (q & 1))) ? 1 : 0);   // in [0, 2^M]
+            const int c = ye != 0 ? ((ye << M) | yf) : (yf != 0 ? ((yf | (1 << M)) >> 1) : 0);
+            code[t] = (uint8_t)c;
+        }
+    }
+};
+template <int E, int M>
+__device__ const CodeLut<E, M> kCodeLut{};
+
+// LDS copy of the table (the code-producing modes; the fused quantise-dequantise pass does not use one: BYTES = 16 there);
+// all threads of the workgroup call it, before the first bf16_block_step.
+template <class F, bool QDQ>
+struct LdsLut {
+    static constexpr int E = F{}.E(), M = F{}.M();
+    static constexpr int BYTES = QDQ ? 16 : (1 << (E + 7));
+    __device__ static inline void fill(uint8_t* lds) {
+        if (QDQ) return;
+        for (int i = threadIdx.x * 16; i < BYTES; i += kThreads * 16)
+            *reinterpret_cast<uint4*>(lds + i) = *reinterpret_cast<const uint4*>(kCodeLut<E, M>.code + i);
+        __syncthreads();
+    }
+};
+
+// two table entries, for the t values in the halves of `t2` (issued here, valid after the caller's s_waitcnt; plain loads into
+// two registers: a load into half a register does not keep the other half on this hardware)
+template <bool UNUSED>
+__device__ inline void lut_pair(uint32_t& lo, uint32_t& hi, uint32_t lds_base, uint32_t t2) {
+    const uint32_t a_lo = lds_base + (t2 & 0xFFFFu), a_hi = lds_base + (t2 >> 16);
+    asm volatile("ds_read_u8 %0, %2\n\tds_read_u8 %1, %3" : "=&v"(lo), "=&v"(hi) : "v"(a_lo), "v"(a_hi));
+}
+
 // The arithmetic of one 128-bit step of the bf16 kernels below: 8 elements of a lane whose three quad neighbours hold the
 // rest of the block.  QDQ false: o[j] = two codes in the low bytes of the halves; true: two quantised bf16 values.
-// Every lane of a quad must call it (DPP).
+// `lut`: LDS address of the table (LdsLut<F, QDQ>).  Every lane of a quad must call it (DPP).
 template <class F, bool QDQ>
-__device__ inline void bf16_block_step(const uint4& raw, const F& f, uint32_t (&o)[4], uint32_t& scale) {
+__device__ inline void bf16_block_step(const uint4& raw, const F& f, uint32_t (&o)[4], uint32_t& scale, uint32_t lut) {
+    constexpr int E = F{}.E(), M = F{}.M();
     const uint32_t h[4] = {raw.x, raw.y, raw.z, raw.w};
     // block maximum of |x| bits: packed max over the lane's four registers, then the two halves,
     // then the four lanes of the block (DPP quad permutes)
@@ -478,8 +528,26 @@ __device__ inline void bf16_block_step(const uint4& raw, const F& f, uint32_t (&
     if (__builtin_amdgcn_ballot_w64(hard) == 0) {
         const uint32_t ssb = (uint32_t)((scale_n - fmt_bias(f)) << 7) & 0xFFFFu;
         const uint32_t ssb2 = ssb | (ssb << 16);
+        if constexpr (QDQ) {
+            // (the fused pass stays on the packed arithmetic: a lane has as many stores as loads to hide it under, and a
+            // workgroup would copy a table half the size of its input; measured slower with the table)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o[j] = QDQ ? PackedBf16<F>::qdq(h[j], ssb2) : PackedBf16<F>::codes(h[j], ssb2);
+            for (int j = 0; j < 4; ++j) o[j] = PackedBf16<F>::qdq(h[j], ssb2);
+            return;
+        }
+        uint32_t hl[4], lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // inputs with a zero exponent field are flushed to +0.0 before encoding (code 0, sign included): clear them here
+            hl[j] = h[j] & PackedBf16<F>::live_mask(h[j] & 0x7FFF7FFFu);
+            const uint32_t t2 = as_u32(__builtin_elementwise_sub_sat(as_u16x2(hl[j] & 0x7FFF7FFFu), as_u16x2(ssb2)));
+            lut_pair<false>(lo[j], hi[j], lut, t2);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]), "+v"(hi[0]), "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3]));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            o[j] = lo[j] | (hi[j] << 16) | ((hl[j] >> (15 - (E + M))) & ((1u << (E + M)) * 0x00010001u));
+        }
     } else {
         // exact per-element routine (the block's lanes agree on amax, so they agree on the result)
         const uint32_t amax32 = amax << 16;
@@ -499,6 +567,7 @@ template <class F, int UNROLL, int MODE>
 __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __restrict__ x, uint8_t* __restrict__ scales,
                                                                   uint2* __restrict__ elements, uint4* __restrict__ out,
                                                                   int64_t n_chunks, F f) {
+    __shared__ __attribute__((aligned(16))) uint8_t lut[LdsLut<F, MODE == 1>::BYTES];
     const int64_t chunk0 = (int64_t)blockIdx.x * (UNROLL * kThreads) + threadIdx.x;
     uint4 raw[UNROLL];
 #pragma unroll
@@ -506,11 +575,13 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
         const int64_t c = chunk0 + (int64_t)r * kThreads;
         raw[r] = c < n_chunks ? ld128(x + c) : make_uint4(0, 0, 0, 0);
     }
+    LdsLut<F, MODE == 1>::fill(lut);
+    const uint32_t lut_addr = (uint32_t)(uintptr_t)lut;
 #pragma unroll
     for (int r = 0; r < UNROLL; ++r) {
         const int64_t c = chunk0 + (int64_t)r * kThreads;
         uint32_t o[4], scale;
-        bf16_block_step<F, MODE == 1>(raw[r], f, o, scale);
+        bf16_block_step<F, MODE == 1>(raw[r], f, o, scale, lut_addr);
         if (c < n_chunks) {
             if (MODE == 0) {
                 // o[j] holds two codes in the low bytes of its halves: gather the 8 code bytes
@@ -531,6 +602,7 @@ template <class F>
 __global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes,
                                                                       uint32_t* __restrict__ scales, int rows, int K, int nmac,
                                                                       uint32_t rows_pad, F f) {
+    __shared__ __attribute__((aligned(16))) uint8_t lut[LdsLut<F, false>::BYTES];
     const uint32_t ms = blockIdx.x % (uint32_t)nmac, row_base = (blockIdx.x / (uint32_t)nmac) * 32u;
     const int t = threadIdx.x;
     uint4 raw[2];
@@ -543,10 +615,12 @@ __global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint1
         off[r] = (size_t)row * K + ms * 128u + (uint32_t)(t & 15) * 8u;
         raw[r] = live[r] ? ld128(x + off[r]) : make_uint4(0, 0, 0, 0);
     }
+    LdsLut<F, false>::fill(lut);
+    const uint32_t lut_addr = (uint32_t)(uintptr_t)lut;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
         uint32_t o[4], scale;
-        bf16_block_step<F, false>(raw[r], f, o, scale);
+        bf16_block_step<F, false>(raw[r], f, o, scale, lut_addr);
         uint32_t w0 = __builtin_amdgcn_perm(o[1], o[0], 0x06040200u), w1 = __builtin_amdgcn_perm(o[3], o[2], 0x06040200u);
         if constexpr (F{}.E() == 4 && F{}.M() == 3) {
             uint32_t top = e4m3_top_bits(w0) | e4m3_top_bits(w1);
@@ -1137,7 +1211,7 @@ int mase_hip_extract_mxfp(const void* x, int x_dtype, uint8_t* scales, uint8_t* 
     return dispatch_fmt(exp_bits, frac_bits, is_finite, round_mode, [&](auto f) {
         if constexpr (decltype(f)::kStatic) {
             if (x_dtype == BF16 && B == 32 && vec) {
-                constexpr int U = MASE_UNROLL_PACKED;
+                constexpr int U = MASE_UNROLL_EXTRACT;
                 hipLaunchKernelGGL((mxfp_bf16_b32_kernel<decltype(f), U, 0>), dim3(grid_for(n / 8, U * kThreads)), dim3(kThreads), 0, s,
                                    static_cast<const uint4*>(x), scales, reinterpret_cast<uint2*>(elements), nullptr, n / 8, f);
                 return check_launch("extract_mxfp");
