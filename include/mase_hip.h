@@ -295,6 +295,17 @@ int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elem
 int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes,
                               const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
                               int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
+/*
+ * The same with room for partial sums, as mase_hip_mxfp_gemm_ws: a product with few 256 x 256 tiles and a long K is
+ * split over K into fp32 partial sums in `workspace` (mase_hip_mxfp_gemm_scaled_workspace_bytes(M, N, K) bytes, 0 when
+ * the shape is not split; 16-byte aligned; NULL or too small: no split), and a second kernel adds them, the bias, and
+ * rounds.  Same reference counterpart as mase_hip_mxfp_gemm_scaled.
+ */
+int64_t mase_hip_mxfp_gemm_scaled_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mase_hip_mxfp_gemm_scaled_ws(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes,
+                                 const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
+                                 int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                 int64_t workspace_bytes, void* stream);
 
 /*
  * y[M,N] = A[M,K] * W[N,K]^T (+ bias) with a DENSE bfloat16 A (used as is, like a_dense of mase_hip_mxfp_gemm) and W in

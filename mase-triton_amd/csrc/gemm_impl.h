@@ -329,12 +329,12 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 }
 
 #include "gemm_tall.h"
-#include "gemm_scaled.h"
 #include "gemm_skinny.h"
 #include "gemm_rows16.h"
 #include "gemm_mid.h"
 #include "gemm_wide.h"
 #include "gemm_split_k.h"
+#include "gemm_scaled.h"
 
 // ---------------------------------------------------------------------------------------------
 // Small-shape kernel: 128 x 128 x 32 tiles, single LDS buffer.  Used when the problem cannot

@@ -65,18 +65,21 @@ __device__ inline void store16_nt(void* dst, const u32x4& v) {
 
 struct ScaledTile {
     int m0, n0;
+    int mac0;        // first macro step of this walk (K split: walk z of a tile takes macro steps z * nmac .. )
+    size_t y_off;    // byte offset of the walk's output array (K split: one fp32 [M, N] array per split)
 };
 
 template <int DT_OUT>
 __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_scaled_kernel(
     const uint8_t* __restrict__ a_codes, const uint32_t* __restrict__ a_scales, const uint8_t* __restrict__ w_codes,
     const uint32_t* __restrict__ w_scales, const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K,
-    int rows_a, int rows_w, int tiles_m, int tiles_n) {
+    int rows_a, int rows_w, int tiles_m, int tiles_n, int splits, int64_t y_split_bytes) {
+    // splits > 1: every tile is walked `splits` times, each time over K / splits of k and into its own [M, N] array of y
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_m = wave >> 1, wave_n = wave & 1;
-    const int nmac = K / SMAC;   // even and at least 4 (the launcher checks)
+    const int nmac = K / SMAC / splits;   // macro steps per walk: even and at least 4 (the launcher checks)
     const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
     // ---- per-lane constants
@@ -96,12 +99,13 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     const uint8_t* const a_sc = lds + S_SC_OFF + wave_m * 512 + (lane & 15) * 4 + (lane >> 4);
     const uint8_t* const w_sc = lds + S_SC_OFF + wave_n * 512 + 128 + (lane & 15) * 4 + (lane >> 4);
 
-    const int n_tiles = tiles_m * tiles_n;
+    const int n_tiles = tiles_m * tiles_n * splits;   // walks
     const int per_xcd = (n_tiles + 7) >> 3;
     const int slots = gridDim.x >> 3;
     auto has_tile = [&](int local) __attribute__((always_inline)) { return local < per_xcd && (int)(blockIdx.x & 7) * per_xcd + local < n_tiles; };
     auto tile_at = [&](int local) __attribute__((always_inline)) {
-        const int pos = (blockIdx.x & 7) * per_xcd + local;
+        const int walk = (blockIdx.x & 7) * per_xcd + local;
+        const int pos = walk / splits, z = walk - pos * splits;      // the splits of a tile run next to each other
         // groups of 4 tile rows, rows fastest: the 32 tiles an XCD runs at once form a 4 x 8 patch
         constexpr int GROUP = 4;
         const int in_group = GROUP * tiles_n;
@@ -111,6 +115,8 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
         ScaledTile t;
         t.m0 = (first_m + rr % rows) * SM;
         t.n0 = (rr / rows) * SN;
+        t.mac0 = z * nmac;
+        t.y_off = (size_t)z * (size_t)y_split_bytes;
         return t;
     };
 
@@ -131,13 +137,13 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     const uint32_t *pas[2], *pws[2];   // ... and its scales
     auto a_stream_to = [&](const ScaledTile& t, int h) __attribute__((always_inline)) {
         const int row = t.m0 + row0_w + 64 * h;
-        pa[h] = a_codes + (size_t)row * K;
-        pas[h] = a_scales + row;
+        pa[h] = a_codes + (size_t)row * K + (size_t)t.mac0 * SMAC;
+        pas[h] = a_scales + (size_t)t.mac0 * rows_a + row;
     };
     auto w_stream_to = [&](const ScaledTile& t, int h) __attribute__((always_inline)) {
         const int row = t.n0 + row0_w + 64 * h;
-        pw[h] = w_codes + (size_t)row * K;
-        pws[h] = w_scales + row;
+        pw[h] = w_codes + (size_t)row * K + (size_t)t.mac0 * SMAC;
+        pws[h] = w_scales + (size_t)t.mac0 * rows_w + row;
     };
     // operation q (0..9) of the next chunk of half H into ring slot SLOT
     auto chunk_dma = [&](auto h_c, auto slot_c, auto q_c) __attribute__((always_inline)) {
@@ -340,7 +346,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
                         const int row = row_base + ip * 32 + 8 * t + (int)(ol >> 3);
                         const int col = st_col + jp * PASS_COLS;
                         if (row < M && col < N) {
-                            uint8_t* const dst = static_cast<uint8_t*>(y) + ((size_t)row * N + col) * OB;
+                            uint8_t* const dst = static_cast<uint8_t*>(y) + cur.y_off + ((size_t)row * N + col) * OB;
                             store16_nt(dst, v[t]);
                         }
                     });
@@ -359,20 +365,59 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-// a_codes [rows_a, K], w_codes [rows_w, K]: rows padded to multiples of 256; scales [K / 128][rows] dwords
+// K split for few tiles and a long K (a [1024, 4096] output has 64 tiles for 256 CUs): the number of walks per tile, chosen so
+// that the walks about fill the CUs; a walk takes an even number of macro steps, at least 4.  Priced like the bf16 kernels'
+// split: macro steps per walk at about 1 us, rounds of walks over the CUs, and for a split the second launch plus the
+// partial sums written and read once.
+inline int plan_scaled_splits(int M, int N, int K, int cus) {
+    const int64_t tiles = (int64_t)((M + SM - 1) / SM) * ((N + SN - 1) / SN);
+    const int nmac = K / SMAC;
+    if (tiles * 2 > cus || cus <= 0) return 1;
+    const double mn_mb = (double)M * N * 4.0 / 1e6;
+    auto price = [&](int s) {
+        const double rounds = (double)((tiles * s + cus - 1) / cus);
+        return rounds * (nmac / s + 3) * 1.0 + (s > 1 ? 4.0 + (2.0 * s + 0.5) * mn_mb * 0.21 : 0.0);
+    };
+    int best = 1;
+    double best_t = price(1);
+    for (int s = 2; s <= 16 && tiles * s <= cus; ++s) {
+        if (nmac % s != 0 || (nmac / s) % 2 != 0 || nmac / s < 4) continue;
+        const double t = price(s);
+        if (t < best_t) { best_t = t; best = s; }
+    }
+    return best;
+}
+
+// a_codes [rows_a, K], w_codes [rows_w, K]: rows padded to multiples of 256; scales [K / 128][rows] dwords.  `workspace`
+// (may be null): room for the fp32 partial sums of a K split, splits * M * N * 4 bytes.
 template <int DT_OUT>
 int launch_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
-                       int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
+                       int bias_dtype, void* y, int M, int N, int K, void* workspace, int64_t workspace_bytes, hipStream_t s) {
     const int tiles_m = (M + SM - 1) / SM, tiles_n = (N + SN - 1) / SN;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
-    if (tiles >= (1 << 30)) return fail(ERR_UNSUPPORTED, "too many tiles");
+    if (tiles >= (1 << 26)) return fail(ERR_UNSUPPORTED, "too many tiles");
     const int cus = device_cu_count();
     if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
+    int splits = workspace ? plan_scaled_splits(M, N, K, cus) : 1;
+    const int64_t mn = (int64_t)M * N;
+    if (splits > 1 && workspace_bytes < splits * mn * 4) splits = 1;
+    const int64_t walks = tiles * splits;
+    const unsigned grid = (unsigned)(walks < cus ? ((walks + 7) / 8) * 8 : (cus / 8) * 8);
+    if (splits > 1) {
+        auto kern = mxfp_gemm_scaled_kernel<F32>;
+        static std::atomic<uint64_t> lds_allowed{0};
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), S_LDS_BYTES, lds_allowed)) return rc;
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), S_LDS_BYTES, s, a_codes, a_scales, w_codes, w_scales, static_cast<const void*>(nullptr), 0,
+                           workspace, M, N, K, tiles_m * SM, tiles_n * SN, tiles_m, tiles_n, splits, mn * 4);
+        if (int rc = check_launch("mxfp_gemm_scaled")) return rc;
+        hipLaunchKernelGGL(split_k_reduce_kernel<DT_OUT>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s,
+                           static_cast<const float*>(workspace), splits, mn, N, bias, bias_dtype, y);
+        return check_launch("mxfp_gemm_scaled");
+    }
     auto kern = mxfp_gemm_scaled_kernel<DT_OUT>;
     static std::atomic<uint64_t> lds_allowed{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), S_LDS_BYTES, lds_allowed)) return rc;
-    const unsigned grid = (unsigned)(tiles < cus ? ((tiles + 7) / 8) * 8 : (cus / 8) * 8);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kGemmThreads), S_LDS_BYTES, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N, K,
-                       tiles_m * SM, tiles_n * SN, tiles_m, tiles_n);
+                       tiles_m * SM, tiles_n * SN, tiles_m, tiles_n, 1, (int64_t)0);
     return check_launch("mxfp_gemm_scaled");
 }

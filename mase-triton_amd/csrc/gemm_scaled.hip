@@ -3,9 +3,9 @@
 
 using namespace mase;
 
-extern "C" int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales,
-                                         const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K,
-                                         void* stream) {
+static int scaled_entry(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales,
+                        const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                        int64_t workspace_bytes, void* stream) {
     if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K >= ((int64_t)1 << 27)) return fail(ERR_INVALID, "M, N must fit in 31 bits and K in 27");
     if (K % 256 != 0 || K < 512) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM needs K to be a multiple of 256, at least 512");
@@ -15,10 +15,31 @@ extern "C" int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t*
     if (!aligned(a_codes, 16) || !aligned(w_codes, 16) || !aligned(a_scales, 4) || !aligned(w_scales, 4) || !aligned(y, 16))
         return fail(ERR_INVALID, "codes and y must be 16-byte aligned, scales 4-byte aligned");
     if (N % (16 / dtype_size(out_dtype)) != 0) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM stores 16 bytes at a time: N must be a multiple of 8 (4 for fp32 output)");
+    if (workspace_bytes < 0) return fail(ERR_INVALID, "workspace_bytes must not be negative");
+    if (workspace && !aligned(workspace, 16)) return fail(ERR_INVALID, "workspace must be 16-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dispatch_dtype(out_dtype, [&](auto dout) {
-        return launch_gemm_scaled<decltype(dout)::value>(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, (int)M, (int)N, (int)K, s);
+        return launch_gemm_scaled<decltype(dout)::value>(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, (int)M, (int)N, (int)K,
+                                                         workspace, workspace ? workspace_bytes : 0, s);
     });
+}
+
+extern "C" int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales,
+                                         const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                         void* stream) {
+    return scaled_entry(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, out_dtype, M, N, K, nullptr, 0, stream);
+}
+
+extern "C" int mase_hip_mxfp_gemm_scaled_ws(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales,
+                                            const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                            void* workspace, int64_t workspace_bytes, void* stream) {
+    return scaled_entry(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, out_dtype, M, N, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int64_t mase_hip_mxfp_gemm_scaled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M < 1 || N < 1 || K < 512 || K % 256 != 0 || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K >= ((int64_t)1 << 27)) return 0;
+    const int splits = plan_scaled_splits((int)M, (int)N, (int)K, device_cu_count());
+    return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
 }
 
 extern "C" int mase_hip_mxfp_gemm_prepared_w(const void* a_dense, int a_dtype, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,

@@ -282,9 +282,13 @@ def scaled_operand_from_mxfp(scales: Tensor, elements: Tensor, meta: MXFPMeta, r
     return ScaledOperand(codes, out_scales, rows, K)
 
 
+_SCALED_WS_BYTES: dict[tuple, int] = {}
+
+
 def mxfp_gemm_scaled(a: ScaledOperand, w: ScaledOperand, bias: Tensor | None, output_dtype: torch.dtype,
-                     out: Tensor | None = None) -> Tensor:
-    """y[M,N] = A @ W^T (+ bias) on the block-scaled matrix instruction, fp32 accumulation."""
+                     out: Tensor | None = None, split_k: bool = True) -> Tensor:
+    """y[M,N] = A @ W^T (+ bias) on the block-scaled matrix instruction, fp32 accumulation.
+    ``split_k``: allow a temporary for partial sums where the library asks for one (few tiles, long K)."""
     assert a.K == w.K
     M, N, K = a.rows, w.rows, a.K
     dev = w.codes.device
@@ -298,10 +302,18 @@ def mxfp_gemm_scaled(a: ScaledOperand, w: ScaledOperand, bias: Tensor | None, ou
     else:
         assert out.is_contiguous() and out.dtype == output_dtype and out.numel() == M * N and out.device == dev
         y = out
+    lib = _lib.load()
     with _lib.on_device(dev):
-        _lib.check(_lib.load().mase_hip_mxfp_gemm_scaled(
+        ws_bytes = 0
+        if split_k:
+            key = (dev.index, M, N, K)
+            ws_bytes = _SCALED_WS_BYTES.get(key)
+            if ws_bytes is None:
+                ws_bytes = _SCALED_WS_BYTES[key] = lib.mase_hip_mxfp_gemm_scaled_workspace_bytes(M, N, K)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes > 0 else None
+        _lib.check(lib.mase_hip_mxfp_gemm_scaled_ws(
             a.codes.data_ptr(), a.scales.data_ptr(), w.codes.data_ptr(), w.scales.data_ptr(), b_ptr, b_dt, y.data_ptr(),
-            _lib.dtype_code(output_dtype), M, N, K, _lib.stream_ptr(dev)))
+            _lib.dtype_code(output_dtype), M, N, K, None if ws is None else ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
     return y
 
 

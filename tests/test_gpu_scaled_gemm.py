@@ -252,6 +252,35 @@ def test_special_blocks_poison_the_same_outputs(mh):
     assert rel_fro(y[ok], y_ref[ok]) <= F32_TOL
 
 
+@pytest.mark.parametrize("MNK", [(256, 256, 4096), (300, 520, 2048), (1024, 512, 14336), (700, 264, 7168)])
+def test_scaled_gemm_k_split(mh, MNK):
+    """Few tiles and a long K: the launcher splits K over several workgroups per tile (fp32 partial sums in a workspace,
+    a second kernel adds them).  Against the checker and against the unsplit call (which it may equal bit for bit: products
+    of two MXFP values have at most eight significant bits, and sums of a few thousand of them are often exact in fp32
+    whatever the order)."""
+    from mase_hip import _lib
+
+    M, N, K = MNK
+    need = _lib.load().mase_hip_mxfp_gemm_scaled_workspace_bytes(M, N, K)
+    if need == 0:
+        pytest.skip("this shape is not split on this device")
+    assert need % (M * N * 4) == 0 and 2 <= need // (M * N * 4) <= 16
+    g = torch.Generator().manual_seed(K + M)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    _, _, x_dq = quantised(x, "MXFP8_E4M3_fn")
+    w_sc, w_el, w_dq = quantised(w, "OCP_MXFP6_E3M2")
+    y_ref = oracle.matmul_nt(x_dq, w_dq) + b.float()
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), mh.meta.MXFP8_E4M3_fn)
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), mh.meta.OCP_MXFP6_E3M2, N, K)
+    for odt, tol in ((torch.float32, F32_TOL), (torch.bfloat16, 1e-3)):
+        y = mh.mxk.mxfp_gemm_scaled(a, wop, b.to(DEV), odt)
+        y_one = mh.mxk.mxfp_gemm_scaled(a, wop, b.to(DEV), odt, split_k=False)
+        assert rel_fro(y, y_ref.to(odt)) <= tol
+        assert rel_fro(y, y_one) <= tol
+
+
 # ---------------------------------------------------------------- the prepared weight on the bf16 kernel
 @pytest.mark.parametrize("MNK", [(512, 256, 512), (1100, 384, 1024), (640, 128, 128)])
 @pytest.mark.parametrize("w_tag", SCALED_TAGS)

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(lib):
     from mase_hip import _lib
 
     names = declared_symbols()
-    assert len(names) == 22
+    assert len(names) == 24
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mase_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of step with the header"
