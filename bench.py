@@ -511,6 +511,7 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
 
     rows = linear_rows(N, K, (16, 64, 128, 256, 384, 512, 768, 1024, 2048, 4096, 8192))
     rows_down = linear_rows(K, N, (16, 64, 256, 512, 1024, 2048, 4096))  # the transposed layer shape: few W rows, long K
+    rows_sq = linear_rows(K, K, (128, 256, 512, 1024, 2048, 4096))
     w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
     n = w.numel()
     cast = {
@@ -522,7 +523,7 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
     }
     cast["extract_in_place_GBps"] = round(n * (3 + 1 / 32) / cast["extract_in_place_us"] / 1e3, 0)
     cast["qdq_in_place_GBps"] = round(n * 4 / cast["qdq_in_place_us"] / 1e3, 0)
-    return {"linear_N14336_K4096": rows, "linear_N4096_K14336": rows_down, "casts_along_axis0": cast}
+    return {"linear_N14336_K4096": rows, "linear_N4096_K14336": rows_down, "linear_N4096_K4096": rows_sq, "casts_along_axis0": cast}
 
 
 def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):

@@ -35,10 +35,12 @@ from .cast import compose_mxfp_tensor, extract_mxfp_components, quantize_dequant
 _LAYER_TYPES = ("XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq")
 _GEMM_DTYPES = (torch.bfloat16, torch.float32)
 _BACKENDS = ("separate", "fused", "fused_bf16", "fused_scaled")
-# rows of x from which "fused" takes the block-scaled route: with fewer the weight-streaming bf16 kernels win (the
-# block-scaled kernel works on 256 x 256 tiles and the weight has to be brought into its form first)
-SCALED_FROM_ROWS = 256
-SCALED_FROM_ROWS_UNPREPARED = 1024   # ... when the weight operand has to be built inside the call
+# rows of x from which "fused" takes the block-scaled route.  With the weight operand at hand (a layer keeps it) the
+# block-scaled kernel, K split over workgroups where its 256 x 256 tiles are few, is level with the weight-streaming bf16
+# kernels at 64 rows and ahead from there (N x K = 14336 x 4096: 29 / 33 / 44 us at 64 / 128 / 256 rows against 29 / 37 /
+# 48 us); when the operand has to be built inside the call (N * K bytes read and written) it pays from about 768 rows
+SCALED_FROM_ROWS = 64
+SCALED_FROM_ROWS_UNPREPARED = 768
 
 
 def parse_mxfp_linear_type(x_meta: MXFPMeta | None, w_tensor_meta: MXFPTensorMeta | None,
