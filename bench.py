@@ -85,6 +85,7 @@ def parse_args():
     ap.add_argument("--only-gemm-kernel", choices=("scaled", "bf16", "bf16-components"), default=None,
                     help="profiling aid: launch only that GEMM kernel (block-scaled FP8; bf16 MFMA on the prepared weight; bf16 MFMA on "
                          "the weight components) on the headline shape, --steps times after --warmup, and print nothing")
+    ap.add_argument("--rows", type=int, default=0, help="with --only-gemm-kernel: the first ROWS rows of C4's x instead of all 16384")
     ap.add_argument("--summarize-sq", metavar="COUNTER_CSV",
                     help="no GPU needed: per-kernel table (stdout, markdown) from the counter_collection.csv of a rocprofv3 --pmc run with "
                          "SQ_BUSY_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_LDS SQ_WAIT_ANY SQ_WAVE_CYCLES SQ_WAVES [SQ_LDS_BANK_CONFLICT]")
@@ -189,6 +190,9 @@ def bench_linear(args, torch, MXFP_F, kernels, fmt):
 
     w_kept = L.scaled_weight_operand(w_sc, w_el, w_tm)      # what a layer keeps
     if args.only_gemm_kernel:
+        if args.rows:
+            M = args.rows
+            x = x[:M].contiguous()
         a_op = kernels.scaled_operand_from_dense(x, fmt)
         a = kernels.quantize_dequantize(x.view(-1), fmt, torch.bfloat16).view(M, K)
         fn = ((lambda: kernels.mxfp_gemm_scaled(a_op, w_kept, None, torch.bfloat16)) if args.only_gemm_kernel == "scaled" else
@@ -660,7 +664,8 @@ def bench_c5(torch, with_cpu, steps=20, warmup=8):
     gate / up [14336, 4096] and down [4096, 14336] ~N(0, 0.02) stored as MXFP6 E3M2, MXFP8 E4M3 activations, block 32,
     x [4 x 2048, 4096] bf16 ~N(0, 1) (tests/workloads.py: make_c5).  Gate and up are stacked into one [28672, 4096] layer
     (MXFP blocks run along in_features, so stacking rows changes no value): x is quantised once and one GEMM serves both.
-    Per block: two quantise kernels, two GEMMs, SiLU and the product in torch."""
+    Per block on backend "fused": quantise x, GEMM, one kernel for SiLU, product and quantisation, GEMM
+    (MXFPLinearPTQ.forward_swiglu); on the other backends SiLU and the product are torch's."""
     import workloads
     from mase_hip.mxfp import kernels
     from mase_hip.mxfp.layers import MXFPLinearPTQ
@@ -684,29 +689,44 @@ def bench_c5(torch, with_cpu, steps=20, warmup=8):
 
         def mlp():
             t = gu(x)
+            if backend == "fused":      # activation, product and quantisation of the down layer's input in one kernel
+                return d.forward_swiglu(t[..., :inter], t[..., inter:])
             return d(torch.nn.functional.silu(t[..., :inter]) * t[..., inter:])
 
         ms[backend] = timed_loop(torch, mlp, steps, warmup)
         if backend == "fused":
-            # the two GEMM kernels of the block on their own, bracketed by events on the launch stream
+            # the block's four kernels launched directly (what the two layer calls above launch), so that events on the
+            # launch stream can bracket the two GEMMs inside the timed loop
             rows = x.shape[0] * x.shape[1]
-            a1 = kernels.scaled_operand_from_dense(x.view(rows, -1), MXFP8_E4M3_fn)
-            h = torch.nn.functional.silu(gu(x)[..., :inter]) * gu(x)[..., inter:]
-            a2 = kernels.scaled_operand_from_dense(h.view(rows, -1), MXFP8_E4M3_fn)
-            w1, w2 = gu._weight_operand(x), d._weight_operand(h)
+            x2d = x.view(rows, -1)
+            w1, w2 = gu._weight_operand(x), d._weight_operand(torch.empty(rows, inter, dtype=x.dtype, device=dev))
             assert w1 is not None and w2 is not None, "the C5 layers did not take the block-scaled route"
-            gemm_ms = []
-            for a_op, w_op in ((a1, w1), (a2, w2)):
-                for _ in range(5):
-                    kernels.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
-                pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-                for e0, e1 in pairs:
-                    e0.record()
-                    kernels.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
-                    e1.record()
-                torch.cuda.synchronize()
-                gemm_ms.append(sum(event_ms(pairs)) / steps)
-            del a1, a2, h, w1, w2
+
+            def block(ev=None):
+                a1 = kernels.scaled_operand_from_dense(x2d, MXFP8_E4M3_fn)
+                if ev is not None:
+                    ev[0][0].record()
+                t = kernels.mxfp_gemm_scaled(a1, w1, None, torch.bfloat16)
+                if ev is not None:
+                    ev[0][1].record()
+                a2 = kernels.scaled_operand_from_swiglu(t[:, :inter], t[:, inter:], MXFP8_E4M3_fn)
+                if ev is not None:
+                    ev[1][0].record()
+                y = kernels.mxfp_gemm_scaled(a2, w2, None, torch.bfloat16)
+                if ev is not None:
+                    ev[1][1].record()
+                return y
+
+            assert torch.equal(block().view(torch.int16).view(-1), mlp().view(torch.int16).view(-1)), "the event-bracketed block differs from the layers' output"
+            for _ in range(warmup):
+                block()
+            torch.cuda.synchronize()
+            evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(2)] for _ in range(steps)]
+            for i in range(steps):
+                block(evs[i])
+            torch.cuda.synchronize()
+            gemm_ms = [sum(event_ms([e[j] for e in evs])) / steps for j in range(2)]
+            del w1, w2
         del ls, gu, d
     tf = lambda t: flop / (t * 1e-3) / 1e12
     kern_tf = tf(sum(gemm_ms))
@@ -718,7 +738,7 @@ def bench_c5(torch, with_cpu, steps=20, warmup=8):
                      "frac": round(kern_tf / MFMA_FP8_PEAK_TFLOPS, 4), "frac_of_bf16_peak": round(kern_tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "kernel": "mxfp_gemm_scaled_kernel", "avg_kernel_ms": {"gate_up": round(gemm_ms[0], 4), "down": round(gemm_ms[1], 4)},
                      "traffic": None},
-        "note": "flop = the three GEMMs; ms_per_block = whole block (quantise kernels, GEMMs, SiLU and product)",
+        "note": "flop = the three GEMMs; ms_per_block = whole block (quantise kernels, GEMMs, SiLU and product; fused: the down layer reads gate and up through forward_swiglu)",
     }
     if with_cpu:
         from oracle import torch_fake

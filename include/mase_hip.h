@@ -292,6 +292,18 @@ int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits,
 int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elements, int exp_bits,
                                       int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
                                       uint32_t* out_scales, void* stream);
+/*
+ * The activations of the down projection of a SwiGLU block, quantised where they are formed: the matrix that is
+ * extracted is silu(gate) * up (gate, up: row-major [rows, K] bfloat16 with a common row stride of `row_stride`
+ * elements, e.g. the two halves of a stacked gate / up projection's output, row_stride = 2 K), each of the two
+ * operations rounded to bfloat16 as a tensor library rounds it; the bfloat16 product itself is never stored.
+ * No counterpart in the reference, where the caller writes  down(silu(gate(x)) * up(x))  between two MXFPLinearPTQ
+ * layers (src/mase_triton/mxfp/layers.py:150-165 is the layer's forward) and the extract of
+ * src/mase_triton/mxfp/functional/linear.py:50-52 then reads the product back from memory.
+ */
+int mase_hip_scaled_operand_from_swiglu(const void* gate, const void* up, int dtype, int64_t row_stride,
+                                        int exp_bits, int frac_bits, int64_t rows, int64_t K,
+                                        uint8_t* out_codes, uint32_t* out_scales, void* stream);
 int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes,
                               const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
                               int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);

@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import argparse
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -18,8 +19,9 @@ CSRC = os.path.join(ROOT, "csrc")
 OBJ = os.path.join(ROOT, "build")
 LIB_DIR = os.path.join(ROOT, "mase_hip", "lib")
 LIB = os.path.join(LIB_DIR, "libmase_hip.so")
-# the benchmark's yardstick (a tuned streaming copy); not part of the product's C ABI
-BENCH_SRC = os.path.join(CSRC, "bench", "stream_copy.hip")
+# helpers of the benchmark and the tests (a tuned streaming copy as yardstick; the SwiGLU arithmetic on its own); not part of
+# the product's C ABI
+BENCH_SRCS = [os.path.join(CSRC, "bench", f) for f in ("stream_copy.hip", "swiglu_probe.hip")]
 BENCH_LIB = os.path.join(LIB_DIR, "libmase_bench.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -34,6 +36,18 @@ def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def _includes(path: str, seen: set[str] | None = None) -> set[str]:
+    """The files `path` includes with quotes, transitively (what its object file depends on besides itself)."""
+    seen = set() if seen is None else seen
+    with open(path) as f:
+        for m in re.finditer(r'^\s*#\s*include\s+"([^"]+)"', f.read(), re.M):
+            inc = os.path.normpath(os.path.join(os.path.dirname(path), m.group(1)))
+            if inc not in seen and os.path.exists(inc):
+                seen.add(inc)
+                _includes(inc, seen)
+    return seen
+
+
 def _stale(target: str, deps: list[str]) -> bool:
     if not os.path.exists(target):
         return True
@@ -44,14 +58,12 @@ def _stale(target: str, deps: list[str]) -> bool:
 def build_library(force: bool = False, save_temps: bool = False, verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
-    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
-    headers.append(os.path.join(os.path.dirname(ROOT), "include", "mase_hip.h"))
     srcs = sources()
     objs = [os.path.join(OBJ, os.path.basename(s)[:-4] + ".o") for s in srcs]
 
     def compile_one(pair):
         src, obj = pair
-        if not (force or _stale(obj, [src] + headers)):
+        if not (force or _stale(obj, [src, *_includes(src)])):
             return
         cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
         if save_temps:
@@ -67,8 +79,8 @@ def build_library(force: bool = False, save_temps: bool = False, verbose: bool =
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)
-    if force or _stale(BENCH_LIB, [BENCH_SRC]):
-        cmd = [HIPCC, *FLAGS, "-shared", BENCH_SRC, "-o", BENCH_LIB]
+    if force or _stale(BENCH_LIB, BENCH_SRCS + [h for src in BENCH_SRCS for h in _includes(src)]):
+        cmd = [HIPCC, *FLAGS, "-shared", *BENCH_SRCS, "-o", BENCH_LIB]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)

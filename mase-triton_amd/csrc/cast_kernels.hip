@@ -8,6 +8,7 @@
 #include "../../include/mase_hip.h"
 #include "mase_host.h"
 #include "mxfp_compose.h"
+#include "swiglu.h"
 
 namespace mase {
 
@@ -594,31 +595,35 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
     }
 }
 
-// bf16 matrix x [rows, K] -> operand of the block-scaled GEMM in one pass (extract, then the re-encoding / embedding
-// above).  A workgroup owns 32 rows x 128 k, the unit whose scale dwords fill one 128-byte line of the transposed scale
-// array: 16 lanes read the 256 bytes of one row (8 elements each, four lanes to a block), a wavefront four rows per
-// step, two steps.  The four scale bytes of a row are gathered into one lane and stored as a dword.
-template <class F>
-__global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes,
-                                                                      uint32_t* __restrict__ scales, int rows, int K, int nmac,
-                                                                      uint32_t rows_pad, F f) {
+// bf16 matrix x [rows, K] (row stride ld elements) -> operand of the block-scaled GEMM in one pass (extract, then the
+// re-encoding / embedding above).  A workgroup owns 32 rows x 128 k, the unit whose scale dwords fill one 128-byte line of
+// the transposed scale array: 16 lanes read the 256 bytes of one row (8 elements each, four lanes to a block), a
+// wavefront four rows per step, two steps.  The four scale bytes of a row are gathered into one lane and stored as a dword.
+// SWIGLU: the matrix that is quantised is silu(x) * up (up [rows, K] with the same row stride), formed in registers.
+template <class F, bool SWIGLU>
+__global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ up, size_t ld,
+                                                                      uint8_t* __restrict__ codes, uint32_t* __restrict__ scales, int rows,
+                                                                      int K, int nmac, uint32_t rows_pad, F f) {
     __shared__ __attribute__((aligned(16))) uint8_t lut[LdsLut<F, false>::BYTES];
     const uint32_t ms = blockIdx.x % (uint32_t)nmac, row_base = (blockIdx.x / (uint32_t)nmac) * 32u;
     const int t = threadIdx.x;
-    uint4 raw[2];
+    uint4 raw[2], raw_up[2];
     size_t off[2];
     bool live[2];
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
         const uint32_t row = row_base + 16u * r + (uint32_t)(t >> 4);
+        const uint32_t col = ms * 128u + (uint32_t)(t & 15) * 8u;
         live[r] = row < (uint32_t)rows;
-        off[r] = (size_t)row * K + ms * 128u + (uint32_t)(t & 15) * 8u;
-        raw[r] = live[r] ? ld128(x + off[r]) : make_uint4(0, 0, 0, 0);
+        off[r] = (size_t)row * K + col;
+        raw[r] = live[r] ? ld128(x + (size_t)row * ld + col) : make_uint4(0, 0, 0, 0);
+        if (SWIGLU) raw_up[r] = live[r] ? ld128(up + (size_t)row * ld + col) : make_uint4(0, 0, 0, 0);
     }
     LdsLut<F, false>::fill(lut);
     const uint32_t lut_addr = (uint32_t)(uintptr_t)lut;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
+        if (SWIGLU) raw[r] = swiglu_x8(raw[r], raw_up[r]);
         uint32_t o[4], scale;
         bf16_block_step<F, false>(raw[r], f, o, scale, lut_addr);
         uint32_t w0 = __builtin_amdgcn_perm(o[1], o[0], 0x06040200u), w1 = __builtin_amdgcn_perm(o[3], o[2], 0x06040200u);
@@ -1435,25 +1440,43 @@ int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elem
     });
 }
 
-int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
-                                       uint32_t* out_scales, void* stream) {
+static int scaled_from_dense_entry(const void* x, const void* up, int64_t ld, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K,
+                                   uint8_t* out_codes, uint32_t* out_scales, void* stream) {
     uint32_t rows_pad;
     if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, rows_pad)) return rc;
     if (x_dtype != BF16) return fail(ERR_UNSUPPORTED, "a dense operand of the block-scaled GEMM must be bfloat16");
     if (!x || !out_codes || !out_scales) return fail(ERR_INVALID, "null pointer");
-    if (!aligned(x, 16) || !aligned(out_codes, 8) || !aligned(out_scales, 4)) return fail(ERR_INVALID, "x must be 16-byte aligned, out_codes 8-byte, out_scales 4-byte");
+    if (ld < K || ld % 8 != 0) return fail(ERR_INVALID, "the row stride must be at least K and a multiple of 8 elements");
+    if (!aligned(x, 16) || (up && !aligned(up, 16)) || !aligned(out_codes, 8) || !aligned(out_scales, 4))
+        return fail(ERR_INVALID, "the dense inputs must be 16-byte aligned, out_codes 8-byte, out_scales 4-byte");
     hipStream_t s = static_cast<hipStream_t>(stream);
     return dispatch_fmt(exp_bits, frac_bits, 1, RN, [&](auto f) {
         if constexpr (decltype(f)::kStatic && decltype(f){}.E() != 5) {
             const int nmac = (int)(K / 128);
             const int64_t blocks = (rows + 31) / 32 * nmac;
             if (blocks > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "operand too large for one launch");
-            hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f)>), dim3((unsigned)blocks), dim3(kThreads), 0, s, static_cast<const uint16_t*>(x),
-                               out_codes, out_scales, (int)rows, (int)K, nmac, rows_pad, f);
+            const uint16_t *xp = static_cast<const uint16_t*>(x), *upp = static_cast<const uint16_t*>(up);
+            if (up)
+                hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f), true>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp, upp, (size_t)ld,
+                                   out_codes, out_scales, (int)rows, (int)K, nmac, rows_pad, f);
+            else
+                hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f), false>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp, upp, (size_t)ld,
+                                   out_codes, out_scales, (int)rows, (int)K, nmac, rows_pad, f);
             return check_launch("scaled_operand_from_dense");
         }
         return fail(ERR_UNSUPPORTED, "element format not supported by the block-scaled GEMM");
     });
+}
+
+int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
+                                       uint32_t* out_scales, void* stream) {
+    return scaled_from_dense_entry(x, nullptr, K, x_dtype, exp_bits, frac_bits, rows, K, out_codes, out_scales, stream);
+}
+
+int mase_hip_scaled_operand_from_swiglu(const void* gate, const void* up, int dtype, int64_t row_stride, int exp_bits, int frac_bits, int64_t rows,
+                                        int64_t K, uint8_t* out_codes, uint32_t* out_scales, void* stream) {
+    if (!up) return fail(ERR_INVALID, "null pointer");
+    return scaled_from_dense_entry(gate, up, row_stride, dtype, exp_bits, frac_bits, rows, K, out_codes, out_scales, stream);
 }
 
 }  // extern "C"

@@ -267,6 +267,24 @@ def scaled_operand_from_dense(x: Tensor, meta: MXFPMeta) -> ScaledOperand:
     return ScaledOperand(codes, scales, rows, K)
 
 
+def scaled_operand_from_swiglu(gate: Tensor, up: Tensor, meta: MXFPMeta) -> ScaledOperand:
+    """silu(gate) * up (bfloat16 [rows, K] each, unit inner stride, the same row stride: e.g. the two halves of a stacked
+    projection's output) quantised straight into a block-scaled GEMM operand; the product is never stored."""
+    assert gate.ndim == 2 and gate.shape == up.shape and gate.dtype == up.dtype == torch.bfloat16
+    assert scaled_format_supported(meta) and meta.round_mode == "rn"
+    _lib.require_gpu(gate, "activations")
+    assert gate.device == up.device
+    if gate.stride(1) != 1 or up.stride(1) != 1 or gate.stride(0) != up.stride(0) or gate.stride(0) % 8 or gate.data_ptr() % 16 or up.data_ptr() % 16:
+        gate, up = gate.contiguous(), up.contiguous()
+    rows, K = gate.shape
+    codes, scales = _scaled_buffers(rows, K, gate.device)
+    with _lib.on_device(gate.device):
+        _lib.check(_lib.load().mase_hip_scaled_operand_from_swiglu(
+            gate.data_ptr(), up.data_ptr(), _lib.dtype_code(gate.dtype), gate.stride(0) if rows > 1 else K,
+            meta.element_exp_bits, meta.element_frac_bits, rows, K, codes.data_ptr(), scales.data_ptr(), _lib.stream_ptr(gate.device)))
+    return ScaledOperand(codes, scales, rows, K)
+
+
 def scaled_operand_from_mxfp(scales: Tensor, elements: Tensor, meta: MXFPMeta, rows: int, K: int) -> ScaledOperand:
     """MXFP components of a row-major [rows, K] matrix, blocked along K -> block-scaled GEMM operand."""
     assert scaled_format_supported(meta)

@@ -114,6 +114,17 @@ class MXFPLinearPTQ(nn.Module):
         through ``.data`` are not."""
         self._scaled_w = self._scaled_w_key = None
 
+    def _takes_scaled_route(self, input: Tensor) -> bool:
+        """Does ``forward(input)`` run on the block-scaled GEMM?"""
+        from .functional import linear as L
+
+        if self.backend in ("separate", "fused_bf16") or not self.layer_type.startswith("XqWq") or input.device.type != "cuda":
+            return False
+        rows = input.numel() // input.shape[-1] if input.numel() else 0
+        bias = self.bias if not self.layer_type.endswith("Bq") else None
+        return ((self.backend == "fused_scaled" or rows >= L.SCALED_FROM_ROWS)
+                and L._scaled_eligible(input, self.x_mxfp_meta, self.w_tensor_meta, bias))
+
     def _weight_operand(self, input: Tensor):
         """The weight in the block-scaled GEMM's form when this call has a kernel that reads it (the block-scaled GEMM for
         quantised bfloat16 activations, the large-tile bf16 kernel from 512 rows on), else None."""
@@ -123,9 +134,7 @@ class MXFPLinearPTQ(nn.Module):
         if self.backend == "separate" or "Wq" not in self.layer_type or input.device.type != "cuda":
             return None
         rows = input.numel() // input.shape[-1] if input.numel() else 0
-        bias = self.bias if not self.layer_type.endswith("Bq") else None
-        scaled = (self.backend != "fused_bf16" and self.layer_type.startswith("XqWq") and (self.backend == "fused_scaled" or rows >= L.SCALED_FROM_ROWS)
-                  and L._scaled_eligible(input, self.x_mxfp_meta, self.w_tensor_meta, bias))
+        scaled = self._takes_scaled_route(input)
         if not scaled:
             tm = self.w_tensor_meta
             bf16 = (self.backend != "fused_scaled" and len(tm.shape) == 2 and kernels.scaled_format_supported(tm.meta) and tm.block_dim % 2 == 1
@@ -146,6 +155,25 @@ class MXFPLinearPTQ(nn.Module):
             w_tensor_meta=self.w_tensor_meta, b=self.bias, b_scales=self.b_scales, b_elements=self.b_elements,
             b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend,
             w_operand=self._weight_operand(input))
+
+    @torch.no_grad()
+    def forward_swiglu(self, gate: Tensor, up: Tensor) -> Tensor:
+        """``self(silu(gate) * up)``, the down projection of a SwiGLU block (not in the reference, where the caller writes
+        that expression).  On the block-scaled route the activation, the product and the quantisation of the result run
+        in one kernel that reads ``gate`` and ``up`` (e.g. the two halves of a stacked gate / up layer's output, as
+        views) and writes FP8 codes: the bfloat16 product never goes to memory.  Each of the two operations is rounded to
+        bfloat16 as torch rounds it, so the result equals the expression's up to the last bit of the SiLU's exponential.
+        Everywhere else this is the expression."""
+        from . import kernels
+
+        if (gate.shape == up.shape and gate.dtype == up.dtype and gate.device == up.device and gate.shape[-1] == self.in_features
+                and self.layer_type == "XqWqB" and self._takes_scaled_route(gate)):
+            w_op = self._weight_operand(gate)
+            a_op = kernels.scaled_operand_from_swiglu(gate.reshape(-1, self.in_features) if gate.ndim != 2 else gate,
+                                                      up.reshape(-1, self.in_features) if up.ndim != 2 else up, self.x_mxfp_meta)
+            y = kernels.mxfp_gemm_scaled(a_op, w_op, self.bias, gate.dtype)
+            return y.view(*gate.shape[:-1], self.out_features)
+        return self.forward(torch.nn.functional.silu(gate) * up)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "

@@ -648,6 +648,47 @@ def test_config_c5_swiglu_chain(mh, backend):
     assert err <= (5 if scaled else 3) * REL_FRO_TOL, f"chain: {err}"
 
 
+def test_forward_swiglu_is_the_expression(mh):
+    """MXFPLinearPTQ.forward_swiglu(gate, up) against layer(silu(gate) * up): on the block-scaled route one kernel forms the
+    product and quantises it (reading the two halves of a stacked projection's output as views), elsewhere the
+    expression itself runs.  The fused kernel rounds where the two tensor operations round, so the outputs agree far
+    inside the path's 1e-3 (the last bit of the exponential may move an element to a neighbouring code now and then);
+    the down projection is also held to 1e-3 against a float64 product of the checker's dequantised operands, computed
+    from the very gate and up values the layer saw."""
+    from workloads import make_c5
+
+    x, wg, wu, wd = make_c5()
+    xfmt, wfmt = preset(mh, "MXFP8_E4M3_fn"), preset(mh, "OCP_MXFP6_E3M2")
+
+    def layer(w, backend):
+        lin = torch.nn.Linear(w.shape[1], w.shape[0], bias=False, dtype=torch.bfloat16, device=DEV)
+        lin.weight.data.copy_(w)
+        return mh.MXFPLinearPTQ.from_linear(lin, xfmt, wfmt, None, "XqWqB", backend)
+
+    inter = wg.shape[0]
+    gu, down = layer(torch.cat([wg, wu]), "fused"), layer(wd, "fused")
+    t = gu(x.to(DEV))                                        # [4, 2048, 2 * 14336]
+    gate, up = t[..., :inter], t[..., inter:]
+    y = down.forward_swiglu(gate, up)
+    y_expr = down(torch.nn.functional.silu(gate) * up)
+    assert y.shape == y_expr.shape == (4, 2048, 4096)
+    assert rel_fro(y, y_expr) <= 1e-4
+    # against the checker on a sample of rows and columns
+    rows = torch.arange(7, 8192, 523)
+    cols = torch.arange(2, 4096, 111)
+    g_cpu, u_cpu = gate.reshape(-1, inter)[rows.to(DEV)].cpu(), up.reshape(-1, inter)[rows.to(DEV)].cpu()
+    h_cpu = torch.nn.functional.silu(g_cpu) * u_cpu
+    ref = oracle.matmul_nt(oracle.qdq_mxfp(h_cpu, 32, 4, 3), oracle.qdq_mxfp(wd[cols], 32, 3, 2)).to(torch.bfloat16)
+    err = rel_fro(y.view(-1, 4096)[rows.to(DEV)][:, cols.to(DEV)], ref)
+    assert err <= REL_FRO_TOL, err
+    # few rows, another backend, mismatched shapes: the expression
+    small = t[0, :16]
+    assert torch.equal(down.forward_swiglu(small[:, :inter], small[:, inter:]), down(torch.nn.functional.silu(small[:, :inter]) * small[:, inter:]))
+    sep = layer(wd, "separate")
+    part = t[0, :256]
+    assert torch.equal(sep.forward_swiglu(part[:, :inter], part[:, inter:]), sep(torch.nn.functional.silu(part[:, :inter]) * part[:, inter:]))
+
+
 @pytest.mark.parametrize("func_type", ["XW", "XqW", "XWq", "XqWq"])
 @pytest.mark.parametrize("backend", ["separate", "fused"])
 def test_mxfp_matmul(mh, func_type, backend):

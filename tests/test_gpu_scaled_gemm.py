@@ -10,14 +10,19 @@ What is checked, against the CPU checker's components of the same inputs:
     16-bit outputs (compared with the reference rounded to that type) and 1e-4 for fp32 outputs (measured 1 - 2e-5:
     the matrix unit adds a block's 32 products with fewer bits than a chain of fp32 FMAs keeps);
   * identity times W returns W's dequantised values exactly;
-  * inf / NaN blocks poison exactly the rows (columns) they poison in dequantise-then-matmul.
+  * inf / NaN blocks poison exactly the rows (columns) they poison in dequantise-then-matmul;
+  * the operand formed from silu(gate) * up inside the kernel equals the one built from torch's two bf16 operations.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
 
 import oracle
 from helpers import PRESETS
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 pytestmark = pytest.mark.gpu
 
@@ -152,6 +157,72 @@ def test_operand_from_components_equals_from_dense(mh, tag):
     assert np.array_equal(ca, cb)
 
 
+def swiglu_inputs(rows, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    t = (2.0 * torch.randn(rows, 2 * K, generator=g)).to(torch.bfloat16)
+    t[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, 100.0, -100.0, 1e-30, -1e-30]).to(torch.bfloat16)
+    t[1, 3] = float("inf")
+    t[2, 4] = float("-inf")
+    t[3, 5] = float("nan")
+    t[4, K + 6] = float("inf")
+    t[5, : 64] = 0.0
+    return t
+
+
+def test_swiglu_arithmetic_on_every_gate_value():
+    """The operand kernel's silu(gate) * up (csrc/swiglu.h: hardware exp2 and reciprocal instead of the library's exp and
+    division), run on its own through the test helper library.  The gate is bfloat16 and the SiLU is rounded to bfloat16
+    before the product, so its 65536 inputs are all the cases there are: with up = 1 the output is that rounded SiLU, and
+    it must be torch's, bit for bit, for every input (NaN for NaN).  Then 2^20 random pairs against torch's expression."""
+    import ctypes
+
+    path = os.path.join(ROOT, "mase-triton_amd", "mase_hip", "lib", "libmase_bench.so")
+    assert os.path.exists(path), "libmase_bench.so is not built (python mase-triton_amd/build.py)"
+    lib = ctypes.CDLL(path)
+    lib.mase_bench_swiglu_bf16.restype = ctypes.c_int
+    lib.mase_bench_swiglu_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+
+    def run(gate, up):
+        out = torch.empty_like(gate)
+        assert lib.mase_bench_swiglu_bf16(gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        return out
+
+    gate = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).to(DEV)
+    got = run(gate, torch.ones_like(gate))
+    want = torch.nn.functional.silu(gate)
+    nan = want.isnan()
+    assert torch.equal(got.isnan(), nan)
+    assert torch.equal(got[~nan].view(torch.int16), want[~nan].view(torch.int16))
+    g = torch.Generator().manual_seed(21)
+    gate = (3.0 * torch.randn(1 << 20, generator=g)).to(torch.bfloat16).to(DEV)
+    up = (torch.randn(1 << 20, generator=g) * torch.exp2(torch.randint(-8, 8, (1 << 20,), generator=g).float())).to(torch.bfloat16).to(DEV)
+    assert torch.equal(run(gate, up).view(torch.int16), (torch.nn.functional.silu(gate) * up).view(torch.int16))
+
+
+@pytest.mark.parametrize("tag", ["MXFP8_E4M3_fn", "OCP_MXFP4_E2M1"])
+def test_operand_from_swiglu_equals_the_two_tensor_operations(mh, tag):
+    """silu(gate) * up formed inside the operand kernel against the same expression as two tensor operations on the GPU
+    (each rounding to bfloat16) followed by the dense operand kernel.  The kernel rounds at the same two places and its SiLU
+    rounds to torch's bfloat16 value for every gate (the test above), so the operands must be equal."""
+    rows, K = 300, 1024
+    t = swiglu_inputs(rows, K, seed=11).to(DEV)
+    gate, up = t[:, :K], t[:, K:]                      # views with row stride 2 K
+    meta = getattr(mh.meta, tag)
+    got = mh.mxk.scaled_operand_from_swiglu(gate, up, meta)
+    h = torch.nn.functional.silu(gate) * up
+    want = mh.mxk.scaled_operand_from_dense(h.contiguous(), meta)
+    cg, sg = operand_arrays(got)
+    cw, sw = operand_arrays(want)
+    assert np.array_equal(sg, sw), "scale bytes"
+    finite = np.repeat(sg != 255, 32, axis=1)     # (which element of an inf / NaN block carries the NaN code is the same too)
+    assert np.array_equal(cg, cw), f"{(cg != cw).sum()} codes differ, {(cg != cw)[finite].sum()} of them in finite blocks"
+    # separate tensors with their own (equal) row stride take the same kernel
+    again = mh.mxk.scaled_operand_from_swiglu(gate.contiguous(), up.contiguous(), meta)
+    ca, sa = operand_arrays(again)
+    assert np.array_equal(ca, cg) and np.array_equal(sa, sg)
+
+
 # ---------------------------------------------------------------- the product
 def quantised(t: torch.Tensor, tag: str):
     E, M = PRESETS[tag]
@@ -178,6 +249,28 @@ def test_scaled_gemm_vs_checker(mh, MNK, x_tag, w_tag):
     assert rel_fro(y32, y_ref) <= F32_TOL
     y16 = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.bfloat16)
     assert rel_fro(y16, y_ref.to(torch.bfloat16)) <= 1e-3
+
+
+@pytest.mark.parametrize("MNK", [(4200, 4808, 512), (2100, 9000, 768), (9000, 520, 512), (257, 65544, 512)])
+def test_scaled_gemm_many_tiles(mh, MNK):
+    """More 256 x 256 tiles than the GPU has compute units, in grids that the workgroups' walk order (patches of 4 x 8
+    tiles per group of 32 workgroups) does not divide: every workgroup walks several tiles as one stream and the last
+    patches are partial.  Every output element against the checker's product."""
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(M ^ N)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    _, _, x_dq = quantised(x, "MXFP8_E4M3_fn")
+    w_sc, w_el, w_dq = quantised(w, "MXFP8_E4M3_fn")
+    y_ref = x_dq.double() @ w_dq.double().t()      # the checker's dequantised operands, float64 product
+    meta = mh.meta.MXFP8_E4M3_fn
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), meta)
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), meta, N, K)
+    y = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.float32).cpu()
+    assert rel_fro(y, y_ref) <= F32_TOL
+    # no element may be far off on its own (a misplaced tile of a large output hides in a Frobenius norm)
+    err = (y.double() - y_ref.double()).abs().view(-1)
+    assert float(err.max()) <= 1e-3 * float(y_ref.double().abs().max())
 
 
 def test_scaled_gemm_bias_and_dtypes(mh):
