@@ -38,7 +38,7 @@ TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_counters_gemm_c4_casts_c1_
 CSRC = os.path.join(ROOT, "mase-triton_amd", "csrc")
 GEMM_SOURCES = ("gemm_tall.h", "gemm_impl.h", "mxfp_compose.h", "mase_device.h")
 SCALED_SOURCES = ("gemm_scaled.h", "gemm_tall.h", "mase_device.h")
-CAST_SOURCES = ("cast_kernels.hip", "mxfp_compose.h", "mase_device.h")
+CAST_SOURCES = ("cast_kernels.hip", "swiglu.h", "mxfp_compose.h", "mase_device.h")
 
 
 def sources_fingerprint(names) -> str:
@@ -558,6 +558,25 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
         w_op = L.scaled_weight_operand(w_sc, w_el, w_tm)
         mxk.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
     del x, w, w_sc, w_el, a, a_op, w_op
+    # C5's kernels on the block-scaled route: gate + up GEMM, SwiGLU operand, down GEMM (after C4's launches of the same kernels)
+    from mase_hip.mxfp.meta import MXFPMeta
+
+    x5, wg, wu, wd = workloads.make_c5()
+    fmt6 = MXFPMeta(32, 8, 3, 2, True, "rn")
+    inter = wg.shape[0]
+    x5 = x5.to(dev).view(-1, x5.shape[-1])
+    ops = []
+    for w5 in (torch.cat([wg, wu]), wd):
+        sc5, el5, tm5 = MXFP_F.extract_mxfp_components(w5.to(dev), block_dim=1, mxfp_meta=fmt6)
+        ops.append(L.scaled_weight_operand(sc5, el5, tm5))
+        del sc5, el5
+    for _ in range(3):
+        t5 = mxk.mxfp_gemm_scaled(mxk.scaled_operand_from_dense(x5, fmt8), ops[0], None, torch.bfloat16)
+    for _ in range(3):
+        a5 = mxk.scaled_operand_from_swiglu(t5[:, :inter], t5[:, inter:], fmt8)
+    for _ in range(3):
+        mxk.mxfp_gemm_scaled(a5, ops[1], None, torch.bfloat16)
+    del x5, t5, a5, ops
     for make, fmt in ((workloads.make_c1, fmt8), (workloads.make_c3, fmt4)):
         t = make().reshape(-1).to(dev)
         for _ in range(3):
@@ -581,11 +600,15 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
 # read, written, sources).  A key is "<kernel row of hbm_kernels> <config>" for the cast rows.
 _N1, _N3, _N2 = 4096 * 4096, 14336 * 4096, 1 << 24
 _M4, _N4, _K4 = 16384, 14336, 4096
+_M5, _H5, _I5 = 8192, 4096, 14336
 COUNTER_ROWS = (
     ("stream_copy_kernel", "calibration copy (256 MiB read, 256 MiB written)", 256 << 20, 256 << 20, None),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C4", (_M4 + _N4) * _K4 * 33 // 32, _M4 * _N4 * 2, SCALED_SOURCES),
     ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", _M4 * _K4 * 2 + _N4 * _K4 * 33 // 32, _M4 * _N4 * 2, GEMM_SOURCES),
-    ("scaled_from_dense_kernel", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
+    ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 gate+up", (_M5 + 2 * _I5) * _H5 * 33 // 32, _M5 * 2 * _I5 * 2, SCALED_SOURCES),
+    ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 down", (_M5 + _H5) * _I5 * 33 // 32, _M5 * _H5 * 2, SCALED_SOURCES),
+    ("scaled_from_dense_kernel|true>(", "scaled_operand_from_swiglu C5", _M5 * _I5 * 4, _M5 * _I5 * 33 // 32, CAST_SOURCES),
+    ("scaled_from_dense_kernel|false>(", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
     ("scaled_operand_kernel", "scaled_operand_from_mxfp C4 W", _N4 * _K4 * 33 // 32, _N4 * _K4 * 33 // 32, CAST_SOURCES),
     ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 0>(", "extract_mxfp C1", _N1 * 2, _N1 + _N1 // 32, CAST_SOURCES),
     ("compose_mxfp_bf16_kernel<mase::SFmt<4, 3", "compose_mxfp C1", _N1 + _N1 // 32, _N1 * 2, CAST_SOURCES),
@@ -601,7 +624,11 @@ COUNTER_ROWS = (
     ("minifloat_f32_kernel<1, mase::SFmt<5, 2", "compose_minifloat C2/E5M2", _N2 * 2, _N2 * 4, CAST_SOURCES),
 )
 # launches of one kernel name at several sizes (the probe also quantises the headline's x and W): the size that is meant, in threads
-_COUNTER_THREADS = {"extract_mxfp C1": _N1 // 16, "extract_mxfp C3": _N3 // 16, "qdq_mxfp_fused C1": _N1 // 16, "qdq_mxfp_fused C3": _N3 // 16}
+_COUNTER_THREADS = {"extract_mxfp C1": _N1 // 16, "extract_mxfp C3": _N3 // 16, "qdq_mxfp_fused C1": _N1 // 16, "qdq_mxfp_fused C3": _N3 // 16,
+                    "scaled_operand_from_dense C4 x": _M4 * _K4 // 16, "scaled_operand_from_mxfp C4 W": _N4 * _K4 // 64}
+# launches of one kernel name at one launch size (the block-scaled GEMM is always one workgroup per compute unit): which of
+# the probe's launches, in dispatch order
+_COUNTER_LAUNCHES = {"mxfp_gemm_scaled_kernel C4": (0, 3), "mxfp_gemm_scaled_kernel C5 gate+up": (3, 6), "mxfp_gemm_scaled_kernel C5 down": (6, 9)}
 
 
 def summarize_counters(fetch_dir, write_dir):
@@ -618,23 +645,29 @@ def summarize_counters(fetch_dir, write_dir):
         if not files:
             raise SystemExit(f"no *counter_collection.csv under {folder}")
         vals = {}
-        for r in csv.DictReader(open(files[0])):
-            if r["Counter_Name"] == counter:   # keyed by kernel name and launch size: the probe also extracts the GEMM's weight
-                vals.setdefault((r["Kernel_Name"], int(r["Grid_Size"])), []).append(float(r["Counter_Value"]))
-        return {k: sum(v) / len(v) for k, v in vals.items()}
+        recs = sorted((r for r in csv.DictReader(open(files[0])) if r["Counter_Name"] == counter), key=lambda r: int(r["Dispatch_Id"]))
+        for r in recs:   # keyed by kernel name and launch size: the probe also extracts the GEMM's weight
+            vals.setdefault((r["Kernel_Name"], int(r["Grid_Size"])), []).append(float(r["Counter_Value"]))
+        return vals
 
     fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
 
-    def pick(table, frag, threads):
+    def pick(table, frag, threads, launches):
         hits = [(k[0], v) for k, v in table.items() if all(part in k[0] for part in frag.split("|")) and (threads is None or k[1] == threads)]
         if len(hits) != 1:
-            raise SystemExit(f"{len(hits)} launches match '{frag}' with {threads} threads: {[k[:80] for k, _ in hits]}")
-        return hits[0]
+            raise SystemExit(f"{len(hits)} kernels match '{frag}' with {threads} threads: {[k[:80] for k, _ in hits]}")
+        name, v = hits[0]
+        if launches is not None:
+            if len(v) < launches[1]:
+                raise SystemExit(f"'{frag}': {len(v)} launches recorded, launches {launches} asked for")
+            v = v[launches[0]:launches[1]]
+        return name, sum(v) / len(v)
 
     rows = []
     for frag, key, rd, wr, sources in COUNTER_ROWS:
         threads = _COUNTER_THREADS.get(key)   # one lane per 2 x 8 elements
-        (name, f_kib), (_, w_kib) = pick(fetch, frag, threads), pick(write, frag, threads)
+        launches = _COUNTER_LAUNCHES.get(key)
+        (name, f_kib), (_, w_kib) = pick(fetch, frag, threads, launches), pick(write, frag, threads, launches)
         rows.append((key, name, f_kib, w_kib, rd, wr, sources))
     cal = rows[0]
     f_fac, w_fac = (cal[4] / 1024) / cal[2], (cal[5] / 1024) / cal[3]
@@ -657,6 +690,12 @@ def summarize_counters(fetch_dir, write_dir):
     print("```json")
     print(json.dumps(table, indent=1))
     print("```")
+
+
+def c5_traffic():
+    """HBM bytes of the block's two GEMM launches together, from the counter summary."""
+    parts = [traffic_bytes(f"mxfp_gemm_scaled_kernel C5 {k}", SCALED_SOURCES) for k in ("gate+up", "down")]
+    return None if None in parts else sum(parts)
 
 
 def bench_c5(torch, with_cpu, steps=20, warmup=8):
@@ -737,7 +776,7 @@ def bench_c5(torch, with_cpu, steps=20, warmup=8):
         "roofline": {"bound": "mfma", "achieved": round(kern_tf, 1), "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kern_tf / MFMA_FP8_PEAK_TFLOPS, 4), "frac_of_bf16_peak": round(kern_tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "kernel": "mxfp_gemm_scaled_kernel", "avg_kernel_ms": {"gate_up": round(gemm_ms[0], 4), "down": round(gemm_ms[1], 4)},
-                     "traffic": None},
+                     "traffic": c5_traffic()},
         "note": "flop = the three GEMMs; ms_per_block = whole block (quantise kernels, GEMMs, SiLU and product; fused: the down layer reads gate and up through forward_swiglu)",
     }
     if with_cpu:

@@ -1045,37 +1045,55 @@ __global__ __launch_bounds__(kThreads) void mxfp_strided_bf16_lines_kernel(const
 }
 
 // MXFP components (reference layout: one code byte per element, scales [rows, K / 32]) -> operand of the block-scaled
-// GEMM.  A workgroup owns 32 rows x 128 k (one line of the transposed scale array): a lane 16 codes, two lanes a block,
-// eight lanes the 128 bytes of a row.  The four scale bytes of a row are one dword on either side.
+// GEMM.  A workgroup owns 32 rows x 512 k (four lines of the transposed scale array, one per 128 k): a lane 16 codes per
+// 128 k, two lanes a block, eight lanes the 128 bytes of a row.  A row's sixteen scale bytes of the 512 k are one 128-bit
+// load (a dword per 128 k where the row ends before that or is not 16-byte aligned there) and four dwords on the way out.
 template <class F>
 __global__ __launch_bounds__(kThreads) void scaled_operand_kernel(const uint8_t* __restrict__ scales, const uint8_t* __restrict__ elements,
                                                                    uint8_t* __restrict__ out_codes, uint32_t* __restrict__ out_scales,
-                                                                   int rows, int K, int nmac, uint32_t rows_pad, F f) {
-    const uint32_t ms = blockIdx.x % (uint32_t)nmac, row = (blockIdx.x / (uint32_t)nmac) * 32u + (threadIdx.x >> 3);
+                                                                   int rows, int K, int nmac, uint32_t rows_pad, bool scales_by_16, F f) {
+    const uint32_t groups = ((uint32_t)nmac + 3u) / 4u;
+    const uint32_t ms0 = (blockIdx.x % groups) * 4u, row = (blockIdx.x / groups) * 32u + (threadIdx.x >> 3);
     const int piece = threadIdx.x & 7;                  // 16 codes of the row's 128
     const bool live = row < (uint32_t)rows;
-    const size_t off = (size_t)row * K + ms * 128u + (uint32_t)piece * 16u;
-    uint4 w = live ? ld128(elements + off) : make_uint4(0, 0, 0, 0);
-    const uint32_t sc4 = live ? *reinterpret_cast<const uint32_t*>(scales + ((size_t)row * (K / 32) + ms * 4u)) : 0u;
-    uint32_t scale = (sc4 >> (8 * (piece >> 1))) & 0xFFu;
-    if constexpr (F{}.E() == 4 && F{}.M() == 3) {
-        uint32_t top = e4m3_top_bits(w.x) | e4m3_top_bits(w.y) | e4m3_top_bits(w.z) | e4m3_top_bits(w.w);
-        top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xF, 0xF, true);  // lane ^ 1
-        if (top != 0u && scale < 254u) {
-            w = make_uint4(e4m3_halve4(w.x), e4m3_halve4(w.y), e4m3_halve4(w.z), e4m3_halve4(w.w));
-            scale += 1u;
-        }
-    } else {
-        w = make_uint4(embed_e4m3_x4(w.x, f), embed_e4m3_x4(w.y, f), embed_e4m3_x4(w.z, f), embed_e4m3_x4(w.w, f));
-    }
-    // the row's four scale bytes (lanes 0, 2, 4, 6 of its 8) into its first lane: row_shl 2, 4, 6
-    uint32_t dw = scale;
-    dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x102, 0xF, 0xF, true) << 8;
-    dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x104, 0xF, 0xF, true) << 16;
-    dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x106, 0xF, 0xF, true) << 24;
+    const size_t off = (size_t)row * K + ms0 * 128u + (uint32_t)piece * 16u;
+    const uint8_t* srow = scales + ((size_t)row * (K / 32) + ms0 * 4u);
+    uint4 w[4];
+    uint32_t sc4[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = live && ms0 + j < (uint32_t)nmac ? ld128(elements + off + j * 128) : make_uint4(0, 0, 0, 0);
     if (live) {
-        st128(out_codes + off, w);
-        if (piece == 0) out_scales[(size_t)ms * rows_pad + row] = dw;
+        if (scales_by_16 && ms0 + 3u < (uint32_t)nmac) {
+            const uint4 v = *reinterpret_cast<const uint4*>(srow);
+            sc4[0] = v.x; sc4[1] = v.y; sc4[2] = v.z; sc4[3] = v.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (ms0 + j < (uint32_t)nmac) sc4[j] = *reinterpret_cast<const uint32_t*>(srow + 4 * j);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t scale = (sc4[j] >> (8 * (piece >> 1))) & 0xFFu;
+        if constexpr (F{}.E() == 4 && F{}.M() == 3) {
+            uint32_t top = e4m3_top_bits(w[j].x) | e4m3_top_bits(w[j].y) | e4m3_top_bits(w[j].z) | e4m3_top_bits(w[j].w);
+            top |= (uint32_t)__builtin_amdgcn_mov_dpp((int)top, 0xB1, 0xF, 0xF, true);  // lane ^ 1
+            if (top != 0u && scale < 254u) {
+                w[j] = make_uint4(e4m3_halve4(w[j].x), e4m3_halve4(w[j].y), e4m3_halve4(w[j].z), e4m3_halve4(w[j].w));
+                scale += 1u;
+            }
+        } else {
+            w[j] = make_uint4(embed_e4m3_x4(w[j].x, f), embed_e4m3_x4(w[j].y, f), embed_e4m3_x4(w[j].z, f), embed_e4m3_x4(w[j].w, f));
+        }
+        // the row's four scale bytes (lanes 0, 2, 4, 6 of its 8) into its first lane: row_shl 2, 4, 6
+        uint32_t dw = scale;
+        dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x102, 0xF, 0xF, true) << 8;
+        dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x104, 0xF, 0xF, true) << 16;
+        dw |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)scale, 0x106, 0xF, 0xF, true) << 24;
+        if (live && ms0 + j < (uint32_t)nmac) {
+            st128(out_codes + off + j * 128, w[j]);
+            if (piece == 0) out_scales[(size_t)(ms0 + j) * rows_pad + row] = dw;
+        }
     }
 }
 
@@ -1430,10 +1448,11 @@ int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elem
     return dispatch_fmt(exp_bits, frac_bits, 1, RN, [&](auto f) {
         if constexpr (decltype(f)::kStatic && decltype(f){}.E() != 5) {
             const int nmac = (int)(K / 128);
-            const int64_t blocks = (rows + 31) / 32 * nmac;
+            const int64_t blocks = (rows + 31) / 32 * ((nmac + 3) / 4);
             if (blocks > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "operand too large for one launch");
+            const bool scales_by_16 = aligned(scales, 16) && (K / 32) % 16 == 0;   // every row's scales of 512 k are one aligned 128-bit word
             hipLaunchKernelGGL((scaled_operand_kernel<decltype(f)>), dim3((unsigned)blocks), dim3(kThreads), 0, s, scales, elements, out_codes,
-                               out_scales, (int)rows, (int)K, nmac, rows_pad, f);
+                               out_scales, (int)rows, (int)K, nmac, rows_pad, scales_by_16, f);
             return check_launch("scaled_operand_from_mxfp");
         }
         return fail(ERR_UNSUPPORTED, "element format not supported by the block-scaled GEMM");

@@ -143,10 +143,10 @@ def test_operand_from_dense_holds_the_reference_values(mh, tag):
         assert np.array_equal(got[finite], ref[finite]), "embedded values"
 
 
+@pytest.mark.parametrize("rows,K", [(260, 768), (300, 1536), (33, 640)])   # scale rows of 24 / 48 / 20 bytes: dword and 128-bit scale loads, ragged ends
 @pytest.mark.parametrize("tag", SCALED_TAGS)
-def test_operand_from_components_equals_from_dense(mh, tag):
+def test_operand_from_components_equals_from_dense(mh, tag, rows, K):
     E, M = PRESETS[tag]
-    rows, K = 260, 768
     x = mixed_inputs(rows, K, seed=3)
     sc, el = oracle.extract_mxfp(x, 32, E, M)
     a = mh.mxk.scaled_operand_from_dense(x.to(DEV), getattr(mh.meta, tag))
