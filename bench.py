@@ -609,7 +609,7 @@ COUNTER_ROWS = (
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 down", (_M5 + _H5) * _I5 * 33 // 32, _M5 * _H5 * 2, SCALED_SOURCES),
     ("scaled_from_dense_kernel|true>(", "scaled_operand_from_swiglu C5", _M5 * _I5 * 4, _M5 * _I5 * 33 // 32, CAST_SOURCES),
     ("scaled_from_dense_kernel|false>(", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
-    ("scaled_operand_kernel", "scaled_operand_from_mxfp C4 W", _N4 * _K4 * 33 // 32, _N4 * _K4 * 33 // 32, CAST_SOURCES),
+    ("scaled_operand_kernel<mase::SFmt<4, 3", "scaled_operand_from_mxfp C4 W", _N4 * _K4 * 33 // 32, _N4 * _K4 * 33 // 32, CAST_SOURCES),
     ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 0>(", "extract_mxfp C1", _N1 * 2, _N1 + _N1 // 32, CAST_SOURCES),
     ("compose_mxfp_bf16_kernel<mase::SFmt<4, 3", "compose_mxfp C1", _N1 + _N1 // 32, _N1 * 2, CAST_SOURCES),
     ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 1>(", "qdq_mxfp_fused C1", _N1 * 2, _N1 * 2, CAST_SOURCES),
