@@ -34,7 +34,7 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0   # MI355X dense fp8, published
 # rocprofv3 --pmc runs of `bench.py --counter-probe` (FETCH_SIZE, then WRITE_SIZE), written by
 # `bench.py --summarize-counters`.  Every entry carries a fingerprint of the kernel sources it was taken with; when the
 # sources have changed since, the figure is reported as null (with a note on stderr) instead of a stale number.
-TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_counters_gemm_c4_casts_c1_c2_c3.md")
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_counters_gemm_c4_c5_casts_c1_c2_c3.md")
 CSRC = os.path.join(ROOT, "mase-triton_amd", "csrc")
 GEMM_SOURCES = ("gemm_tall.h", "gemm_impl.h", "mxfp_compose.h", "mase_device.h")
 SCALED_SOURCES = ("gemm_scaled.h", "gemm_tall.h", "mase_device.h")

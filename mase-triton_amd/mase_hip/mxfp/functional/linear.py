@@ -37,10 +37,11 @@ _GEMM_DTYPES = (torch.bfloat16, torch.float32)
 _BACKENDS = ("separate", "fused", "fused_bf16", "fused_scaled")
 # rows of x from which "fused" takes the block-scaled route.  With the weight operand at hand (a layer keeps it) the
 # block-scaled kernel, K split over workgroups where its 256 x 256 tiles are few, is level with the weight-streaming bf16
-# kernels at 64 rows and ahead from there (N x K = 14336 x 4096: 29 / 33 / 44 us at 64 / 128 / 256 rows against 29 / 37 /
-# 48 us); when the operand has to be built inside the call (N * K bytes read and written) it pays from about 768 rows
+# kernels at 64 rows and ahead from there (N x K = 14336 x 4096: 30 / 33 / 44 / 45 us at 64 / 128 / 256 / 512 rows against
+# 30 / 37 / 49 / 73 us); when the operand has to be built inside the call (N * K bytes read and written, 25 us there) it
+# pays from about 512 rows (71 against 73 us; 72 against 104 at 768)
 SCALED_FROM_ROWS = 64
-SCALED_FROM_ROWS_UNPREPARED = 768
+SCALED_FROM_ROWS_UNPREPARED = 512
 
 
 def parse_mxfp_linear_type(x_meta: MXFPMeta | None, w_tensor_meta: MXFPTensorMeta | None,
