@@ -3,7 +3,7 @@
 // Both operands stay MXFP all the way into the matrix unit: one FP8 (E4M3) code per element and one E8M0 scale per
 // 32 elements along K, which the instruction applies itself.  Nothing is composed to bf16, no operand byte passes
 // through a VGPR on its way to LDS, and an operand row costs one byte per element of LDS and L2 traffic instead of two.
-// The operands come from the prepare kernels (scaled_prepare.hip), which
+// The operands come from the operand kernels (cast_kernels.hip), which
 //   * re-encode every block that holds the code S.1111.111 one scale step up (the instruction reads that code as NaN,
 //     the reference as +-480) and embed the narrower element formats into E4M3 bytes (exact),
 //   * pad the rows to a multiple of 256 and store the scales transposed: dword [K/128][rows], the four bytes of a dword
@@ -365,6 +365,9 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+#include "gemm_scaled_rows.h"   // the weight-streaming kernel for up to 32 rows of A
+
+
 // K split for few tiles and a long K (a [1024, 4096] output has 64 tiles for 256 CUs): the number of walks per tile, chosen so
 // that the walks about fill the CUs; a walk takes an even number of macro steps, at least 4.  Priced like the bf16 kernels'
 // split: macro steps per walk at about 1 us, rounds of walks over the CUs, and for a split the second launch plus the
@@ -372,7 +375,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
 inline int plan_scaled_splits(int M, int N, int K, int cus) {
     const int64_t tiles = (int64_t)((M + SM - 1) / SM) * ((N + SN - 1) / SN);
     const int nmac = K / SMAC;
-    if (tiles * 2 > cus || cus <= 0) return 1;
+    if (tiles * 2 > cus || cus <= 0 || scaled_rows_shape_ok(M, K)) return 1;
     const double mn_mb = (double)M * N * 4.0 / 1e6;
     auto price = [&](int s) {
         const double rounds = (double)((tiles * s + cus - 1) / cus);
@@ -398,6 +401,7 @@ int launch_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const u
     if (tiles >= (1 << 26)) return fail(ERR_UNSUPPORTED, "too many tiles");
     const int cus = device_cu_count();
     if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
+    if (scaled_rows_shape_ok(M, K)) return launch_gemm_scaled_rows<DT_OUT>(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N, K, s);
     int splits = workspace ? plan_scaled_splits(M, N, K, cus) : 1;
     const int64_t mn = (int64_t)M * N;
     if (splits > 1 && workspace_bytes < splits * mn * 4) splits = 1;

@@ -1,0 +1,176 @@
+// Block-scaled MXFP GEMM for a few rows of A (decode-sized calls: M <= 32):  y[M,N] = A[M,K] * W[N,K]^T (+ bias) as a
+// read of W.  Operands in the prepared form of gemm_scaled.h (FP8 bytes [rows_pad, K], scales [K/128][rows_pad] dwords).
+//
+// The product is bound by HBM: W is N * K * 33/32 bytes, read once, against 2 M N K flop.  With the block-scaled
+// instruction a wavefront turns 2 KB of W (16 rows x 128 k) into one MFMA without a single VALU instruction on the
+// codes (the bf16 kernels for this size compose every code to bf16 first and are bound by that), so the kernel is
+// loads and a few MFMAs.  What decides its speed is the shape of the loads: a lane-for-lane load of the instruction's
+// operand layout (16 rows x 64 bytes per load instruction, the rows K bytes apart) reads W at 3.9 TB/s where 1 KB of one
+// row per instruction reaches 6.3 (measured with the bare patterns on 58.7 MB: rows a power of two apart land on the same
+// L2 channel).  So:
+//   * a workgroup owns 16 rows of W over all of K and walks K in chunks of 1 KB per row; a load instruction of a wavefront
+//     is 1 KB of ONE row (wave w: rows 4 w .. 4 w + 3 of W, and of each 16-row tile of A), two chunks ahead in registers;
+//   * the chunk goes through LDS (rows 1040 bytes apart: conflict-free 128-bit writes and fragment reads) and comes
+//     back as operand fragments: lane 16 g + r reads pieces g and g + 4 of row r of a 128-k macro step; wave w multiplies
+//     the chunk's macro steps 2 w and 2 w + 1, its scale dwords straight from global memory (16 rows = 64 contiguous bytes);
+//   * the wavefronts' partial sums meet in LDS at the end.
+// A (16 MB rows, at most a few hundred KB, shared by every workgroup) takes the same route from L2.
+// (included from gemm_impl.h's namespace, after gemm_scaled.h's typedefs)
+
+// the same instruction as mfma_scaled with the accumulator in ordinary registers (a kernel that asks for accumulation
+// registers gets its register budget split in two halves, and this one needs the ordinary half whole); the leading s_nop
+// keeps VALU writes of the scale operands (v_bfe) clear of the matrix instruction's read of them, which the compiler cannot
+// see inside an asm statement
+__device__ inline void mfma_scaled_after_valu(floatx4& c, const intx8& w, const intx8& a, uint32_t sw, uint32_t sa) {
+    asm volatile("s_nop 3\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]" : "+v"(c) : "v"(w), "v"(a), "v"(sw), "v"(sa));
+}
+
+constexpr int SR_CHUNK = 1024;            // bytes of k per row and chunk: 8 macro steps
+constexpr int SR_ROW = SR_CHUNK + 16;     // LDS row pitch
+
+template <int MB>
+struct RowsChunk {
+    intx4 w[4], a[MB][4];                 // this wave's four rows of W and of each A tile: 16 bytes per lane and row
+    uint32_t w_sc[2], a_sc[MB][2];        // scale dwords of the wave's two macro steps (row = lane & 15)
+};
+
+// OCC: wavefronts per SIMD the register budget is set for (workgroups per CU)
+template <int DT_OUT, int MB, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void mxfp_gemm_scaled_rows_kernel(const uint8_t* __restrict__ a_codes, const uint32_t* __restrict__ a_scales,
+                                                                    const uint8_t* __restrict__ w_codes, const uint32_t* __restrict__ w_scales,
+                                                                    const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N,
+                                                                    int K, int rows_a, int rows_w) {
+    __shared__ __attribute__((aligned(16))) uint8_t tile[(16 + 16 * MB) * SR_ROW];   // W rows 0..15, then the A tiles
+    __shared__ float red[3][MB][256];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 4, r = lane & 15;
+    const int n0 = blockIdx.x * 16;
+    const int nmac = K / 128;
+    const int nchunk = (K + SR_CHUNK - 1) / SR_CHUNK;
+
+    // global side: lane l reads bytes 16 l .. 16 l + 15 of a row's chunk (uniform row addresses, a 32-bit lane offset)
+    const uint8_t* const w_src = w_codes + (size_t)(n0 + 4 * wave) * K;
+    const uint8_t* const a_src = a_codes + (size_t)(4 * wave) * K;
+    const uint32_t* const w_sc_src = w_scales + n0;
+    // Every step issues the same loads, whatever its chunk (the compiler can then count exactly which loads a step has to
+    // wait for and leaves the younger chunk in flight): a chunk past the end reads one line, the lanes past the end of a K
+    // that is not a multiple of 1 KB their row's first bytes; what they bring is never multiplied.
+    auto issue = [&](RowsChunk<MB>& c, int chunk) __attribute__((always_inline)) {
+        const bool live = chunk < nchunk;                                   // uniform
+        const uint32_t k = live ? (uint32_t)chunk * SR_CHUNK : 0u;
+        const uint32_t off = live && k + 16u * lane < (uint32_t)K ? k + 16u * lane : 0u;
+        const size_t pitch = live ? (size_t)K : 0;                          // a chunk past the end: one line for the whole wavefront
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            c.w[i] = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(w_src + i * pitch + off));
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) c.a[mb][i] = *reinterpret_cast<const intx4*>(a_src + (16 * mb + i) * pitch + off);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int mac = min(chunk * 8 + 2 * wave + j, nmac - 1);
+            c.w_sc[j] = __builtin_nontemporal_load(w_sc_src + (size_t)mac * rows_w + r);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) c.a_sc[mb][j] = a_scales[(size_t)mac * rows_a + 16 * mb + r];
+        }
+    };
+    // LDS side
+    uint8_t* const st_w = tile + (4 * wave) * SR_ROW + 16 * lane;
+    uint8_t* const st_a = tile + (16 + 4 * wave) * SR_ROW + 16 * lane;
+    const uint8_t* const frag_w = tile + r * SR_ROW + 16 * g;
+    const uint8_t* const frag_a = tile + (16 + r) * SR_ROW + 16 * g;
+
+    floatx4 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto step = [&](RowsChunk<MB>& c, int chunk) __attribute__((always_inline)) {
+        __syncthreads();                                   // the fragment reads of the chunk before are done
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<intx4*>(st_w + i * SR_ROW) = c.w[i];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) *reinterpret_cast<intx4*>(st_a + (16 * mb + i) * SR_ROW) = c.a[mb][i];
+        }
+        uint32_t w_sc[2], a_sc[MB][2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            w_sc[j] = c.w_sc[j];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) a_sc[mb][j] = c.a_sc[mb][j];
+        }
+        issue(c, chunk + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int ms = 2 * wave + j;
+            if (chunk * 8 + ms < nmac) {
+                const intx4 w_lo = *reinterpret_cast<const intx4*>(frag_w + ms * 128), w_hi = *reinterpret_cast<const intx4*>(frag_w + ms * 128 + 64);
+                const intx8 wf = __builtin_shufflevector(w_lo, w_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                const uint32_t sw = (w_sc[j] >> (8 * g)) & 0xFFu;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+                    const uint8_t* fa = frag_a + 16 * mb * SR_ROW + ms * 128;
+                    const intx4 a_lo = *reinterpret_cast<const intx4*>(fa), a_hi = *reinterpret_cast<const intx4*>(fa + 64);
+                    const intx8 af = __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    mfma_scaled_after_valu(acc[mb], wf, af, sw, (a_sc[mb][j] >> (8 * g)) & 0xFFu);
+                }
+            }
+        }
+    };
+
+    RowsChunk<MB> c0, c1;
+    issue(c0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(c1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int chunk = 0; chunk < nchunk; chunk += 2) {      // (an odd count ends with a step that multiplies nothing)
+        step(c0, chunk);
+        step(c1, chunk + 1);
+    }
+    // the matrix unit's last results must have left its pipeline before ordinary instructions read the accumulators
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- add the wavefronts' partial sums (lane l holds n = 4 (l >> 4) + v, m = l & 15 of each 16 x 16 tile) and store
+    if (wave > 0) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) *reinterpret_cast<floatx4*>(&red[wave - 1][mb][lane * 4]) = acc[mb];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int n = n0 + 4 * g;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            floatx4 s = acc[mb];
+#pragma unroll
+            for (int w = 0; w < 3; ++w) s += *reinterpret_cast<const floatx4*>(&red[w][mb][lane * 4]);
+            const int m = 16 * mb + r;
+            if (m < M && n < N) {
+                float out[4] = {s[0], s[1], s[2], s[3]};
+                const int valid = min(4, N - n);
+                if (bias)
+                    for (int t = 0; t < valid; ++t) out[t] += load_bias(bias, bias_dtype, n + t);
+                store_out4<DT_OUT>(y, (int64_t)m * N + n, out, true, valid);
+            }
+        }
+    }
+}
+
+// the shapes this kernel takes: up to 32 rows of A (two 16-row operand tiles)
+inline bool scaled_rows_shape_ok(int M, int K) { return M <= 32 && K >= 128; }
+
+template <int DT_OUT>
+int launch_gemm_scaled_rows(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
+                            int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
+    const int rows_a = (M + 255) / 256 * 256, rows_w = (N + 255) / 256 * 256;
+    const unsigned groups = (unsigned)((N + 15) / 16);
+    if (M <= 16)
+        hipLaunchKernelGGL((mxfp_gemm_scaled_rows_kernel<DT_OUT, 1, 4>), dim3(groups), dim3(256), 0, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y,
+                           M, N, K, rows_a, rows_w);
+    else
+        hipLaunchKernelGGL((mxfp_gemm_scaled_rows_kernel<DT_OUT, 2, 2>), dim3(groups), dim3(256), 0, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y,
+                           M, N, K, rows_a, rows_w);
+    return check_launch("mxfp_gemm_scaled");
+}

@@ -12,7 +12,8 @@ families and picks between them by format and shape:
 * the block-scaled route (``fused_scaled`` forces it): x is quantised straight into FP8 bytes and E8M0 scales, the
   weight components are turned into the same form (once per layer when a layer calls, see ``w_operand``), and the GEMM
   feeds both to the block-scaled matrix instruction, which applies the scales itself.  Taken for quantised x and W in
-  the element formats E4M3 / E3M2 / E2M3 / E2M1, bfloat16 x, K a multiple of 256, from ``SCALED_FROM_ROWS`` rows of x;
+  the element formats E4M3 / E3M2 / E2M3 / E2M1, bfloat16 x, K a multiple of 256, for the row counts of x that
+  ``takes_scaled_route`` names;
 * the bf16 route (``fused_bf16`` forces it): activations go through the single-pass QDQ kernel and the GEMM composes
   the MXFP weight tiles to bf16 in registers on their way to the bf16 matrix instruction.  Every MXFP value has at most
   four significant bits, so bf16 operands are exact.
@@ -42,6 +43,17 @@ _BACKENDS = ("separate", "fused", "fused_bf16", "fused_scaled")
 # pays from about 512 rows (71 against 73 us; 72 against 104 at 768)
 SCALED_FROM_ROWS = 64
 SCALED_FROM_ROWS_UNPREPARED = 512
+# ... and, with the weight operand at hand, the rows of x up to which it takes it as well: decode-sized calls are a read of
+# W, which the block-scaled weight-streaming kernel does without touching the codes (up to 16 rows, one operand tile of x:
+# 17 against 21 us at N x K = 14336 x 4096, 17 against 25 at 4096 x 14336; between 17 and 63 rows the bf16 kernels are ahead)
+SCALED_UP_TO_ROWS = 16
+
+
+def takes_scaled_route(rows: int, prepared: bool) -> bool:
+    """Does backend="fused" take the block-scaled kernels for this many rows of x (given that the operands qualify)?"""
+    if prepared:
+        return rows >= SCALED_FROM_ROWS or 1 <= rows <= SCALED_UP_TO_ROWS
+    return rows >= SCALED_FROM_ROWS_UNPREPARED
 
 
 def parse_mxfp_linear_type(x_meta: MXFPMeta | None, w_tensor_meta: MXFPTensorMeta | None,
@@ -133,7 +145,7 @@ def mxfp_linear(
     # ---- fused
     rows = x.numel() // x.shape[-1] if x.numel() else 0
     if quantised_x and quantised_w and backend != "fused_bf16" and _scaled_eligible(x, x_meta, w_tensor_meta, bias):
-        if backend == "fused_scaled" or rows >= (SCALED_FROM_ROWS if w_operand is not None else SCALED_FROM_ROWS_UNPREPARED):
+        if backend == "fused_scaled" or takes_scaled_route(rows, w_operand is not None):
             out_features, in_features = w_tensor_meta.shape
             assert x.shape[-1] == in_features
             a_op = kernels.scaled_operand_from_dense(x.reshape(-1, in_features), x_meta)

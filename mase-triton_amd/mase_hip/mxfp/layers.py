@@ -122,7 +122,7 @@ class MXFPLinearPTQ(nn.Module):
             return False
         rows = input.numel() // input.shape[-1] if input.numel() else 0
         bias = self.bias if not self.layer_type.endswith("Bq") else None
-        return ((self.backend == "fused_scaled" or rows >= L.SCALED_FROM_ROWS)
+        return ((self.backend == "fused_scaled" or L.takes_scaled_route(rows, True))
                 and L._scaled_eligible(input, self.x_mxfp_meta, self.w_tensor_meta, bias))
 
     def _weight_operand(self, input: Tensor):

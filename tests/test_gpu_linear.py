@@ -515,7 +515,8 @@ def test_config_c4_full_size(mh, backend):
 def test_fused_backend_picks_the_kernel_family_by_rows(mh):
     """backend="fused": the bf16 kernels below the row thresholds (bit-identical to "fused_bf16"), the block-scaled
     kernel from there on (bit-identical to "fused_scaled"); with a prepared weight operand the threshold is the lower
-    one.  Every result within the tolerance of the float64 checker."""
+    one, and decode-sized calls (up to SCALED_UP_TO_ROWS rows) take the block-scaled weight-streaming kernel as well.
+    Every result within the tolerance of the float64 checker."""
     from mase_hip.mxfp.functional import linear as lin
 
     fmt = preset(mh, "MXFP8_E4M3_fn")
@@ -524,14 +525,16 @@ def test_fused_backend_picks_the_kernel_family_by_rows(mh):
     w_sc, w_el, w_tm = mh.F.extract_mxfp_components(w.to(DEV), block_dim=1, mxfp_meta=fmt)
     w_op = lin.scaled_weight_operand(w_sc, w_el, w_tm)
     w_dq = oracle.qdq_mxfp(w, 32, 4, 3)
-    for rows in (lin.SCALED_FROM_ROWS - 8, lin.SCALED_FROM_ROWS, lin.SCALED_FROM_ROWS_UNPREPARED - 8, lin.SCALED_FROM_ROWS_UNPREPARED):
+    for rows in (1, lin.SCALED_UP_TO_ROWS, lin.SCALED_UP_TO_ROWS + 1, lin.SCALED_FROM_ROWS - 8, lin.SCALED_FROM_ROWS, lin.SCALED_FROM_ROWS_UNPREPARED - 8,
+                 lin.SCALED_FROM_ROWS_UNPREPARED):
         x = torch.randn(rows, 512, generator=g).to(torch.bfloat16)
         args = dict(x=x.to(DEV), x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
                     b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
         y_bf16 = mh.F.mxfp_linear(**args, backend="fused_bf16")
         y_scaled = mh.F.mxfp_linear(**args, backend="fused_scaled")
         assert torch.equal(mh.F.mxfp_linear(**args, backend="fused"), y_scaled if rows >= lin.SCALED_FROM_ROWS_UNPREPARED else y_bf16)
-        assert torch.equal(mh.F.mxfp_linear(**args, backend="fused", w_operand=w_op), y_scaled if rows >= lin.SCALED_FROM_ROWS else y_bf16)
+        assert torch.equal(mh.F.mxfp_linear(**args, backend="fused", w_operand=w_op),
+                           y_scaled if rows >= lin.SCALED_FROM_ROWS or rows <= lin.SCALED_UP_TO_ROWS else y_bf16)
         y_ref = oracle.matmul_nt(oracle.qdq_mxfp(x, 32, 4, 3), w_dq).to(torch.bfloat16)
         assert rel_fro(y_bf16, y_ref) <= REL_FRO_TOL
         assert rel_fro(y_scaled, y_ref) <= REL_FRO_TOL
@@ -553,10 +556,10 @@ def test_layer_keeps_and_refreshes_its_weight_operand(mh):
     lin = torch.nn.Linear(512, 264, bias=True, dtype=torch.bfloat16, device=DEV)
     layer = mh.MXFPLinearPTQ.from_linear(lin, fmt, wfmt, None, "XqWqB", "fused")
     sep = mh.MXFPLinearPTQ.from_linear(lin, fmt, wfmt, None, "XqWqB", "separate")
-    small = torch.randn(16, 512, generator=g).to(torch.bfloat16).to(DEV)
+    small = torch.randn(40, 512, generator=g).to(torch.bfloat16).to(DEV)
     big = torch.randn(3, 200, 512, generator=g).to(torch.bfloat16).to(DEV)
     layer(small)
-    assert layer._scaled_w is None              # few rows: the bf16 kernels, nothing cached
+    assert layer._scaled_w is None              # between 17 and 63 rows: the bf16 kernels, nothing cached
     y = layer(big)
     first = layer._scaled_w
     assert first is not None and y.shape == (3, 200, 264)

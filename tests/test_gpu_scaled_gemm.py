@@ -273,6 +273,34 @@ def test_scaled_gemm_many_tiles(mh, MNK):
     assert float(err.max()) <= 1e-3 * float(y_ref.double().abs().max())
 
 
+@pytest.mark.parametrize("MNK", [(1, 4096, 4096), (7, 520, 1024), (16, 14336, 512), (17, 264, 2304), (32, 1032, 14336), (3, 8, 512)])
+@pytest.mark.parametrize("x_tag,w_tag", [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP4_E2M1")])
+def test_scaled_gemm_few_rows(mh, MNK, x_tag, w_tag):
+    """Up to 32 rows of x: the weight-streaming kernel (a workgroup per 16 rows of W, its wavefronts taking the macro steps
+    of K in turn and adding their partial sums through LDS).  Row counts on both sides of its 16-row operand tiles, N that
+    is not a multiple of 16, K with fewer macro steps than a workgroup has wavefronts and with a count they do not divide;
+    bias and every output type."""
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (0.02 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    _, _, x_dq = quantised(x, x_tag)
+    w_sc, w_el, w_dq = quantised(w, w_tag)
+    y_ref = x_dq.double() @ w_dq.double().t()
+    a = mh.mxk.scaled_operand_from_dense(x.to(DEV), getattr(mh.meta, x_tag))
+    wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), getattr(mh.meta, w_tag), N, K)
+    y32 = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.float32)
+    assert y32.shape == (M, N)
+    assert rel_fro(y32, y_ref) <= F32_TOL
+    err = (y32.cpu().double() - y_ref).abs().max()
+    assert float(err) <= 1e-3 * float(y_ref.abs().max())
+    y_b = y_ref + b.double()
+    for odt in (torch.bfloat16, torch.float16):
+        y16 = mh.mxk.mxfp_gemm_scaled(a, wop, b.to(DEV), odt)
+        assert y16.dtype == odt and rel_fro(y16, y_b.to(odt)) <= 1e-3
+
+
 def test_scaled_gemm_bias_and_dtypes(mh):
     M, N, K = 300, 264, 512
     g = torch.Generator().manual_seed(5)
