@@ -281,7 +281,8 @@ int mase_hip_mxfp_gemm_static_ws(const void* a_dense, int a_dtype, const uint8_t
  *       y[M,N] = A[M,K] * W[N,K]^T (+ bias), A and W prepared as above with rows M and N.
  *
  * K % 256 == 0 and K >= 512; N a multiple of 8 (4 for fp32 output); codes and y 16-byte aligned.  Other shapes: -2,
- * use mase_hip_mxfp_gemm.
+ * use mase_hip_mxfp_gemm.  Up to 32 rows of A take a weight-streaming kernel (the product is a read of W), more rows
+ * 256 x 256 tiles.
  * Replaces, like mase_hip_mxfp_gemm, the unimplemented backend="fused" of mxfp_linear_XqWq
  *   src/mase_triton/mxfp/functional/linear.py:36-64
  * (extract of x :50-52, the two composes :53-54 and the linear :61 in one prepare call and one GEMM).
