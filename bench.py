@@ -39,6 +39,7 @@ CSRC = os.path.join(ROOT, "mase-triton_amd", "csrc")
 GEMM_SOURCES = ("gemm_tall.h", "gemm_impl.h", "mxfp_compose.h", "mase_device.h")
 SCALED_SOURCES = ("gemm_scaled.h", "gemm_tall.h", "mase_device.h")
 CAST_SOURCES = ("cast_kernels.hip", "swiglu.h", "mxfp_compose.h", "mase_device.h")
+ROWS_SOURCES = ("gemm_scaled_rows.h", "mase_device.h")
 
 
 def sources_fingerprint(names) -> str:
@@ -364,14 +365,14 @@ def bench_hbm(torch, with_cpu):
             copy_cache[half] = round(best, 1)
         return copy_cache[half]
 
-    def roof(name, cfg, workload, bytes_per_launch, avg_ms, best_ms, cached_ms):
+    def roof(name, cfg, workload, bytes_per_launch, avg_ms, best_ms, cached_ms, sources=CAST_SOURCES):
         gbs = bytes_per_launch / (avg_ms * 1e-3) / 1e9
         copy = tuned_copy_gbps(bytes_per_launch)
         out.append({
             "kernel": name, "workload": workload, "bytes_per_launch": bytes_per_launch,
             "avg_ms": round(avg_ms, 5), "best_ms": round(best_ms, 5),
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic_bytes(f"{name} {cfg}", CAST_SOURCES)},
+                         "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic_bytes(f"{name} {cfg}", sources)},
             "cache_resident_GBps": round(bytes_per_launch / (cached_ms * 1e-3) / 1e9, 1),
             "tuned_copy_same_bytes_GBps": copy, "frac_of_tuned_copy": round(gbs / copy, 3),
             "cpu_baseline": cpu.get((name, cfg)),
@@ -441,6 +442,37 @@ def bench_hbm(torch, with_cpu):
             avg, best = time_kernel(torch, fn, len(xs))
             cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
             roof(name, f"C2/E{e}M{m}", wl, nbytes, avg, best, cavg)
+    del xs, ys, cs
+
+    # Decode-sized mxfp_linear is a read of W: C4's weight against the first 16 rows of C4's x, both as the operands a layer
+    # keeps / builds, on the block-scaled weight-streaming kernel; the weight rotates through seven copies (424 MB) so that
+    # none of it is served from the 256 MB memory-side cache.  The bf16 weight-streaming kernel on the same data beside it.
+    from mase_hip.mxfp import kernels
+    from mase_hip.mxfp.meta import MXFP8_E4M3_fn
+
+    x_cpu, w_cpu = workloads.make_c4()
+    N, K = w_cpu.shape
+    x16 = x_cpu[:16].contiguous().to(dev)
+    w_sc, w_el = kernels.extract_mxfp_components(w_cpu.to(dev).reshape(-1), MXFP8_E4M3_fn)
+    del x_cpu, w_cpu
+    comps = [(w_sc, w_el)] + [(w_sc.clone(), w_el.clone()) for _ in range(6)]
+    wops = [kernels.scaled_operand_from_mxfp(sc, el, MXFP8_E4M3_fn, N, K) for sc, el in comps]
+    a_op = kernels.scaled_operand_from_dense(x16, MXFP8_E4M3_fn)
+    a_dq = kernels.quantize_dequantize(x16.view(-1), MXFP8_E4M3_fn, torch.bfloat16).view(16, K)
+    y16 = torch.empty(16, N, dtype=torch.bfloat16, device=dev)
+
+    def rows_gemm(i):
+        kernels.mxfp_gemm_scaled(a_op, wops[i], None, torch.bfloat16, out=y16)
+
+    def rows_gemm_bf16(i):
+        kernels.mxfp_gemm(a_dq, None, None, None, comps[i][0], comps[i][1], MXFP8_E4M3_fn, None, 16, N, K, torch.bfloat16, out=y16)
+
+    w_bytes = N * K * (1 + 1 / 32)
+    for name, fn in (("mxfp_gemm_scaled_rows", rows_gemm), ("mxfp_gemm_skinny (bf16)", rows_gemm_bf16)):
+        avg, best = time_kernel(torch, fn, len(wops))
+        cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
+        roof(name, "C4 W x 16 rows", f"decode: 16 rows of C4's x against W [{N},{K}] MXFP8 E4M3, bf16 out (bytes = W's codes and scales)", w_bytes, avg, best, cavg,
+             ROWS_SOURCES if fn is rows_gemm else GEMM_SOURCES)
     return out
 
 
@@ -557,7 +589,10 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
         a_op = mxk.scaled_operand_from_dense(x, fmt8)
         w_op = L.scaled_weight_operand(w_sc, w_el, w_tm)
         mxk.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
-    del x, w, w_sc, w_el, a, a_op, w_op
+    a16 = mxk.scaled_operand_from_dense(x[:16].contiguous(), fmt8)
+    for _ in range(3):
+        mxk.mxfp_gemm_scaled(a16, w_op, None, torch.bfloat16)          # decode-sized: the weight-streaming kernel
+    del x, w, w_sc, w_el, a, a_op, w_op, a16
     # C5's kernels on the block-scaled route: gate + up GEMM, SwiGLU operand, down GEMM (after C4's launches of the same kernels)
     from mase_hip.mxfp.meta import MXFPMeta
 
@@ -604,6 +639,7 @@ _M5, _H5, _I5 = 8192, 4096, 14336
 COUNTER_ROWS = (
     ("stream_copy_kernel", "calibration copy (256 MiB read, 256 MiB written)", 256 << 20, 256 << 20, None),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C4", (_M4 + _N4) * _K4 * 33 // 32, _M4 * _N4 * 2, SCALED_SOURCES),
+    ("mxfp_gemm_scaled_rows_kernel", "mxfp_gemm_scaled_rows C4 W x 16 rows", _N4 * _K4 * 33 // 32 + 16 * _K4 * 33 // 32, 16 * _N4 * 2, ROWS_SOURCES),
     ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", _M4 * _K4 * 2 + _N4 * _K4 * 33 // 32, _M4 * _N4 * 2, GEMM_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 gate+up", (_M5 + 2 * _I5) * _H5 * 33 // 32, _M5 * 2 * _I5 * 2, SCALED_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 down", (_M5 + _H5) * _I5 * 33 // 32, _M5 * _H5 * 2, SCALED_SOURCES),
