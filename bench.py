@@ -559,7 +559,65 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
     }
     cast["extract_in_place_GBps"] = round(n * (3 + 1 / 32) / cast["extract_in_place_us"] / 1e3, 0)
     cast["qdq_in_place_GBps"] = round(n * 4 / cast["qdq_in_place_us"] / 1e3, 0)
-    return {"linear_N14336_K4096": rows, "linear_N4096_K14336": rows_down, "linear_N4096_K4096": rows_sq, "casts_along_axis0": cast}
+    return {"linear_N14336_K4096": rows, "linear_N4096_K14336": rows_down, "linear_N4096_K4096": rows_sq, "casts_along_axis0": cast,
+            "casts_over_size": casts_over_size(torch, fmt)}
+
+
+def casts_over_size(torch, fmt):
+    """The MXFP casts of configuration C1 (bf16, E4M3, block 32) and the tuned streaming copy at 1, 2, 4 and 8 times C1's
+    16.8 M elements: kernel time per launch (HIP graph of 48 launches over rotating buffers, as in the benchmark), and a
+    least-squares line  t = t0 + bytes / bandwidth  through the four points of each kernel.  t0 is what a launch costs
+    whatever its size (ramp and tail); the slope is the rate the kernel sustains."""
+    import workloads
+    from mase_hip import _lib
+
+    dev = "cuda:0"
+    lib = _lib.load()
+    blib = load_bench_lib()
+    sp = lambda: _lib.stream_ptr(torch.device(dev))
+    e, m = fmt.element_exp_bits, fmt.element_frac_bits
+    base = workloads.make_c1().reshape(-1).to(dev)
+    points = {k: [] for k in ("extract_mxfp", "compose_mxfp", "qdq_mxfp_fused", "tuned_copy (bytes of extract)")}
+    for mult in (1, 2, 4, 8):
+        x0 = base.repeat(mult)
+        n = x0.numel()
+        copies = max(2, int((400 << 20) // (3 * n)) + 1)
+        xs = [x0] + [x0.clone() for _ in range(copies - 1)]
+        scs = [torch.empty(n // 32, dtype=torch.uint8, device=dev) for _ in xs]
+        els = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in xs]
+        ys = [torch.empty_like(x) for x in xs]
+
+        def ext(i):
+            _lib.check(lib.mase_hip_extract_mxfp(xs[i].data_ptr(), 2, scs[i].data_ptr(), els[i].data_ptr(), n, 32, e, m, 1, 0, sp()))
+
+        def cmp(i):
+            _lib.check(lib.mase_hip_compose_mxfp(scs[i].data_ptr(), els[i].data_ptr(), ys[i].data_ptr(), 2, n, 32, e, m, 1, sp()))
+
+        def qdq(i):
+            _lib.check(lib.mase_hip_qdq_mxfp(xs[i].data_ptr(), 2, ys[i].data_ptr(), 2, n, 32, e, m, 1, 0, sp()))
+
+        half = int(n * (3 + 1 / 32) / 2) // 16 * 16
+        src = [x.view(torch.uint8)[:half] for x in xs]
+        dst = [y.view(torch.uint8)[:half] for y in ys]
+
+        def cp(i):
+            assert blib.mase_bench_stream_copy(src[i].data_ptr(), dst[i].data_ptr(), half, 1, sp()) == 0
+
+        for i in range(copies):
+            ext(i)
+        for name, fn, nbytes in (("extract_mxfp", ext, n * (3 + 1 / 32)), ("compose_mxfp", cmp, n * (3 + 1 / 32)), ("qdq_mxfp_fused", qdq, n * 4.0),
+                                 ("tuned_copy (bytes of extract)", cp, 2.0 * half)):
+            avg, _ = time_kernel(torch, fn, copies)
+            points[name].append({"elements": n, "bytes": int(nbytes), "us": round(avg * 1e3, 2), "GBps": round(nbytes / (avg * 1e-3) / 1e9, 0)})
+        del xs, scs, els, ys, src, dst, x0
+    out = {}
+    for name, pts in points.items():
+        bx, ty = [p["bytes"] for p in pts], [p["us"] for p in pts]
+        k = len(pts)
+        mx, my = sum(bx) / k, sum(ty) / k
+        slope = sum((a - mx) * (b - my) for a, b in zip(bx, ty)) / sum((a - mx) ** 2 for a in bx)      # us per byte
+        out[name] = {"points": pts, "fit": {"t0_us": round(my - slope * mx, 2), "sustained_GBps": round(1e-3 / slope, 0)}}
+    return out
 
 
 def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
