@@ -301,6 +301,34 @@ def test_scaled_gemm_few_rows(mh, MNK, x_tag, w_tag):
         assert y16.dtype == odt and rel_fro(y16, y_b.to(odt)) <= 1e-3
 
 
+def test_scaled_gemm_random_shapes(mh):
+    """A seeded sweep over shapes on every route of the entry point (decode-sized kernel, lone tiles, K split, several
+    tiles per workgroup): M 1 .. 700, N a multiple of 8 up to 1040, K a multiple of 256 up to 3072, format pairs in turn;
+    every element of the fp32 result against a float64 product of the checker's dequantised operands."""
+    import random
+
+    rng = random.Random(1234)
+    pairs = [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP6_E3M2"), ("OCP_MXFP6_E2M3", "OCP_MXFP4_E2M1")]
+    for case in range(24):
+        M = rng.choice([rng.randint(1, 32), rng.randint(33, 300), rng.randint(301, 700)])
+        N = 8 * rng.randint(1, 130)
+        K = 256 * rng.randint(2, 12)
+        x_tag, w_tag = pairs[case % len(pairs)]
+        g = torch.Generator().manual_seed(case)
+        x = (torch.randn(M, K, generator=g) * torch.exp2(torch.randint(-6, 6, (M, 1), generator=g).float())).to(torch.bfloat16)
+        w = (0.05 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+        b = torch.randn(N, generator=g)
+        _, _, x_dq = quantised(x, x_tag)
+        w_sc, w_el, w_dq = quantised(w, w_tag)
+        y_ref = x_dq.double() @ w_dq.double().t() + b.double()
+        a = mh.mxk.scaled_operand_from_dense(x.to(DEV), getattr(mh.meta, x_tag))
+        wop = mh.mxk.scaled_operand_from_mxfp(w_sc.to(DEV), w_el.to(DEV), getattr(mh.meta, w_tag), N, K)
+        y = mh.mxk.mxfp_gemm_scaled(a, wop, b.to(DEV), torch.float32).cpu().double()
+        assert y.shape == (M, N), (M, N, K)
+        assert rel_fro(y, y_ref) <= F32_TOL, (M, N, K)
+        assert float((y - y_ref).abs().max()) <= 1e-3 * float(y_ref.abs().max()), (M, N, K)
+
+
 def test_scaled_gemm_bias_and_dtypes(mh):
     M, N, K = 300, 264, 512
     g = torch.Generator().manual_seed(5)
