@@ -697,7 +697,7 @@ _M5, _H5, _I5 = 8192, 4096, 14336
 COUNTER_ROWS = (
     ("stream_copy_kernel", "calibration copy (256 MiB read, 256 MiB written)", 256 << 20, 256 << 20, None),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C4", (_M4 + _N4) * _K4 * 33 // 32, _M4 * _N4 * 2, SCALED_SOURCES),
-    ("mxfp_gemm_scaled_rows_kernel", "mxfp_gemm_scaled_rows C4 W x 16 rows", _N4 * _K4 * 33 // 32 + 16 * _K4 * 33 // 32, 16 * _N4 * 2, ROWS_SOURCES),
+    ("mxfp_gemm_scaled_rows_resident_kernel", "mxfp_gemm_scaled_rows C4 W x 16 rows", _N4 * _K4 * 33 // 32 + 16 * _K4 * 33 // 32, 16 * _N4 * 2, ROWS_SOURCES),
     ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", _M4 * _K4 * 2 + _N4 * _K4 * 33 // 32, _M4 * _N4 * 2, GEMM_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 gate+up", (_M5 + 2 * _I5) * _H5 * 33 // 32, _M5 * 2 * _I5 * 2, SCALED_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 down", (_M5 + _H5) * _I5 * 33 // 32, _M5 * _H5 * 2, SCALED_SOURCES),

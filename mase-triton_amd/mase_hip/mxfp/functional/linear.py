@@ -45,7 +45,7 @@ SCALED_FROM_ROWS = 64
 SCALED_FROM_ROWS_UNPREPARED = 512
 # ... and, with the weight operand at hand, the rows of x up to which it takes it as well: decode-sized calls are a read of
 # W, which the block-scaled weight-streaming kernel does without touching the codes (up to 16 rows, one operand tile of x:
-# 17 against 21 us at N x K = 14336 x 4096, 17 against 25 at 4096 x 14336; between 17 and 63 rows the bf16 kernels are ahead)
+# 15 against 21 us at N x K = 14336 x 4096, 17 against 25 at 4096 x 14336; between 17 and 63 rows the bf16 kernels are ahead)
 SCALED_UP_TO_ROWS = 16
 
 
