@@ -8,7 +8,9 @@ backend="fused" (NotImplementedError in the reference, :21-22) quantises ``other
 along its second-to-last axis (no transposed copy).  When ``other`` is quantised it stays in MXFP
 form: its codes come out as [.., N, K], the layout the GEMM kernels read, and all leading batch
 axes (broadcast ones included) go into ONE batched GEMM launch that composes the codes to bf16
-on their way to the MFMA units.  Everything else goes through the one-pass quantise-dequantise
+on their way to the MFMA units.  A product of two quantised bfloat16 operands against ONE matrix
+(``other`` without batch axes) with enough rows takes the block-scaled FP8 matrix instruction instead, as
+``mxfp_linear`` does (functional/linear.py).  Everything else goes through the one-pass quantise-dequantise
 kernels and ``torch.matmul``.
 """
 from __future__ import annotations
@@ -82,7 +84,30 @@ def gemm_over_batches(a: Tensor, w_scales: Tensor, w_elements: Tensor, w_meta: M
     return y.view(*batch, M, N)
 
 
+def _scaled_route(input: Tensor, other: Tensor, input_meta: MXFPMeta | None, other_meta: MXFPMeta) -> bool:
+    """Both operands quantised, bfloat16, one weight matrix, formats and shape the block-scaled GEMM takes, and enough rows
+    to pay for turning ``other``'s codes into its operand form inside the call."""
+    from . import linear as L
+
+    if input_meta is None or input.dtype != torch.bfloat16 or _prod(other.shape[:-2]) != 1:
+        return False
+    if not (kernels.scaled_format_supported(input_meta) and kernels.scaled_format_supported(other_meta)):
+        return False
+    if input_meta.round_mode != "rn" or other_meta.round_mode != "rn":
+        return False
+    K, N = other.shape[-2], other.shape[-1]
+    return kernels.scaled_shape_supported(N, K, input.dtype) and L.takes_scaled_route(input.numel() // K, False)
+
+
 def _matmul_through_gemm(input: Tensor, other: Tensor, input_meta: MXFPMeta | None, other_meta: MXFPMeta) -> Tensor:
+    if _scaled_route(input, other, input_meta, other_meta):
+        K, N = other.shape[-2], other.shape[-1]
+        w_scales, w_elements = kernels.extract_mxfp_components_strided(other.reshape(K, N), -2, other_meta)   # [N, K] order
+        w_op = kernels.scaled_operand_from_mxfp(w_scales, w_elements, other_meta, N, K)
+        a_op = kernels.scaled_operand_from_dense(input.reshape(-1, K), input_meta)
+        y = kernels.mxfp_gemm_scaled(a_op, w_op, None, input.dtype)
+        lead = torch.broadcast_shapes(tuple(input.shape[:-2]), tuple(other.shape[:-2]))
+        return y.view(*lead, input.shape[-2], N)
     a = input
     if input_meta is not None:
         # MXFP values are exact in bf16 whatever input.dtype is

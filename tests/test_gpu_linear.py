@@ -692,6 +692,37 @@ def test_forward_swiglu_is_the_expression(mh):
     assert torch.equal(sep.forward_swiglu(part[:, :inter], part[:, inter:]), sep(torch.nn.functional.silu(part[:, :inter]) * part[:, inter:]))
 
 
+def test_mxfp_matmul_one_matrix_takes_the_block_scaled_route(mh):
+    """mxfp_matmul(XqWq, fused) of bfloat16 operands against ONE matrix with enough rows: the block-scaled GEMM, as in
+    mxfp_linear.  Bit-identical to the same three kernels called by hand, within 1e-3 of backend="separate" and of a float64
+    product of the checker's dequantised operands; with fewer rows, or batched `other`, the bf16 route as before."""
+    from mase_hip.mxfp.functional import linear as lin
+
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    g = torch.Generator().manual_seed(8)
+    K, N = 1024, 520
+    a = torch.randn(2, 300, K, generator=g).to(torch.bfloat16)
+    b = (0.05 * torch.randn(K, N, generator=g)).to(torch.bfloat16)
+    assert 2 * 300 >= lin.SCALED_FROM_ROWS_UNPREPARED
+    ad, bd = a.to(DEV), b.to(DEV)
+    y = mh.F.mxfp_matmul(ad, bd, fmt, fmt, "XqWq", "fused")
+    assert y.shape == (2, 300, N)
+    w_sc, w_el = mh.mxk.extract_mxfp_components_strided(bd, -2, fmt)
+    by_hand = mh.mxk.mxfp_gemm_scaled(mh.mxk.scaled_operand_from_dense(ad.reshape(-1, K), fmt),
+                                      mh.mxk.scaled_operand_from_mxfp(w_sc, w_el, fmt, N, K), None, torch.bfloat16)
+    assert torch.equal(y.view(-1, N), by_hand)
+    assert rel_fro(y, mh.F.mxfp_matmul(ad, bd, fmt, fmt, "XqWq", "separate")) <= REL_FRO_TOL
+    a_dq = oracle.qdq_mxfp(a.view(-1, K), 32, 4, 3)
+    b_dq = oracle.qdq_mxfp(b.t().contiguous(), 32, 4, 3)            # blocks along K: rows of b^T
+    y_ref = (a_dq.double() @ b_dq.double().t()).to(torch.bfloat16)
+    assert rel_fro(y.view(-1, N), y_ref) <= REL_FRO_TOL
+    # `other` with batch axes of one is the same matrix
+    assert torch.equal(mh.F.mxfp_matmul(ad, bd.view(1, K, N), fmt, fmt, "XqWq", "fused"), y)
+    # few rows: the bf16 kernels (another summation order: equal within the tolerance, not bit for bit required)
+    few = ad[0, :64]
+    assert rel_fro(mh.F.mxfp_matmul(few, bd, fmt, fmt, "XqWq", "fused"), mh.F.mxfp_matmul(few, bd, fmt, fmt, "XqWq", "separate")) <= REL_FRO_TOL
+
+
 @pytest.mark.parametrize("func_type", ["XW", "XqW", "XWq", "XqWq"])
 @pytest.mark.parametrize("backend", ["separate", "fused"])
 def test_mxfp_matmul(mh, func_type, backend):
