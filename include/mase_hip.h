@@ -294,6 +294,19 @@ int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elem
                                       int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
                                       uint32_t* out_scales, void* stream);
 /*
+ * The activations of a minifloat linear layer as an operand of the same GEMM: every element of the row-major [rows, K]
+ * bfloat16 matrix x is rounded by itself to the minifloat format (E, M) (finite, round to nearest: the codes of
+ * mase_hip_extract_minifloat, one byte each) and every block carries the scale 2^0, under which a minifloat code is an
+ * MXFP element of the same value.  The weight codes of such a layer go through mase_hip_scaled_operand_from_mxfp with
+ * scale bytes of 127.  Formats and the E4M3 re-encoding as above.
+ * Replaces, with mase_hip_mxfp_gemm_scaled, the unimplemented backend="fused" of minifloat_linear_XqWq
+ *   src/mase_triton/minifloat/functional/linear.py:33-58
+ * (extract and compose of x :45-46, compose of W :47 and the linear :55 in one prepare call and one GEMM).
+ */
+int mase_hip_scaled_operand_from_dense_minifloat(const void* x, int x_dtype, int exp_bits, int frac_bits,
+                                                 int64_t rows, int64_t K, uint8_t* out_codes,
+                                                 uint32_t* out_scales, void* stream);
+/*
  * The activations of the down projection of a SwiGLU block, quantised where they are formed: the matrix that is
  * extracted is silu(gate) * up (gate, up: row-major [rows, K] bfloat16 with a common row stride of `row_stride`
  * elements, e.g. the two halves of a stacked gate / up projection's output, row_stride = 2 K), each of the two

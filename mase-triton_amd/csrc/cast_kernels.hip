@@ -599,12 +599,16 @@ __global__ __launch_bounds__(kThreads) void mxfp_bf16_b32_kernel(const uint4* __
 // re-encoding / embedding above).  A workgroup owns 32 rows x 128 k, the unit whose scale dwords fill one 128-byte line of
 // the transposed scale array: 16 lanes read the 256 bytes of one row (8 elements each, four lanes to a block), a
 // wavefront four rows per step, two steps.  The four scale bytes of a row are gathered into one lane and stored as a dword.
-// SWIGLU: the matrix that is quantised is silu(x) * up (up [rows, K] with the same row stride), formed in registers.
-template <class F, bool SWIGLU>
+// MODE 1 (SwiGLU): the matrix that is quantised is silu(x) * up (up [rows, K] with the same row stride), formed in registers.
+// MODE 2 (minifloat): every element is rounded by itself to the minifloat format F (what extract_minifloat_kernel computes)
+// and every block carries the scale 2^0: a minifloat code is the MXFP element of a block with that scale.
+enum { FROM_DENSE = 0, FROM_SWIGLU = 1, FROM_DENSE_MINIFLOAT = 2 };
+template <class F, int MODE>
 __global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ up, size_t ld,
                                                                       uint8_t* __restrict__ codes, uint32_t* __restrict__ scales, int rows,
                                                                       int K, int nmac, uint32_t rows_pad, F f) {
-    __shared__ __attribute__((aligned(16))) uint8_t lut[LdsLut<F, false>::BYTES];
+    constexpr bool SWIGLU = MODE == FROM_SWIGLU, MINIFLOAT = MODE == FROM_DENSE_MINIFLOAT;
+    __shared__ __attribute__((aligned(16))) uint8_t lut[LdsLut<F, MINIFLOAT>::BYTES];   // (no table for the per-element rounding)
     const uint32_t ms = blockIdx.x % (uint32_t)nmac, row_base = (blockIdx.x / (uint32_t)nmac) * 32u;
     const int t = threadIdx.x;
     uint4 raw[2], raw_up[2];
@@ -619,13 +623,29 @@ __global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint1
         raw[r] = live[r] ? ld128(x + (size_t)row * ld + col) : make_uint4(0, 0, 0, 0);
         if (SWIGLU) raw_up[r] = live[r] ? ld128(up + (size_t)row * ld + col) : make_uint4(0, 0, 0, 0);
     }
-    LdsLut<F, false>::fill(lut);
+    LdsLut<F, MINIFLOAT>::fill(lut);
     const uint32_t lut_addr = (uint32_t)(uintptr_t)lut;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
         if (SWIGLU) raw[r] = swiglu_x8(raw[r], raw_up[r]);
         uint32_t o[4], scale;
-        bf16_block_step<F, false>(raw[r], f, o, scale, lut_addr);
+        if constexpr (MINIFLOAT) {
+            const uint32_t h[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
+            // inf / NaN anywhere in the wavefront's elements: the per-element routine for all of them
+            bool special = false;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) special |= (h[j] & 0x7F80u) == 0x7F80u || (h[j] & 0x7F800000u) == 0x7F800000u;
+            if (__builtin_amdgcn_ballot_w64(special) == 0) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o[j] = encode_f32_finite_rn(h[j] << 16, f) | (encode_f32_finite_rn(h[j] & 0xFFFF0000u, f) << 16);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o[j] = encode_f32_bits(h[j] << 16, f) | (encode_f32_bits(h[j] & 0xFFFF0000u, f) << 16);
+            }
+            scale = 127u;
+        } else {
+            bf16_block_step<F, false>(raw[r], f, o, scale, lut_addr);
+        }
         uint32_t w0 = __builtin_amdgcn_perm(o[1], o[0], 0x06040200u), w1 = __builtin_amdgcn_perm(o[3], o[2], 0x06040200u);
         if constexpr (F{}.E() == 4 && F{}.M() == 3) {
             uint32_t top = e4m3_top_bits(w0) | e4m3_top_bits(w1);
@@ -1465,7 +1485,7 @@ int mase_hip_scaled_operand_from_mxfp(const uint8_t* scales, const uint8_t* elem
 }
 
 static int scaled_from_dense_entry(const void* x, const void* up, int64_t ld, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K,
-                                   uint8_t* out_codes, uint32_t* out_scales, void* stream) {
+                                   uint8_t* out_codes, uint32_t* out_scales, void* stream, bool minifloat = false) {
     uint32_t rows_pad;
     if (int rc = scaled_operand_args(rows, K, exp_bits, frac_bits, rows_pad)) return rc;
     if (x_dtype != BF16) return fail(ERR_UNSUPPORTED, "a dense operand of the block-scaled GEMM must be bfloat16");
@@ -1480,11 +1500,14 @@ static int scaled_from_dense_entry(const void* x, const void* up, int64_t ld, in
             const int64_t blocks = (rows + 31) / 32 * nmac;
             if (blocks > 0x7FFFFFFFll) return fail(ERR_UNSUPPORTED, "operand too large for one launch");
             const uint16_t *xp = static_cast<const uint16_t*>(x), *upp = static_cast<const uint16_t*>(up);
-            if (up)
-                hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f), true>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp, upp, (size_t)ld,
+            if (minifloat)
+                hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f), FROM_DENSE_MINIFLOAT>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp, upp,
+                                   (size_t)ld, out_codes, out_scales, (int)rows, (int)K, nmac, rows_pad, f);
+            else if (up)
+                hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f), FROM_SWIGLU>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp, upp, (size_t)ld,
                                    out_codes, out_scales, (int)rows, (int)K, nmac, rows_pad, f);
             else
-                hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f), false>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp, upp, (size_t)ld,
+                hipLaunchKernelGGL((scaled_from_dense_kernel<decltype(f), FROM_DENSE>), dim3((unsigned)blocks), dim3(kThreads), 0, s, xp, upp, (size_t)ld,
                                    out_codes, out_scales, (int)rows, (int)K, nmac, rows_pad, f);
             return check_launch("scaled_operand_from_dense");
         }
@@ -1495,6 +1518,11 @@ static int scaled_from_dense_entry(const void* x, const void* up, int64_t ld, in
 int mase_hip_scaled_operand_from_dense(const void* x, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K, uint8_t* out_codes,
                                        uint32_t* out_scales, void* stream) {
     return scaled_from_dense_entry(x, nullptr, K, x_dtype, exp_bits, frac_bits, rows, K, out_codes, out_scales, stream);
+}
+
+int mase_hip_scaled_operand_from_dense_minifloat(const void* x, int x_dtype, int exp_bits, int frac_bits, int64_t rows, int64_t K,
+                                                 uint8_t* out_codes, uint32_t* out_scales, void* stream) {
+    return scaled_from_dense_entry(x, nullptr, K, x_dtype, exp_bits, frac_bits, rows, K, out_codes, out_scales, stream, true);
 }
 
 int mase_hip_scaled_operand_from_swiglu(const void* gate, const void* up, int dtype, int64_t row_stride, int exp_bits, int frac_bits, int64_t rows,

@@ -38,6 +38,7 @@ SIGNATURES = {
                                             _vp, _i32, _i64, _i64, _i64, _i32, _vp]),
     "mase_hip_scaled_padded_rows": (_i64, [_i64]),
     "mase_hip_scaled_operand_from_dense": (_i32, [_vp, _i32, _i32, _i32, _i64, _i64, _vp, _vp, _vp]),
+    "mase_hip_scaled_operand_from_dense_minifloat": (_i32, [_vp, _i32, _i32, _i32, _i64, _i64, _vp, _vp, _vp]),
     "mase_hip_scaled_operand_from_swiglu": (_i32, [_vp, _vp, _i32, _i64, _i32, _i32, _i64, _i64, _vp, _vp, _vp]),
     "mase_hip_scaled_operand_from_mxfp": (_i32, [_vp, _vp, _i32, _i32, _i64, _i64, _vp, _vp, _vp]),
     "mase_hip_mxfp_gemm_scaled": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _vp]),

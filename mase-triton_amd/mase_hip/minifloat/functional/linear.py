@@ -12,6 +12,14 @@ element whose block scale is 2^0, so the codes are narrowed to one byte each and
 composes them to bf16 in registers on their way to the MFMA units.  Such values have at most
 four significant bits, so the bf16 operands are exact and the result differs from "separate"
 only by the summation order.  Other formats fall back to compose + dense GEMM.
+
+With bfloat16 activations that are quantised too (XqWq), both formats among E4M3 / E3M2 / E2M3 /
+E2M1 and round to nearest, "fused" takes the block-scaled matrix instruction instead, for the row
+counts ``mxfp.functional.linear.takes_scaled_route`` names: x is rounded straight into code bytes
+with unit scales, W's codes are put into the same form (once per layer when a layer calls), and
+the GEMM multiplies the codes themselves at twice the bf16 rate.  The only difference in value is
+the re-encoding of E4M3 blocks that hold the top code (see include/mase_hip.h).
+``backend="fused_bf16"`` / ``"fused_scaled"`` (not in the reference) force one route or the other.
 """
 from __future__ import annotations
 
@@ -21,6 +29,7 @@ import torch
 from torch import Tensor
 
 from ...mxfp import kernels as mxfp_kernels
+from ...mxfp.functional.linear import takes_scaled_route
 from ...mxfp.meta import MXFPMeta
 from .. import kernels
 from ..meta import MinifloatMeta, MinifloatTensorMeta
@@ -71,8 +80,39 @@ def _gemm_eligible(x: Tensor, x_meta: MinifloatMeta | None, w_tensor_meta: Minif
     return b is None or b.dtype in (torch.bfloat16, torch.float16, torch.float32)
 
 
+def _scaled_format(meta: MinifloatMeta) -> bool:
+    return meta.is_finite and meta.round_mode == "rn" and (meta.exp_bits, meta.frac_bits) in mxfp_kernels._SCALED_FORMATS
+
+
+def _scaled_eligible(x: Tensor, x_meta: MinifloatMeta | None, w_tensor_meta: MinifloatTensorMeta, b: Tensor | None) -> bool:
+    """Can the block-scaled matrix instruction take this product?"""
+    if x_meta is None or x.device.type != "cuda" or x.dtype != torch.bfloat16 or len(w_tensor_meta.shape) != 2:
+        return False
+    if not (_scaled_format(x_meta) and _scaled_format(w_tensor_meta.meta)) or getattr(torch, w_tensor_meta.dtype) != x.dtype:
+        return False
+    out_features, in_features = w_tensor_meta.shape
+    if not mxfp_kernels.scaled_shape_supported(out_features, in_features, x.dtype) or x.numel() == 0:
+        return False
+    return b is None or b.dtype in (torch.bfloat16, torch.float16, torch.float32)
+
+
+def scaled_weight_operand(w_element: Tensor, w_tensor_meta: MinifloatTensorMeta,
+                          narrowed: tuple[Tensor, Tensor] | None = None) -> "mxfp_kernels.ScaledOperand":
+    """The weight codes in the block-scaled GEMM's form (a copy: N * K bytes of codes, N * K / 32 of unit scales).
+    A layer builds it once and passes it to ``minifloat_linear(..., _w_operand=...)``."""
+    scales, codes = narrowed if narrowed is not None else narrow_weight_codes(w_element, w_tensor_meta)
+    out_features, in_features = w_tensor_meta.shape
+    wm = w_tensor_meta.meta
+    as_mxfp = MXFPMeta(block_size=32, scale_exp_bits=8, element_exp_bits=wm.exp_bits, element_frac_bits=wm.frac_bits,
+                       element_is_finite=True, round_mode="rn")
+    return mxfp_kernels.scaled_operand_from_mxfp(scales, codes, as_mxfp, out_features, in_features)
+
+
+_BACKENDS = ("separate", "fused", "fused_bf16", "fused_scaled")
+
+
 def _check_backend(backend: str) -> None:
-    if backend not in ("separate", "fused"):
+    if backend not in _BACKENDS:
         raise NotImplementedError(f"backend {backend!r} not implemented")
 
 
@@ -86,11 +126,12 @@ def minifloat_linear(
     b_element: Tensor | None,
     b_tensor_meta: MinifloatTensorMeta | None,
     layer_type: Literal["XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq"],
-    backend: Literal["separate", "fused"],
+    backend: Literal["separate", "fused", "fused_bf16", "fused_scaled"],
     _narrowed: tuple[Tensor, Tensor] | None = None,
+    _w_operand: "mxfp_kernels.ScaledOperand | None" = None,
 ) -> Tensor:
-    """``_narrowed`` (not in the reference's signature): the result of ``narrow_weight_codes``
-    for this weight, kept by a caller that applies the same weight many times."""
+    """``_narrowed`` and ``_w_operand`` (not in the reference's signature): the results of ``narrow_weight_codes`` and
+    ``scaled_weight_operand`` for this weight, kept by a caller that applies the same weight many times."""
     if layer_type not in _LAYER_TYPES:
         raise NotImplementedError(f"Layer type {layer_type} not implemented")
     _check_backend(backend)
@@ -101,13 +142,29 @@ def minifloat_linear(
         # is passed as well; with b=None (what MinifloatLinearPTQ passes) no bias is added
         b = compose_minifloat_component(b_element, b_tensor_meta) if b is not None else None
 
-    if backend == "fused" and quantised_w and _gemm_eligible(x, x_meta if quantised_x else None, w_tensor_meta, b):
+    fused = backend != "separate"
+    if fused and backend != "fused_bf16" and quantised_x and quantised_w:
+        ok = _scaled_eligible(x, x_meta, w_tensor_meta, b)
+        if backend == "fused_scaled" and not ok:
+            raise NotImplementedError("fused_scaled: this product does not fit the block-scaled GEMM (bfloat16 x, formats E4M3 / "
+                                      "E3M2 / E2M3 / E2M1 rounded to nearest, K a multiple of 256 and at least 512, N of 8)")
+        rows = x.numel() // x.shape[-1] if x.numel() else 0
+        if ok and (backend == "fused_scaled" or takes_scaled_route(rows, _w_operand is not None)):
+            if _w_operand is None:
+                _w_operand = scaled_weight_operand(w_element, w_tensor_meta, _narrowed)
+            a_op = mxfp_kernels.scaled_operand_from_dense_minifloat(x.reshape(-1, x.shape[-1]), x_meta.exp_bits, x_meta.frac_bits)
+            y = mxfp_kernels.mxfp_gemm_scaled(a_op, _w_operand, b, x.dtype)
+            return y.view(*x.shape[:-1], w_tensor_meta.shape[0])
+    elif backend == "fused_scaled":
+        raise NotImplementedError("fused_scaled needs quantised activations and weights (XqWq layer types)")
+
+    if fused and quantised_w and _gemm_eligible(x, x_meta if quantised_x else None, w_tensor_meta, b):
         if _narrowed is None:
             _narrowed = narrow_weight_codes(w_element, w_tensor_meta)
         return _fused_gemm(x, x_meta if quantised_x else None, _narrowed, w_tensor_meta, b)
 
     if quantised_x:
-        if backend == "fused":
+        if fused:
             x = quantize_dequantize(x, x_meta)
         else:
             x_element, x_tensor_meta = extract_minifloat_component(x, x_meta)

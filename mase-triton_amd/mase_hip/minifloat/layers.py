@@ -34,7 +34,7 @@ class MinifloatLinearPTQ(nn.Module):
         w_minifloat_meta: MinifloatMeta | None,
         b_minifloat_meta: MinifloatMeta | None,
         layer_type: LayerType,
-        backend: Literal["separate", "fused"] = "fused",
+        backend: Literal["separate", "fused", "fused_bf16", "fused_scaled"] = "fused",
         dtype: torch.dtype | None = None,
         device: torch.device | None = None,
         w_element: Tensor | None = None,
@@ -67,6 +67,7 @@ class MinifloatLinearPTQ(nn.Module):
         self.w_element = self.w_tensor_meta = None
         self.b_element = self.b_tensor_meta = None
         self._narrowed = self._narrowed_key = None
+        self._scaled_w = self._scaled_w_key = None
 
         if "Wq" in layer_type:
             if w_element is None:
@@ -90,6 +91,7 @@ class MinifloatLinearPTQ(nn.Module):
         before = {n: getattr(self, n).dtype for n in self._CODE_PARAMS if getattr(self, n) is not None}
         result = super()._apply(fn, recurse)
         self._narrowed = self._narrowed_key = None
+        self._scaled_w = self._scaled_w_key = None
         for name, dt in before.items():
             now = getattr(self, name).dtype
             if now != dt:
@@ -104,7 +106,7 @@ class MinifloatLinearPTQ(nn.Module):
         """One-byte copy of the weight codes for the fused GEMM (not part of ``state_dict``),
         rebuilt when ``w_element`` is replaced, written in place or moved."""
         w = self.w_element
-        if (self.backend != "fused" or w is None or w.device.type != "cuda"
+        if (self.backend == "separate" or w is None or w.device.type != "cuda"
                 or not MinifloatF.gemm_weight_eligible(self.w_tensor_meta)):
             return None
         key = (w.data_ptr(), w._version, w.device)
@@ -113,13 +115,33 @@ class MinifloatLinearPTQ(nn.Module):
             self._narrowed_key = key
         return self._narrowed
 
+    def _weight_operand(self, input: Tensor):
+        """The weight in the block-scaled GEMM's form when this call takes that GEMM (quantised bfloat16 activations, see
+        ``minifloat_linear``), else None.  Not part of ``state_dict``; rebuilt like the one-byte copy."""
+        from ..mxfp.functional.linear import takes_scaled_route
+        from .functional import linear as L
+
+        w = self.w_element
+        if self.backend in ("separate", "fused_bf16") or w is None or not self.layer_type.startswith("XqWq") or input.device.type != "cuda":
+            return None
+        rows = input.numel() // input.shape[-1] if input.numel() else 0
+        bias = self.bias if not self.layer_type.endswith("Bq") else None
+        if not ((self.backend == "fused_scaled" or takes_scaled_route(rows, True))
+                and L._scaled_eligible(input, self.x_minifloat_meta, self.w_tensor_meta, bias)):
+            return None
+        key = (w.data_ptr(), w._version, w.device)
+        if self._scaled_w_key != key:
+            self._scaled_w = L.scaled_weight_operand(w, self.w_tensor_meta, self._narrowed_weight())
+            self._scaled_w_key = key
+        return self._scaled_w
+
     @torch.no_grad()
     def forward(self, input: Tensor) -> Tensor:
         return MinifloatF.minifloat_linear(
             x=input, x_meta=self.x_minifloat_meta, w=self.weight, w_element=self.w_element,
             w_tensor_meta=self.w_tensor_meta, b=self.bias, b_element=self.b_element,
             b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend,
-            _narrowed=self._narrowed_weight())
+            _narrowed=self._narrowed_weight(), _w_operand=self._weight_operand(input))
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "

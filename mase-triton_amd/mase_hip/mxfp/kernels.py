@@ -267,6 +267,21 @@ def scaled_operand_from_dense(x: Tensor, meta: MXFPMeta) -> ScaledOperand:
     return ScaledOperand(codes, scales, rows, K)
 
 
+def scaled_operand_from_dense_minifloat(x: Tensor, exp_bits: int, frac_bits: int) -> ScaledOperand:
+    """Round every element of the bfloat16 matrix x [rows, K] to the finite minifloat format (exp_bits, frac_bits), to
+    nearest, straight into a block-scaled GEMM operand whose blocks all carry the scale 2^0."""
+    assert x.ndim == 2 and x.dtype == torch.bfloat16 and (exp_bits, frac_bits) in _SCALED_FORMATS
+    _lib.require_gpu(x, "activations")
+    x = _lib.dense(x)
+    rows, K = x.shape
+    codes, scales = _scaled_buffers(rows, K, x.device)
+    with _lib.on_device(x.device):
+        _lib.check(_lib.load().mase_hip_scaled_operand_from_dense_minifloat(
+            x.data_ptr(), _lib.dtype_code(x.dtype), exp_bits, frac_bits, rows, K,
+            codes.data_ptr(), scales.data_ptr(), _lib.stream_ptr(x.device)))
+    return ScaledOperand(codes, scales, rows, K)
+
+
 def scaled_operand_from_swiglu(gate: Tensor, up: Tensor, meta: MXFPMeta) -> ScaledOperand:
     """silu(gate) * up (bfloat16 [rows, K] each, unit inner stride, the same row stride: e.g. the two halves of a stacked
     projection's output) quantised straight into a block-scaled GEMM operand; the product is never stored."""

@@ -219,3 +219,118 @@ def test_minifloat_matmul_fused_takes_the_gemm(mf, monkeypatch):
     monkeypatch.setattr(torch, "matmul", boom)
     y = mf.F.minifloat_matmul(a, b, mf.meta.FP8_E4M3_fn, mf.meta.FP8_E4M3_fn, "XqWq", "fused")
     assert y.shape == (3, 40, 64)
+
+
+# ------------------------------------------------------------------ the block-scaled route
+SCALED_TAGS = ["FP8_E4M3_fn", "FP6_E2M3_fn", "FP6_E3M2_fn", "FP4_E2M1_fn"]
+
+
+def _awkward_activations(rows, K, g):
+    """bf16 values over the whole range of the formats: saturating ones (the top E4M3 code, which the operand re-encodes),
+    subnormals of the target formats, zeros of both signs, bf16 subnormals, inf and NaN."""
+    x = torch.randn(rows, K, generator=g) * torch.exp2(torch.randint(-12, 10, (rows, K), generator=g).float())
+    x = x.to(torch.bfloat16)
+    flat = x.view(-1)
+    specials = torch.tensor([float("inf"), float("-inf"), float("nan"), 0.0, -0.0, 480.0, -480.0, 448.0, 1e-40, -1e-40, 7.5, 28.0, 6.0],
+                            dtype=torch.float32).to(torch.bfloat16)
+    idx = torch.randperm(flat.numel(), generator=g)[: 16 * specials.numel()]
+    flat[idx] = specials.repeat(16)
+    return x
+
+
+@pytest.mark.parametrize("tag", SCALED_TAGS)
+@pytest.mark.parametrize("rows,K", [(70, 512), (256, 128), (1, 1280)])
+def test_minifloat_scaled_operand_is_the_extracted_codes(mf, tag, rows, K):
+    """The one-pass operand of x holds, bit for bit, what the separate steps give: extract_minifloat (checked against the CPU
+    checker), one byte per code, unit scales, the MXFP operand kernel."""
+    from mase_hip.mxfp import kernels as K_
+
+    meta = getattr(mf.meta, tag)
+    g = torch.Generator().manual_seed(rows + K)
+    x = _awkward_activations(rows, K, g)
+    codes16, tm = mf.F.extract_minifloat_component(x.to(DEV), meta)
+    assert torch.equal(codes16.cpu(), oracle.extract_minifloat(x, meta.exp_bits, meta.frac_bits))
+    by_steps = mf.F.linear.scaled_weight_operand(codes16, tm)
+    one_pass = K_.scaled_operand_from_dense_minifloat(x.to(DEV), meta.exp_bits, meta.frac_bits)
+    assert torch.equal(one_pass.codes[:rows], by_steps.codes[:rows])
+    assert torch.equal(one_pass.scales[:, :rows], by_steps.scales[:, :rows])
+    unit = one_pass.scales[:, :rows].view(torch.uint8)
+    assert bool(((unit == 127) | (unit == 128)).all())          # 128: a block re-encoded for the top E4M3 code
+    assert bool((unit == 128).any()) == (tag == "FP8_E4M3_fn")
+
+
+@pytest.mark.parametrize("x_tag,w_tag", [("FP8_E4M3_fn", "FP8_E4M3_fn"), ("FP8_E4M3_fn", "FP4_E2M1_fn"), ("FP6_E3M2_fn", "FP6_E2M3_fn"),
+                                         ("FP4_E2M1_fn", "FP8_E4M3_fn")])
+@pytest.mark.parametrize("MNK", [(300, 264, 768), (16, 512, 512), (1030, 256, 1024)])
+def test_minifloat_linear_scaled_vs_checker(mf, x_tag, w_tag, MNK):
+    """XqWqB on the block-scaled matrix instruction (forced) against fp64 on the checker's values and against the bf16 route;
+    the activations saturate here and there, so E4M3 blocks of x get re-encoded."""
+    M, N, K = MNK
+    g = torch.Generator().manual_seed(M + N)
+    x = (3 * torch.randn(M, K, generator=g)).to(torch.bfloat16)
+    x.view(-1)[torch.randperm(M * K, generator=g)[: M * K // 64]] = 1000.0
+    w = (0.5 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    b = torch.randn(N, generator=g).to(torch.bfloat16)
+    x_meta, w_meta = getattr(mf.meta, x_tag), getattr(mf.meta, w_tag)
+    w_codes, w_tm = mf.F.extract_minifloat_component(w.to(DEV), w_meta)
+    kw = dict(x=x.to(DEV), x_meta=x_meta, w=None, w_element=w_codes, w_tensor_meta=w_tm, b=b.to(DEV), b_element=None,
+              b_tensor_meta=None, layer_type="XqWqB")
+    y = mf.F.minifloat_linear(**kw, backend="fused_scaled")
+    assert y.dtype == torch.bfloat16 and y.shape == (M, N)
+    assert rel_fro(y, checker_linear(x, x_meta, w_codes, w_meta, b).to(y.dtype)) <= REL_FRO_TOL
+    assert rel_fro(y, mf.F.minifloat_linear(**kw, backend="fused_bf16")) <= REL_FRO_TOL
+    assert rel_fro(y, mf.F.minifloat_linear(**kw, backend="separate")) <= REL_FRO_TOL
+
+
+def test_minifloat_layer_routes(mf, monkeypatch):
+    """Which GEMM a layer's call takes: the block-scaled one for quantised bf16 activations in its formats at the row
+    counts of ``takes_scaled_route``, the bf16 one otherwise; the weight operand is built once and follows the codes."""
+    from mase_hip.mxfp import kernels as K_
+    from mase_hip.mxfp.functional.linear import SCALED_FROM_ROWS, SCALED_UP_TO_ROWS
+
+    calls = {"scaled": 0, "bf16": 0, "prepare": 0}
+    real_scaled, real_bf16, real_prepare = K_.mxfp_gemm_scaled, K_.mxfp_gemm, K_.scaled_operand_from_mxfp
+
+    def count(name, fn):
+        def wrapped(*a, **k):
+            calls[name] += 1
+            return fn(*a, **k)
+        return wrapped
+
+    monkeypatch.setattr(K_, "mxfp_gemm_scaled", count("scaled", real_scaled))
+    monkeypatch.setattr(K_, "mxfp_gemm", count("bf16", real_bf16))
+    monkeypatch.setattr(K_, "scaled_operand_from_mxfp", count("prepare", real_prepare))
+    N, K = 256, 512
+    lin = torch.nn.Linear(K, N, bias=True, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        lin.weight.mul_(16)  # minifloat has no block scale: bring the weights into FP6's range
+    g = torch.Generator().manual_seed(21)
+    layer = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")
+    separate = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "separate")
+    for rows, scaled in ((SCALED_FROM_ROWS, True), (SCALED_UP_TO_ROWS, True), (SCALED_UP_TO_ROWS + 8, False), (4 * SCALED_FROM_ROWS, True)):
+        before = dict(calls)
+        x = torch.randn(rows, K, generator=g).to(torch.bfloat16).to(DEV)
+        y = layer(x)
+        assert (calls["scaled"] - before["scaled"], calls["bf16"] - before["bf16"]) == ((1, 0) if scaled else (0, 1)), rows
+        assert rel_fro(y, separate(x)) <= REL_FRO_TOL
+    assert calls["prepare"] == 1
+    x = torch.randn(128, K, generator=g).to(torch.bfloat16).to(DEV)
+    y_before = layer(x)
+    with torch.no_grad():
+        for l in (layer, separate):
+            l.w_element.copy_((l.w_element.to(torch.int32) ^ 0x20).to(torch.uint16))   # flip every sign (E3M2 is 6 bits wide)
+    y_after = layer(x)
+    assert calls["prepare"] == 2
+    assert rel_fro(y_after, separate(x)) <= REL_FRO_TOL and rel_fro(y_after, y_before) > 0.5
+    # formats and dtypes the instruction does not take stay on the bf16 route; forcing it says why not
+    e5m2 = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP8_E5M2_fn, None, "XqWqB", "fused")
+    before = dict(calls)
+    e5m2(x)
+    assert (calls["scaled"], calls["bf16"]) == (before["scaled"], before["bf16"] + 1)
+    forced = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP8_E5M2_fn, None, "XqWqB", "fused_scaled")
+    with pytest.raises(NotImplementedError):
+        forced(x)
+    rd = mf.meta.MinifloatMeta(4, 3, True, "rd")
+    before = dict(calls)
+    mf.Layer.from_linear(lin, rd, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")(x)
+    assert calls["scaled"] == before["scaled"]

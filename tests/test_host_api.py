@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(lib):
     from mase_hip import _lib
 
     names = declared_symbols()
-    assert len(names) == 25
+    assert len(names) == 26
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mase_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of step with the header"
@@ -63,6 +63,9 @@ def test_argument_errors_without_a_gpu(lib):
     assert lib.mase_hip_scaled_operand_from_dense(p, 2, 4, 3, 8, 96, p, p, None) == -2     # K % 128
     assert lib.mase_hip_scaled_operand_from_dense(p, 2, 5, 2, 8, 128, p, p, None) == -2    # E5M2
     assert lib.mase_hip_scaled_operand_from_dense(p, 0, 4, 3, 8, 128, p, p, None) == -2    # fp32 input
+    assert lib.mase_hip_scaled_operand_from_dense_minifloat(p, 2, 5, 2, 8, 128, p, p, None) == -2    # E5M2
+    assert lib.mase_hip_scaled_operand_from_dense_minifloat(p, 1, 4, 3, 8, 128, p, p, None) == -2    # fp16 input
+    assert lib.mase_hip_scaled_operand_from_dense_minifloat(None, 2, 4, 3, 8, 128, p, p, None) == -1
     assert lib.mase_hip_scaled_operand_from_swiglu(p, None, 2, 128, 4, 3, 8, 128, p, p, None) == -1   # no up
     assert lib.mase_hip_scaled_operand_from_swiglu(p, p, 2, 64, 4, 3, 8, 128, p, p, None) == -1     # row stride below K
     assert lib.mase_hip_scaled_operand_from_swiglu(p, p, 2, 132, 4, 3, 8, 128, p, p, None) == -1    # row stride not a multiple of 8
