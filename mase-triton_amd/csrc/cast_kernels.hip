@@ -608,7 +608,7 @@ __global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint1
                                                                       uint8_t* __restrict__ codes, uint32_t* __restrict__ scales, int rows,
                                                                       int K, int nmac, uint32_t rows_pad, F f) {
     constexpr bool SWIGLU = MODE == FROM_SWIGLU, MINIFLOAT = MODE == FROM_DENSE_MINIFLOAT;
-    __shared__ __attribute__((aligned(16))) uint8_t lut[LdsLut<F, MINIFLOAT>::BYTES];   // (no table for the per-element rounding)
+    __shared__ __attribute__((aligned(16))) uint8_t lut[LdsLut<F, false>::BYTES + 16];   // (one more entry in the minifloat mode)
     const uint32_t ms = blockIdx.x % (uint32_t)nmac, row_base = (blockIdx.x / (uint32_t)nmac) * 32u;
     const int t = threadIdx.x;
     uint4 raw[2], raw_up[2];
@@ -623,7 +623,12 @@ __global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint1
         raw[r] = live[r] ? ld128(x + (size_t)row * ld + col) : make_uint4(0, 0, 0, 0);
         if (SWIGLU) raw_up[r] = live[r] ? ld128(up + (size_t)row * ld + col) : make_uint4(0, 0, 0, 0);
     }
-    LdsLut<F, MINIFLOAT>::fill(lut);
+    // minifloat mode: the same table serves (with the scale fixed at 2^0 the rounding of the reference's minifloat extract
+    // is the MXFP element's, step for step); values past the top binade, which a block's own scale rules out, saturate
+    // through one more entry
+    constexpr int LUT_N = LdsLut<F, false>::BYTES;
+    if (MINIFLOAT && t == 0) lut[LUT_N] = (uint8_t)((1u << (F{}.E() + F{}.M())) - 1u);
+    LdsLut<F, false>::fill(lut);
     const uint32_t lut_addr = (uint32_t)(uintptr_t)lut;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
@@ -631,13 +636,25 @@ __global__ __launch_bounds__(kThreads) void scaled_from_dense_kernel(const uint1
         uint32_t o[4], scale;
         if constexpr (MINIFLOAT) {
             const uint32_t h[4] = {raw[r].x, raw[r].y, raw[r].z, raw[r].w};
+            constexpr int E = F{}.E(), M = F{}.M();
             // inf / NaN anywhere in the wavefront's elements: the per-element routine for all of them
-            bool special = false;
+            const u16x2 m2 = __builtin_elementwise_max(__builtin_elementwise_max(as_u16x2(h[0] & 0x7FFF7FFFu), as_u16x2(h[1] & 0x7FFF7FFFu)),
+                                                       __builtin_elementwise_max(as_u16x2(h[2] & 0x7FFF7FFFu), as_u16x2(h[3] & 0x7FFF7FFFu)));
+            if (__builtin_amdgcn_ballot_w64(max((uint32_t)m2[0], (uint32_t)m2[1]) >= 0x7F80u) == 0) {
+                constexpr uint32_t OFF = (uint32_t)(127 - ((1 << (E - 1)) - 1)) << 7;   // t = |x| bits - OFF, saturating: below the format's range gives entry 0
+                uint32_t lo[4], hi[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) special |= (h[j] & 0x7F80u) == 0x7F80u || (h[j] & 0x7F800000u) == 0x7F800000u;
-            if (__builtin_amdgcn_ballot_w64(special) == 0) {
+                for (int j = 0; j < 4; ++j) {
+                    const u16x2 d = __builtin_elementwise_sub_sat(as_u16x2(h[j] & 0x7FFF7FFFu), as_u16x2(OFF * 0x00010001u));
+                    lut_pair<false>(lo[j], hi[j], lut_addr, as_u32(__builtin_elementwise_min(d, as_u16x2((uint32_t)LUT_N * 0x00010001u))));
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]), "+v"(hi[0]), "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3]));
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] = encode_f32_finite_rn(h[j] << 16, f) | (encode_f32_finite_rn(h[j] & 0xFFFF0000u, f) << 16);
+                for (int j = 0; j < 4; ++j) {
+                    // the sign code goes with every negative input but -0.0, flushed ones included
+                    const uint32_t sign = h[j] & ((h[j] & 0x7FFF7FFFu) + 0x7FFF7FFFu) & 0x80008000u;
+                    o[j] = lo[j] | (hi[j] << 16) | (sign >> (15 - (E + M)));
+                }
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) o[j] = encode_f32_bits(h[j] << 16, f) | (encode_f32_bits(h[j] & 0xFFFF0000u, f) << 16);

@@ -259,6 +259,22 @@ def test_minifloat_scaled_operand_is_the_extracted_codes(mf, tag, rows, K):
     assert bool((unit == 128).any()) == (tag == "FP8_E4M3_fn")
 
 
+@pytest.mark.parametrize("tag", SCALED_TAGS)
+def test_minifloat_scaled_operand_every_bf16_pattern(mf, tag):
+    """All 65536 bfloat16 bit patterns, in order (so that most wavefronts take the table look-up and the ones that hold inf
+    and NaN the per-element routine): the same codes as the separate steps."""
+    from mase_hip.mxfp import kernels as K_
+
+    meta = getattr(mf.meta, tag)
+    x = torch.arange(65536, dtype=torch.int32).to(torch.uint16).view(torch.bfloat16).view(512, 128)
+    codes16, tm = mf.F.extract_minifloat_component(x.to(DEV), meta)
+    assert torch.equal(codes16.cpu(), oracle.extract_minifloat(x, meta.exp_bits, meta.frac_bits))
+    by_steps = mf.F.linear.scaled_weight_operand(codes16, tm)
+    one_pass = K_.scaled_operand_from_dense_minifloat(x.to(DEV), meta.exp_bits, meta.frac_bits)
+    assert torch.equal(one_pass.codes[:512], by_steps.codes[:512])
+    assert torch.equal(one_pass.scales[:, :512], by_steps.scales[:, :512])
+
+
 @pytest.mark.parametrize("x_tag,w_tag", [("FP8_E4M3_fn", "FP8_E4M3_fn"), ("FP8_E4M3_fn", "FP4_E2M1_fn"), ("FP6_E3M2_fn", "FP6_E2M3_fn"),
                                          ("FP4_E2M1_fn", "FP8_E4M3_fn")])
 @pytest.mark.parametrize("MNK", [(300, 264, 768), (16, 512, 512), (1030, 256, 1024)])
