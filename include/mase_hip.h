@@ -168,7 +168,8 @@ int mase_hip_unpack_codes(const uint8_t* packed, uint8_t* elements, int64_t n, i
  *      mase_hip_extract_mxfp on the row-major [N,K] weight.
  *   bias: NULL or bias[N] of dtype bias_dtype, added in fp32 before the output rounding.
  *
- * K must be a multiple of block_size, block_size must be 32, M, N, K >= 1.
+ * K must be a multiple of block_size, block_size must be 32, N, K >= 1; M == 0 (no rows of A) is a
+ * valid call that does nothing, here and in every GEMM entry point below.
  * Replaces the body of mxfp_linear_XqWq / mxfp_linear_XWq with backend="fused", which the
  * reference leaves unimplemented (src/mase_triton/mxfp/functional/linear.py:31-32,63-64); the
  * result equals the "separate" backend (compose, then torch.nn.functional.linear, :50-61) up

@@ -11,7 +11,8 @@ static int gemm_entry(const void* a_dense, int a_dtype, const uint8_t* a_scales,
                       const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, int block_size,
                       void* workspace, int64_t workspace_bytes, void* stream, int64_t batches = 1, int64_t a_batch_stride = 0,
                       int64_t w_batch_stride = 0, int64_t y_batch_stride = 0) {
-    if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
+    if (M < 0 || N < 1 || K < 1) return fail(ERR_INVALID, "M must not be negative, N and K must be positive");
+    if (M == 0) return OK;   // no rows of A: nothing to compute
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(ERR_INVALID, "M, N, K must fit in 31 bits");
     if (block_size != 32) return fail(ERR_UNSUPPORTED, "the GEMM supports block_size 32 only");
     if (K % 32 != 0) return fail(ERR_INVALID, "K must be a multiple of the block size");

@@ -6,7 +6,8 @@ using namespace mase;
 static int scaled_entry(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales,
                         const void* bias, int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
                         int64_t workspace_bytes, void* stream) {
-    if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
+    if (M < 0 || N < 1 || K < 1) return fail(ERR_INVALID, "M must not be negative, N and K must be positive");
+    if (M == 0) return OK;   // no rows of A: nothing to compute
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K >= ((int64_t)1 << 27)) return fail(ERR_INVALID, "M, N must fit in 31 bits and K in 27");
     if (K % 256 != 0 || K < 512) return fail(ERR_UNSUPPORTED, "the block-scaled GEMM needs K to be a multiple of 256, at least 512");
     if (!a_codes || !a_scales || !w_codes || !w_scales || !y) return fail(ERR_INVALID, "null pointer");
@@ -44,7 +45,8 @@ extern "C" int64_t mase_hip_mxfp_gemm_scaled_workspace_bytes(int64_t M, int64_t 
 
 extern "C" int mase_hip_mxfp_gemm_prepared_w(const void* a_dense, int a_dtype, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
                                              int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
-    if (M < 1 || N < 1 || K < 1) return fail(ERR_INVALID, "M, N, K must be positive");
+    if (M < 0 || N < 1 || K < 1) return fail(ERR_INVALID, "M must not be negative, N and K must be positive");
+    if (M == 0) return OK;   // no rows of A: nothing to compute
     if (M > 0x7FFFFFFF || N > 0x7FFFFFFF || K > 0x7FFFFFFF) return fail(ERR_INVALID, "M, N, K must fit in 31 bits");
     if (!a_dense || !w_codes || !w_scales || !y) return fail(ERR_INVALID, "null pointer");
     if (a_dtype != BF16) return fail(ERR_UNSUPPORTED, "a dense A operand must be bfloat16");

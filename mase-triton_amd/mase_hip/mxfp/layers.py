@@ -69,6 +69,7 @@ class MXFPLinearPTQ(nn.Module):
         self.dtype, self.device = dtype, device
 
         self._scaled_w = self._scaled_w_key = None   # the weight in the block-scaled GEMM's form, and what it was built from
+        self._fast_sig = None                        # what the last call on the block-scaled route looked like (see forward)
         self.weight = self.bias = None
         self.w_scales = self.w_elements = self.w_tensor_meta = None
         self.b_scales = self.b_elements = self.b_tensor_meta = None
@@ -112,7 +113,7 @@ class MXFPLinearPTQ(nn.Module):
         """Drop the cached block-scaled form of the weight.  Writes to ``w_scales`` / ``w_elements`` that torch records
         (``copy_`` under ``no_grad``, ``load_state_dict``, moving the module) are noticed without this call; writes
         through ``.data`` are not."""
-        self._scaled_w = self._scaled_w_key = None
+        self._scaled_w = self._scaled_w_key = self._fast_sig = None
 
     def _takes_scaled_route(self, input: Tensor) -> bool:
         """Does ``forward(input)`` run on the block-scaled GEMM?"""
@@ -148,13 +149,29 @@ class MXFPLinearPTQ(nn.Module):
             self._scaled_w_key = key
         return self._scaled_w
 
+    def _call_signature(self, input: Tensor) -> tuple:
+        return (input.shape, input.dtype, input.device, self.backend, self.layer_type, self.x_mxfp_meta)
+
     @torch.no_grad()
     def forward(self, input: Tensor) -> Tensor:
+        # A call that looks like the last one that ran on the block-scaled GEMM with the kept weight operand, the weight
+        # unchanged since, goes straight to the two kernels: the checks below cost more host time than a decode-sized
+        # product takes on the GPU.
+        if self._fast_sig is not None and self._fast_sig == self._call_signature(input):
+            w_elements, w_scales = self.w_elements, self.w_scales
+            if self._scaled_w_key == (w_elements.data_ptr(), w_elements._version, w_scales.data_ptr(), w_scales._version):
+                from . import kernels
+
+                a_op = kernels.scaled_operand_from_dense(input.reshape(-1, self.in_features), self.x_mxfp_meta)
+                bias = None if self.layer_type.endswith("Bq") else self.bias
+                return kernels.mxfp_gemm_scaled(a_op, self._scaled_w, bias, input.dtype).view(*input.shape[:-1], self.out_features)
+        w_operand = self._weight_operand(input)
+        self._fast_sig = self._call_signature(input) if w_operand is not None and self._takes_scaled_route(input) else None
         return MXFP_F.mxfp_linear(
             x=input, x_meta=self.x_mxfp_meta, w=self.weight, w_scales=self.w_scales, w_elements=self.w_elements,
             w_tensor_meta=self.w_tensor_meta, b=self.bias, b_scales=self.b_scales, b_elements=self.b_elements,
             b_tensor_meta=self.b_tensor_meta, layer_type=self.layer_type, backend=self.backend,
-            w_operand=self._weight_operand(input))
+            w_operand=w_operand)
 
     @torch.no_grad()
     def forward_swiglu(self, gate: Tensor, up: Tensor) -> Tensor:

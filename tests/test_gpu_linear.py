@@ -583,6 +583,65 @@ def test_layer_keeps_and_refreshes_its_weight_operand(mh):
     assert rel_fro(layer(big), sep(big)) <= REL_FRO_TOL and layer._scaled_w is not second
 
 
+def test_layer_repeat_calls_skip_the_checks_and_notice_changes(mh, monkeypatch):
+    """A call like the previous one on the block-scaled route goes straight to the two kernels (same bits as the checked
+    path); another shape, backend, activation format or weight goes through the checks again."""
+    import mase_hip.mxfp.functional as MXFP_F
+    import mase_hip.mxfp.layers as layers_mod
+
+    calls = [0]
+    real = MXFP_F.mxfp_linear
+
+    def counted(*a, **k):
+        calls[0] += 1
+        return real(*a, **k)
+
+    monkeypatch.setattr(layers_mod.MXFP_F, "mxfp_linear", counted)
+    fmt, fmt4 = preset(mh, "MXFP8_E4M3_fn"), preset(mh, "OCP_MXFP4_E2M1")
+    g = torch.Generator().manual_seed(8)
+    lin = torch.nn.Linear(512, 264, bias=True, dtype=torch.bfloat16, device=DEV)
+    layer = mh.MXFPLinearPTQ.from_linear(lin, fmt, fmt, None, "XqWqB", "fused")
+    x = torch.randn(2, 8, 512, generator=g).to(torch.bfloat16).to(DEV)
+    y0 = layer(x)
+    y1 = layer(x)
+    y2 = layer(x + 0)                                   # another tensor of the same kind
+    assert calls[0] == 1 and torch.equal(y0, y1) and torch.equal(y0, y2) and y1.shape == (2, 8, 264)
+    layer(x[:1])                                        # other shape
+    assert calls[0] == 2
+    layer(x)
+    layer(x)
+    assert calls[0] == 3
+    layer.x_mxfp_meta = fmt4                            # other activation format
+    y4 = layer(x)
+    assert calls[0] == 4 and not torch.equal(y4, y0)
+    assert torch.equal(y4, mh.MXFPLinearPTQ.from_linear(lin, fmt4, fmt, None, "XqWqB", "fused")(x))
+    calls[0] = 4                                        # (the line above counted one for the other layer)
+    layer.x_mxfp_meta = fmt
+    layer(x)
+    assert calls[0] == 5
+    with torch.no_grad():
+        layer.w_elements.copy_(layer.w_elements ^ 0x80)  # every sign flipped
+        layer.bias.zero_()
+    y5 = layer(x)
+    assert calls[0] == 6
+    layer.bias = None                                   # the fast path reads the bias of the moment
+    y6 = layer(x)
+    assert calls[0] == 6 and torch.equal(y5, y6)
+    lin0 = torch.nn.Linear(512, 264, bias=False, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        lin0.weight.copy_(lin.weight)
+    assert torch.equal(y6, -mh.MXFPLinearPTQ.from_linear(lin0, fmt, fmt, None, "XqWqB", "fused")(x))
+    calls[0] = 6
+    layer.backend = "separate"
+    y7 = layer(x)
+    assert calls[0] == 7 and rel_fro(y7, y6) <= REL_FRO_TOL
+    layer.backend = "fused"
+    layer(x)
+    assert layer._fast_sig is not None
+    y8 = layer(x[:, :0])                                # no rows: nothing to compute, nothing to remember
+    assert y8.shape == (2, 0, 264) and layer._fast_sig is None
+
+
 @pytest.mark.parametrize("backend", ["fused", "fused_bf16"])
 def test_config_c5_swiglu_chain(mh, backend):
     """down(silu(gate(x)) * up(x)) with MXFP6 E3M2 weights and MXFP8 E4M3 activations, on either kernel family ("fused"

@@ -350,3 +350,41 @@ def test_minifloat_layer_routes(mf, monkeypatch):
     before = dict(calls)
     mf.Layer.from_linear(lin, rd, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")(x)
     assert calls["scaled"] == before["scaled"]
+
+
+def test_minifloat_layer_repeat_calls_skip_the_checks_and_notice_changes(mf, monkeypatch):
+    """As for the MXFP layer: a call like the previous one on the block-scaled route goes straight to the two kernels,
+    with the same bits; other shapes, formats and codes go through the checks again."""
+    import mase_hip.minifloat.layers as layers_mod
+
+    calls = [0]
+    real = layers_mod.MinifloatF.minifloat_linear
+
+    def counted(*a, **k):
+        calls[0] += 1
+        return real(*a, **k)
+
+    monkeypatch.setattr(layers_mod.MinifloatF, "minifloat_linear", counted)
+    lin = torch.nn.Linear(512, 264, bias=True, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        lin.weight.mul_(16)
+    g = torch.Generator().manual_seed(31)
+    layer = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")
+    x = (3 * torch.randn(2, 8, 512, generator=g)).to(torch.bfloat16).to(DEV)
+    y0, y1 = layer(x), layer(x)
+    assert calls[0] == 1 and torch.equal(y0, y1) and y1.shape == (2, 8, 264)
+    layer(x[:1])
+    layer(x)
+    assert calls[0] == 3
+    layer.x_minifloat_meta = mf.meta.FP4_E2M1_fn
+    y2 = layer(x)
+    assert calls[0] == 4 and not torch.equal(y2, y0)
+    assert torch.equal(layer(x), y2) and calls[0] == 4
+    assert torch.equal(y2, mf.Layer.from_linear(lin, mf.meta.FP4_E2M1_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")(x))
+    calls[0] = 4                                         # (the line above counted one for the other layer)
+    with torch.no_grad():
+        layer.w_element.copy_((layer.w_element.to(torch.int32) ^ 0x20).to(torch.uint16))
+    y3 = layer(x)
+    assert calls[0] == 5 and not torch.equal(y3, y2)
+    y4 = layer(x[:, :0])
+    assert y4.shape == (2, 0, 264) and layer._fast_sig is None

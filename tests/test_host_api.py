@@ -76,7 +76,12 @@ def test_argument_errors_without_a_gpu(lib):
     assert lib.mase_hip_mxfp_gemm(p, 2, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, 16, 16, 48, 32, None) == -1
     assert lib.mase_hip_mxfp_gemm(p, 2, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, 16, 16, 64, 16, None) == -2
     assert lib.mase_hip_mxfp_gemm(p, 0, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, 16, 16, 64, 32, None) == -2
-    # n == 0 is a valid no-op
+    # n == 0 is a valid no-op, and so is a product with no rows of A
+    assert lib.mase_hip_mxfp_gemm(None, 2, None, None, 0, 0, None, None, 4, 3, None, 0, None, 2, 0, 16, 64, 32, None) == 0
+    assert lib.mase_hip_mxfp_gemm_scaled(None, None, None, None, None, 0, None, 2, 0, 8, 512, None) == 0
+    assert lib.mase_hip_mxfp_gemm_prepared_w(None, 2, None, None, None, 0, None, 2, 0, 128, 128, None) == 0
+    assert lib.mase_hip_mxfp_gemm(p, 2, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, -1, 16, 64, 32, None) == -1
+    assert lib.mase_hip_mxfp_gemm(p, 2, None, None, 0, 0, p, p, 4, 3, None, 0, p, 2, 0, 0, 64, 32, None) == -1
     assert lib.mase_hip_extract_mxfp(None, 2, None, None, 0, 32, 4, 3, 1, 0, None) == 0
     assert lib.mase_hip_qdq_minifloat(None, 0, None, 0, 0, 4, 3, 1, 0, None) == 0
 
