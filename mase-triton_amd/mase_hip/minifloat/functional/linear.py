@@ -91,7 +91,7 @@ def _scaled_eligible(x: Tensor, x_meta: MinifloatMeta | None, w_tensor_meta: Min
     if not (_scaled_format(x_meta) and _scaled_format(w_tensor_meta.meta)) or getattr(torch, w_tensor_meta.dtype) != x.dtype:
         return False
     out_features, in_features = w_tensor_meta.shape
-    if not mxfp_kernels.scaled_shape_supported(out_features, in_features, x.dtype) or x.numel() == 0:
+    if not mxfp_kernels.scaled_shape_supported(out_features, in_features, x.dtype):
         return False
     return b is None or b.dtype in (torch.bfloat16, torch.float16, torch.float32)
 

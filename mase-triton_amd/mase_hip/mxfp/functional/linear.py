@@ -96,7 +96,7 @@ def _scaled_eligible(x: Tensor, x_meta: MXFPMeta | None, w_tensor_meta: MXFPTens
     if x_meta.round_mode != "rn" or w_tensor_meta.block_dim % 2 != 1 or getattr(torch, w_tensor_meta.dtype) != x.dtype:
         return False
     out_features, in_features = w_tensor_meta.shape
-    if not kernels.scaled_shape_supported(out_features, in_features, x.dtype) or x.numel() == 0:
+    if not kernels.scaled_shape_supported(out_features, in_features, x.dtype):
         return False
     return b is None or b.dtype in (torch.bfloat16, torch.float16, torch.float32)
 

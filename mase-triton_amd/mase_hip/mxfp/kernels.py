@@ -260,6 +260,8 @@ def scaled_operand_from_dense(x: Tensor, meta: MXFPMeta) -> ScaledOperand:
     x = _lib.dense(x)
     rows, K = x.shape
     codes, scales = _scaled_buffers(rows, K, x.device)
+    if rows == 0:
+        return ScaledOperand(codes, scales, rows, K)   # nothing to quantise
     with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_scaled_operand_from_dense(
             x.data_ptr(), _lib.dtype_code(x.dtype), meta.element_exp_bits, meta.element_frac_bits, rows, K,
@@ -275,6 +277,8 @@ def scaled_operand_from_dense_minifloat(x: Tensor, exp_bits: int, frac_bits: int
     x = _lib.dense(x)
     rows, K = x.shape
     codes, scales = _scaled_buffers(rows, K, x.device)
+    if rows == 0:
+        return ScaledOperand(codes, scales, rows, K)   # nothing to quantise
     with _lib.on_device(x.device):
         _lib.check(_lib.load().mase_hip_scaled_operand_from_dense_minifloat(
             x.data_ptr(), _lib.dtype_code(x.dtype), exp_bits, frac_bits, rows, K,
@@ -293,6 +297,8 @@ def scaled_operand_from_swiglu(gate: Tensor, up: Tensor, meta: MXFPMeta) -> Scal
         gate, up = gate.contiguous(), up.contiguous()
     rows, K = gate.shape
     codes, scales = _scaled_buffers(rows, K, gate.device)
+    if rows == 0:
+        return ScaledOperand(codes, scales, rows, K)   # nothing to quantise
     with _lib.on_device(gate.device):
         _lib.check(_lib.load().mase_hip_scaled_operand_from_swiglu(
             gate.data_ptr(), up.data_ptr(), _lib.dtype_code(gate.dtype), gate.stride(0) if rows > 1 else K,

@@ -642,6 +642,45 @@ def test_layer_repeat_calls_skip_the_checks_and_notice_changes(mh, monkeypatch):
     assert y8.shape == (2, 0, 264) and layer._fast_sig is None
 
 
+@pytest.mark.filterwarnings("ignore:mase_hip. an operand is not 16-byte aligned")
+@pytest.mark.parametrize("backend", ["fused", "fused_bf16", "fused_scaled"])
+@pytest.mark.parametrize("layer_type", ["XqWqB", "XWqB"])
+def test_linear_input_layouts(mh, backend, layer_type):
+    """Inputs as torch.nn.functional.linear takes them: one vector, no rows, a strided view, many leading axes; every fused
+    backend against float64 on the quantised operands (the casts that produce them are checked bit for bit elsewhere), and
+    in shape and dtype against "separate" on the same layer (whose bf16 result is rounded twice, product and bias, when
+    torch is handed a strided 3-D input: not a yardstick for 1e-3)."""
+    if backend == "fused_scaled" and layer_type != "XqWqB":
+        pytest.skip("the block-scaled route needs quantised activations")
+    fmt = preset(mh, "MXFP8_E4M3_fn")
+    g = torch.Generator().manual_seed(12)
+    lin = torch.nn.Linear(512, 136, bias=True, dtype=torch.bfloat16, device=DEV)
+    x_meta = fmt if layer_type.startswith("Xq") else None
+    layer = mh.MXFPLinearPTQ.from_linear(lin, x_meta, fmt, None, layer_type, backend)
+    sep = mh.MXFPLinearPTQ.from_linear(lin, x_meta, fmt, None, layer_type, "separate")
+    base = torch.randn(6, 70, 1024, generator=g).to(torch.bfloat16).to(DEV)
+    cases = {
+        "vector": base[0, 0, :512],
+        "no rows": base[:, :0, :512],
+        "no batch": base[:0, :, :512],
+        "row-strided view": base[..., :512],
+        "element-strided view": base[..., ::2],
+        "transposed batch axes": base[..., :512].transpose(0, 1),
+        "five axes": base[..., :512].reshape(2, 3, 7, 10, 512),
+        "offset by one element": base.view(-1)[1:1 + 9 * 512].view(9, 512),
+    }
+    w_dq = mh.F.compose_mxfp_tensor(sep.w_scales, sep.w_elements, sep.w_tensor_meta).double()
+    for name, x in cases.items():
+        y, y_sep = layer(x), sep(x)
+        assert y.shape == y_sep.shape == (*x.shape[:-1], 136) and y.dtype == y_sep.dtype, name
+        if x.numel():
+            x_dq = mh.F.quantize_dequantize(x, block_dim=-1, mxfp_meta=x_meta) if x_meta is not None else x
+            y_ref = (x_dq.double() @ w_dq.t() + lin.bias.double()).to(y.dtype)
+            assert rel_fro(y, y_ref) <= REL_FRO_TOL, name
+            assert rel_fro(layer(x), y_ref) <= REL_FRO_TOL, name      # and again (the layer's repeat-call path)
+            assert rel_fro(y_sep, y_ref) <= 4 * REL_FRO_TOL, name
+
+
 @pytest.mark.parametrize("backend", ["fused", "fused_bf16"])
 def test_config_c5_swiglu_chain(mh, backend):
     """down(silu(gate(x)) * up(x)) with MXFP6 E3M2 weights and MXFP8 E4M3 activations, on either kernel family ("fused"

@@ -388,3 +388,32 @@ def test_minifloat_layer_repeat_calls_skip_the_checks_and_notice_changes(mf, mon
     assert calls[0] == 5 and not torch.equal(y3, y2)
     y4 = layer(x[:, :0])
     assert y4.shape == (2, 0, 264) and layer._fast_sig is None
+
+
+@pytest.mark.filterwarnings("ignore:mase_hip. an operand is not 16-byte aligned")
+@pytest.mark.parametrize("backend", ["fused", "fused_bf16", "fused_scaled"])
+def test_minifloat_linear_input_layouts(mf, backend):
+    """One vector, no rows, strided and misaligned views, many leading axes through the layer, against float64 on the
+    checker's values."""
+    lin = torch.nn.Linear(512, 136, bias=True, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        lin.weight.mul_(16)
+    x_meta, w_meta = mf.meta.FP8_E4M3_fn, mf.meta.FP6_E2M3_fn
+    layer = mf.Layer.from_linear(lin, x_meta, w_meta, None, "XqWqB", backend)
+    g = torch.Generator().manual_seed(14)
+    base = (2 * torch.randn(6, 70, 1024, generator=g)).to(torch.bfloat16).to(DEV)
+    cases = {
+        "vector": base[0, 0, :512],
+        "no rows": base[:, :0, :512],
+        "row-strided view": base[..., :512],
+        "element-strided view": base[..., ::2],
+        "five axes": base[..., :512].reshape(2, 3, 7, 10, 512),
+        "offset by one element": base.view(-1)[1:1 + 9 * 512].view(9, 512),
+    }
+    for name, x in cases.items():
+        y = layer(x)
+        assert y.shape == (*x.shape[:-1], 136) and y.dtype == torch.bfloat16, name
+        if x.numel():
+            y_ref = checker_linear(x, x_meta, layer.w_element, w_meta, lin.bias.detach()).to(y.dtype)
+            assert rel_fro(y, y_ref) <= REL_FRO_TOL, name
+            assert rel_fro(layer(x), y_ref) <= REL_FRO_TOL, name
