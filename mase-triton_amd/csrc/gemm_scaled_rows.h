@@ -265,8 +265,148 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 }
 
-// the shapes this kernel takes: up to 32 rows of A (two 16-row operand tiles)
-inline bool scaled_rows_shape_ok(int M, int K) { return M <= 32 && K >= 128; }
+// ---- The same with A in registers (K <= 4096, M <= 16 MT, MT = 2 or 4 operand tiles of 16 rows: 17 - 64 rows of A).  A
+// wavefront multiplies the same macro steps of every unit (wave w: SPW w .. SPW w + SPW - 1, SPW = 32 / WAVES), so the
+// fragments of A it needs are the same for the whole launch: MT x SPW x 8 registers (128 for four tiles on eight
+// wavefronts), filled once.  LDS then holds W alone and no byte of A is read a second time.  W takes the route of the
+// kernel above: 1 KB of one row per load instruction, one unit ahead in registers, through LDS; so does A on its way to
+// the registers, tile by tile through W's place in LDS (read straight from global memory in the operand layout, 64 bytes
+// of a row at a time, every cache line is fetched twice, and with every CU of an XCD asking its L2 for the same A that is
+// what the prologue costs: 22 against 19 us at 64 rows, N x K = 14336 x 4096).  Eight wavefronts: 15.6 against 18.4 us with
+// four at 32 rows (sixteen: the same, and the registers of four tiles no longer fit).  N x K = 14336 x 4096: 15.6 / 19.2 us at
+// 32 / 64 rows against 23.2 / 30.8 on the bf16 weight-streaming kernels and 23.8 / 26.9 on the chunked and the tile kernel; 4096 x
+// 4096: 7.6 / 10.0 against 10.7 / 16.9.  (One tile, 16 rows: 15.2 us, level with the kernel above, which keeps them.)
+constexpr int SRG_WAVES = 8;
+
+template <int DT_OUT, int MT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void mxfp_gemm_scaled_rows_regs_kernel(
+    const uint8_t* __restrict__ a_codes, const uint32_t* __restrict__ a_scales, const uint8_t* __restrict__ w_codes,
+    const uint32_t* __restrict__ w_scales, const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int rows_a,
+    int rows_w) {
+    constexpr int SPW = 32 / WAVES;          // macro steps of a unit per wavefront
+    constexpr int RPW = 16 / WAVES;          // rows of W a wavefront carries from global memory to LDS
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];            // W [16][SRR_ROW], partial sums [WAVES][MT][256]
+    uint8_t* const tile_w = lds;
+    float (*const red)[MT][256] = reinterpret_cast<float (*)[MT][256]>(lds + 16 * SRR_ROW);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 4, r = lane & 15;
+    const int nmac = K / 128;
+    const int groups = (N + 15) / 16;
+    const int units = ((int)blockIdx.x < groups) ? (groups - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    uint32_t off[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) off[q] = min(1024u * q + 16u * lane, (uint32_t)K - 16u);
+
+    intx4 wreg[RPW][4];
+    uint32_t w_sc_next[SPW];
+    auto issue = [&](int u) __attribute__((always_inline)) {
+        // (plain arithmetic: a unit past the end has pitch 0 and offset 0, every lane of a wavefront reads the same line)
+        const uint32_t live = u < units ? 1u : 0u;
+        const int group = (int)blockIdx.x + u * (int)gridDim.x;
+        const uint8_t* row0 = w_codes + (size_t)live * (size_t)(group * 16 + RPW * wave) * K;
+        const size_t pitch = (size_t)live * (size_t)K;
+#pragma unroll
+        for (int i = 0; i < RPW; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) wreg[i][q] = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(row0 + i * pitch + live * off[q]));
+#pragma unroll
+        for (int j = 0; j < SPW; ++j)
+            w_sc_next[j] = __builtin_nontemporal_load(w_scales + (size_t)live * ((size_t)min(SPW * wave + j, nmac - 1) * rows_w + group * 16 + r));
+    };
+    // ---- this wavefront's fragments of A and their scale bytes, once.  A tile takes W's route (whole 1 KB pieces of a row per
+    // load instruction, through LDS): read in the operand layout straight from global memory, 64 bytes of a row at a time,
+    // every cache line is fetched twice, and with every CU of an XCD asking for the same A that is what the prologue costs
+    // (a macro step past the end of K: the last one's bytes, under scale bytes 0 on W's side)
+    const uint8_t* const frag_w = tile_w + r * SRR_ROW + 16 * g;
+    intx8 af[MT][SPW];
+    uint32_t a_sc[MT][SPW], keep[SPW];
+#pragma unroll
+    for (int j = 0; j < SPW; ++j) keep[j] = SPW * wave + j < nmac ? 0xFFu : 0u;
+    intx4 areg[2][RPW][4];                                      // a tile's rows on their way to LDS, the next tile's behind them
+    auto load_a = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < RPW; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) areg[t & 1][i][q] = *reinterpret_cast<const intx4*>(a_codes + (size_t)(16 * t + RPW * wave + i) * K + off[q]);
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) a_sc[t][j] = a_scales[(size_t)min(SPW * wave + j, nmac - 1) * rows_a + 16 * t + r];
+    };
+    load_a(0);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < MT) load_a(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t > 0) __syncthreads();                              // the fragment reads of the tile before are done
+#pragma unroll
+        for (int i = 0; i < RPW; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *reinterpret_cast<intx4*>(tile_w + (RPW * wave + i) * SRR_ROW + 1024 * q + 16 * lane) = areg[t & 1][i][q];
+        if (t == MT - 1) {
+            __builtin_amdgcn_sched_barrier(0);
+            issue(0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) {
+            const int ms = min(SPW * wave + j, nmac - 1);
+            const intx4 lo = *reinterpret_cast<const intx4*>(frag_w + ms * 128), hi = *reinterpret_cast<const intx4*>(frag_w + ms * 128 + 64);
+            af[t][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            a_sc[t][j] = (a_sc[t][j] >> (8 * g)) & 0xFFu;
+        }
+    }
+    for (int u = 0; u < units; ++u) {
+        const int group = (int)blockIdx.x + u * (int)gridDim.x;
+        __syncthreads();                                         // the reads of the unit before (fragments, partial sums) are done
+#pragma unroll
+        for (int i = 0; i < RPW; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) *reinterpret_cast<intx4*>(tile_w + (RPW * wave + i) * SRR_ROW + 1024 * q + 16 * lane) = wreg[i][q];
+        uint32_t w_sc[SPW];
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) w_sc[j] = (w_sc_next[j] >> (8 * g)) & keep[j];
+        __builtin_amdgcn_sched_barrier(0);
+        issue(u + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        floatx4 acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < SPW; ++j) {
+            const int ms = SPW * wave + j;
+            const intx4 w_lo = *reinterpret_cast<const intx4*>(frag_w + ms * 128), w_hi = *reinterpret_cast<const intx4*>(frag_w + ms * 128 + 64);
+            const intx8 wf = __builtin_shufflevector(w_lo, w_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) mfma_scaled_after_valu(acc[t], wf, af[t][j], w_sc[j], a_sc[t][j]);
+        }
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");     // the matrix unit's last results have left its pipeline
+#pragma unroll
+        for (int t = 0; t < MT; ++t) *reinterpret_cast<floatx4*>(&red[wave][t][lane * 4]) = acc[t];
+        __syncthreads();
+        // wavefront t adds tile t (lane l holds n = 4 (l >> 4) + v, m = l & 15 of it) and stores it
+        if (wave < MT) {
+            const int t = wave;
+            floatx4 s = *reinterpret_cast<const floatx4*>(&red[0][t][lane * 4]);
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) s += *reinterpret_cast<const floatx4*>(&red[w][t][lane * 4]);
+            const int n = group * 16 + 4 * g, m = 16 * t + r;
+            if (m < M && n < N) {
+                float out[4] = {s[0], s[1], s[2], s[3]};
+                const int valid = min(4, N - n);
+                if (bias)
+                    for (int v = 0; v < valid; ++v) out[v] += load_bias(bias, bias_dtype, n + v);
+                store_out4<DT_OUT>(y, (int64_t)m * N + n, out, true, valid);
+            }
+        }
+    }
+}
+
+// the shapes these kernels take: up to 32 rows of A (two 16-row operand tiles), up to 64 when a wavefront's share of A fits
+// its registers
+inline bool scaled_rows_shape_ok(int M, int K) { return K >= 128 && (M <= 32 || (M <= 64 && K <= 4096)); }
 
 template <int DT_OUT>
 int launch_gemm_scaled_rows(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
@@ -284,6 +424,22 @@ int launch_gemm_scaled_rows(const uint8_t* a_codes, const uint32_t* a_scales, co
         hipLaunchKernelGGL(kern, dim3((unsigned)min((int)groups, cus)), dim3(256), lds_bytes, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N, K,
                            rows_a, rows_w);
         return check_launch("mxfp_gemm_scaled");
+    }
+    if (K <= 4096 && M > 16) {
+        // a wavefront's share of A stays in its registers: persistent workgroups of eight wavefronts, one per CU
+        const int cus = device_cu_count();
+        if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
+        auto go = [&](auto kern, int mt, std::atomic<uint64_t>& allowed) {
+            // (more than half a CU's LDS, so that no CU is given two of these workgroups while another has none)
+            const int lds_bytes = max(16 * SRR_ROW + SRG_WAVES * mt * 256 * (int)sizeof(float), 84 * 1024);
+            if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, allowed)) return rc;
+            hipLaunchKernelGGL(kern, dim3((unsigned)min((int)groups, cus)), dim3(SRG_WAVES * 64), lds_bytes, s, a_codes, a_scales, w_codes, w_scales, bias,
+                               bias_dtype, y, M, N, K, rows_a, rows_w);
+            return check_launch("mxfp_gemm_scaled");
+        };
+        static std::atomic<uint64_t> allowed2{0}, allowed4{0};
+        if (M <= 32) return go(mxfp_gemm_scaled_rows_regs_kernel<DT_OUT, 2, SRG_WAVES>, 2, allowed2);
+        return go(mxfp_gemm_scaled_rows_regs_kernel<DT_OUT, 4, SRG_WAVES>, 4, allowed4);
     }
     if (M <= 16)
         hipLaunchKernelGGL((mxfp_gemm_scaled_rows_kernel<DT_OUT, 1, 4>), dim3(groups), dim3(256), 0, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y,

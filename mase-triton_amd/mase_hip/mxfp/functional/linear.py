@@ -44,15 +44,22 @@ _BACKENDS = ("separate", "fused", "fused_bf16", "fused_scaled")
 SCALED_FROM_ROWS = 64
 SCALED_FROM_ROWS_UNPREPARED = 512
 # ... and, with the weight operand at hand, the rows of x up to which it takes it as well: decode-sized calls are a read of
-# W, which the block-scaled weight-streaming kernel does without touching the codes (up to 16 rows, one operand tile of x:
-# 15 against 21 us at N x K = 14336 x 4096, 17 against 25 at 4096 x 14336; between 17 and 63 rows the bf16 kernels are ahead)
+# W, which the block-scaled weight-streaming kernels do without touching the codes.  Up to 16 rows (one operand tile of x)
+# for any K: 15 against 21 us at N x K = 14336 x 4096, 17 against 25 at 4096 x 14336.  Up to 64 rows when K <= 4096 (a
+# wavefront's share of x stays in its registers: 15.6 / 19.2 us at 32 / 64 rows of 14336 x 4096 against 23 / 31 us on the
+# bf16 kernels), which closes the gap to SCALED_FROM_ROWS: with K <= 4096 every row count takes this route.  With a longer K,
+# 17 to 63 rows stay on the bf16 kernels.
 SCALED_UP_TO_ROWS = 16
+SCALED_UP_TO_ROWS_SHORT_K = 64
+SHORT_K = 4096
 
 
-def takes_scaled_route(rows: int, prepared: bool) -> bool:
-    """Does backend="fused" take the block-scaled kernels for this many rows of x (given that the operands qualify)?"""
+def takes_scaled_route(rows: int, prepared: bool, in_features: int | None = None) -> bool:
+    """Does backend="fused" take the block-scaled kernels for this many rows of x (given that the operands qualify)?
+    ``in_features``: K of the product, where known."""
     if prepared:
-        return rows >= SCALED_FROM_ROWS or 1 <= rows <= SCALED_UP_TO_ROWS
+        up_to = SCALED_UP_TO_ROWS_SHORT_K if in_features is not None and in_features <= SHORT_K else SCALED_UP_TO_ROWS
+        return rows >= SCALED_FROM_ROWS or 1 <= rows <= up_to
     return rows >= SCALED_FROM_ROWS_UNPREPARED
 
 
@@ -145,7 +152,7 @@ def mxfp_linear(
     # ---- fused
     rows = x.numel() // x.shape[-1] if x.numel() else 0
     if quantised_x and quantised_w and backend != "fused_bf16" and _scaled_eligible(x, x_meta, w_tensor_meta, bias):
-        if backend == "fused_scaled" or takes_scaled_route(rows, w_operand is not None):
+        if backend == "fused_scaled" or takes_scaled_route(rows, w_operand is not None, x.shape[-1]):
             out_features, in_features = w_tensor_meta.shape
             assert x.shape[-1] == in_features
             a_op = kernels.scaled_operand_from_dense(x.reshape(-1, in_features), x_meta)

@@ -323,13 +323,26 @@ def test_minifloat_layer_routes(mf, monkeypatch):
     g = torch.Generator().manual_seed(21)
     layer = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")
     separate = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "separate")
-    for rows, scaled in ((SCALED_FROM_ROWS, True), (SCALED_UP_TO_ROWS, True), (SCALED_UP_TO_ROWS + 8, False), (4 * SCALED_FROM_ROWS, True)):
+    for rows in (SCALED_FROM_ROWS, SCALED_UP_TO_ROWS, SCALED_UP_TO_ROWS + 8, 4 * SCALED_FROM_ROWS):
         before = dict(calls)
         x = torch.randn(rows, K, generator=g).to(torch.bfloat16).to(DEV)
         y = layer(x)
-        assert (calls["scaled"] - before["scaled"], calls["bf16"] - before["bf16"]) == ((1, 0) if scaled else (0, 1)), rows
+        assert (calls["scaled"] - before["scaled"], calls["bf16"] - before["bf16"]) == (1, 0), rows
         assert rel_fro(y, separate(x)) <= REL_FRO_TOL
     assert calls["prepare"] == 1
+    # a K beyond what the weight-streaming kernels keep in registers: 17 to 63 rows stay on the bf16 kernels
+    lin_long = torch.nn.Linear(4608, N, bias=False, dtype=torch.bfloat16, device=DEV)
+    with torch.no_grad():
+        lin_long.weight.mul_(16)
+    long_k = mf.Layer.from_linear(lin_long, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")
+    long_sep = mf.Layer.from_linear(lin_long, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "separate")
+    for rows, scaled in ((SCALED_UP_TO_ROWS, True), (SCALED_UP_TO_ROWS + 8, False), (SCALED_FROM_ROWS, True)):
+        before = dict(calls)
+        x = torch.randn(rows, 4608, generator=g).to(torch.bfloat16).to(DEV)
+        y = long_k(x)
+        assert (calls["scaled"] - before["scaled"], calls["bf16"] - before["bf16"]) == ((1, 0) if scaled else (0, 1)), rows
+        assert rel_fro(y, long_sep(x)) <= REL_FRO_TOL
+    calls["prepare"] = 1
     x = torch.randn(128, K, generator=g).to(torch.bfloat16).to(DEV)
     y_before = layer(x)
     with torch.no_grad():

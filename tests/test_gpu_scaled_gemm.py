@@ -273,13 +273,16 @@ def test_scaled_gemm_many_tiles(mh, MNK):
     assert float(err.max()) <= 1e-3 * float(y_ref.double().abs().max())
 
 
-@pytest.mark.parametrize("MNK", [(1, 4096, 4096), (7, 520, 1024), (16, 14336, 512), (17, 264, 2304), (32, 1032, 14336), (3, 8, 512)])
+@pytest.mark.parametrize("MNK", [(1, 4096, 4096), (7, 520, 1024), (16, 14336, 512), (17, 264, 2304), (32, 1032, 14336), (3, 8, 512),
+                                 (17, 4104, 4096), (32, 14336, 4096), (33, 520, 768), (48, 4096, 3840), (49, 8, 512), (64, 4120, 4096),
+                                 (24, 40, 4352), (64, 6160, 2048)])
 @pytest.mark.parametrize("x_tag,w_tag", [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP4_E2M1")])
 def test_scaled_gemm_few_rows(mh, MNK, x_tag, w_tag):
-    """Up to 32 rows of x: the weight-streaming kernel (a workgroup per 16 rows of W, its wavefronts taking the macro steps
-    of K in turn and adding their partial sums through LDS).  Row counts on both sides of its 16-row operand tiles, N that
-    is not a multiple of 16, K with fewer macro steps than a workgroup has wavefronts and with a count they do not divide;
-    bias and every output type."""
+    """Up to 64 rows of x: the weight-streaming kernels (a workgroup per 16 rows of W, its wavefronts taking the macro steps
+    of K in turn and adding their partial sums through LDS; x in LDS up to 16 rows, in registers from 17 to 64 when K <= 4096,
+    streamed beside W for a longer K up to 32 rows).  Row counts on both sides of the 16-row operand tiles, N that is not a
+    multiple of 16, more and fewer row groups of W than the chip has CUs, K with fewer macro steps than a workgroup has
+    wavefronts and with a count they do not divide; bias and every output type."""
     M, N, K = MNK
     g = torch.Generator().manual_seed(M * 7 + N + K)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -309,8 +312,8 @@ def test_scaled_gemm_random_shapes(mh):
 
     rng = random.Random(1234)
     pairs = [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP6_E3M2"), ("OCP_MXFP6_E2M3", "OCP_MXFP4_E2M1")]
-    for case in range(24):
-        M = rng.choice([rng.randint(1, 32), rng.randint(33, 300), rng.randint(301, 700)])
+    for case in range(32):
+        M = rng.choice([rng.randint(1, 32), rng.randint(17, 64), rng.randint(65, 300), rng.randint(301, 700)])
         N = 8 * rng.randint(1, 130)
         K = 256 * rng.randint(2, 12)
         x_tag, w_tag = pairs[case % len(pairs)]
