@@ -401,6 +401,8 @@ int launch_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, const u
     if (tiles >= (1 << 26)) return fail(ERR_UNSUPPORTED, "too many tiles");
     const int cus = device_cu_count();
     if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
+    if (const int slices = scaled_rows_slices(M, N, K); slices > 0 && workspace && workspace_bytes >= (int64_t)slices * M * N * 4)
+        return launch_gemm_scaled_rows_sliced<DT_OUT>(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N, K, static_cast<float*>(workspace), s);
     if (scaled_rows_shape_ok(M, K)) return launch_gemm_scaled_rows<DT_OUT>(a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N, K, s);
     int splits = workspace ? plan_scaled_splits(M, N, K, cus) : 1;
     const int64_t mn = (int64_t)M * N;

@@ -39,6 +39,7 @@ extern "C" int mase_hip_mxfp_gemm_scaled_ws(const uint8_t* a_codes, const uint32
 
 extern "C" int64_t mase_hip_mxfp_gemm_scaled_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M < 1 || N < 1 || K < 512 || K % 256 != 0 || M > 0x7FFFFFFF || N > 0x7FFFFFFF || K >= ((int64_t)1 << 27)) return 0;
+    if (const int slices = scaled_rows_slices((int)M, (int)N, (int)K)) return (int64_t)slices * M * N * 4;
     const int splits = plan_scaled_splits((int)M, (int)N, (int)K, device_cu_count());
     return splits > 1 ? (int64_t)splits * M * N * 4 : 0;
 }

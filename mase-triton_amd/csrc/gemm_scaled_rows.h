@@ -282,7 +282,7 @@ template <int DT_OUT, int MT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void mxfp_gemm_scaled_rows_regs_kernel(
     const uint8_t* __restrict__ a_codes, const uint32_t* __restrict__ a_scales, const uint8_t* __restrict__ w_codes,
     const uint32_t* __restrict__ w_scales, const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int rows_a,
-    int rows_w) {
+    int rows_w, int slices, int slice_macs, float* __restrict__ partial) {
     constexpr int SPW = 32 / WAVES;          // macro steps of a unit per wavefront
     constexpr int RPW = 16 / WAVES;          // rows of W a wavefront carries from global memory to LDS
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];            // W [16][SRR_ROW], partial sums [WAVES][MT][256]
@@ -291,19 +291,30 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 4, r = lane & 15;
-    const int nmac = K / 128;
+    // A K beyond 4096 is cut into `slices` pieces of `slice_macs` macro steps (the last one may be shorter): a workgroup stays
+    // with ONE slice (its share of A in registers is that slice's) and walks the row groups of W with the workgroups of the
+    // same slice; the slices' sums go to `partial` [slices][M][N] as fp32 and a second kernel adds them.  slices == 1: the
+    // whole K, results straight to y.
+    const int slice = (int)blockIdx.x % slices, first_group = (int)blockIdx.x / slices, group_step = (int)gridDim.x / slices;
+    const int mac0 = slice * slice_macs;
+    const int nmac = min(slice_macs, K / 128 - mac0);            // this slice's macro steps: at most 32
+    const size_t k0 = (size_t)mac0 * 128;
     const int groups = (N + 15) / 16;
-    const int units = ((int)blockIdx.x < groups) ? (groups - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    const int units = first_group < groups ? (groups - first_group + group_step - 1) / group_step : 0;
     uint32_t off[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) off[q] = min(1024u * q + 16u * lane, (uint32_t)K - 16u);
+    for (int q = 0; q < 4; ++q) off[q] = min(1024u * q + 16u * lane, (uint32_t)nmac * 128u - 16u);
+    a_codes += k0;
+    w_codes += k0;
+    a_scales += (size_t)mac0 * rows_a;
+    w_scales += (size_t)mac0 * rows_w;
 
     intx4 wreg[RPW][4];
     uint32_t w_sc_next[SPW];
     auto issue = [&](int u) __attribute__((always_inline)) {
         // (plain arithmetic: a unit past the end has pitch 0 and offset 0, every lane of a wavefront reads the same line)
         const uint32_t live = u < units ? 1u : 0u;
-        const int group = (int)blockIdx.x + u * (int)gridDim.x;
+        const int group = first_group + u * group_step;
         const uint8_t* row0 = w_codes + (size_t)live * (size_t)(group * 16 + RPW * wave) * K;
         const size_t pitch = (size_t)live * (size_t)K;
 #pragma unroll
@@ -358,7 +369,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
         }
     }
     for (int u = 0; u < units; ++u) {
-        const int group = (int)blockIdx.x + u * (int)gridDim.x;
+        const int group = first_group + u * group_step;
         __syncthreads();                                         // the reads of the unit before (fragments, partial sums) are done
 #pragma unroll
         for (int i = 0; i < RPW; ++i)
@@ -396,9 +407,14 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
             if (m < M && n < N) {
                 float out[4] = {s[0], s[1], s[2], s[3]};
                 const int valid = min(4, N - n);
-                if (bias)
-                    for (int v = 0; v < valid; ++v) out[v] += load_bias(bias, bias_dtype, n + v);
-                store_out4<DT_OUT>(y, (int64_t)m * N + n, out, true, valid);
+                if (partial) {
+                    float* const dst = partial + ((size_t)slice * M + m) * N + n;
+                    for (int v = 0; v < valid; ++v) dst[v] = out[v];
+                } else {
+                    if (bias)
+                        for (int v = 0; v < valid; ++v) out[v] += load_bias(bias, bias_dtype, n + v);
+                    store_out4<DT_OUT>(y, (int64_t)m * N + n, out, true, valid);
+                }
             }
         }
     }
@@ -407,6 +423,40 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
 // the shapes these kernels take: up to 32 rows of A (two 16-row operand tiles), up to 64 when a wavefront's share of A fits
 // its registers
 inline bool scaled_rows_shape_ok(int M, int K) { return K >= 128 && (M <= 32 || (M <= 64 && K <= 4096)); }
+
+// K beyond what a wavefront's registers hold of A in one piece, 17 - 64 rows: slices of at most 32 macro steps, their sums added
+// by a second kernel (room for them: slices * M * N * 4 bytes).  0: not a shape for this.  N x K = 4096 x 14336: 18.4 / 23.0 us
+// at 32 / 64 rows against 23.3 (the chunked kernel) / 31.0 (the tile kernel, K split) and 27.8 / 49.4 on the bf16 kernels; 8192 x
+// 8192: 19.4 / 24.4 against 23.2 / 30.2 and 29.5 / 42.6.  (Up to 16 rows the chunked kernel is level: 17.7 us, one launch.)
+inline int scaled_rows_slices(int M, int N, int K) {
+    if (M <= 16 || M > 64 || K <= 4096 || K % 128 != 0 || N % 4 != 0) return 0;
+    return (K / 128 + 31) / 32;
+}
+
+template <int DT_OUT>
+int launch_gemm_scaled_rows_sliced(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
+                                   int bias_dtype, void* y, int M, int N, int K, float* partial, hipStream_t s) {
+    const int rows_a = (M + 255) / 256 * 256, rows_w = (N + 255) / 256 * 256;
+    const int groups = (N + 15) / 16, slices = scaled_rows_slices(M, N, K), slice_macs = (K / 128 + slices - 1) / slices;
+    const int cus = device_cu_count();
+    if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
+    auto go = [&](auto kern, int mt, std::atomic<uint64_t>& allowed) {
+        const int lds_bytes = max(16 * SRR_ROW + SRG_WAVES * mt * 256 * (int)sizeof(float), 84 * 1024);
+        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, allowed)) return rc;
+        // as many workgroups per slice as fill the CUs between them (every slice the same count)
+        const int per_slice = max(1, min(groups, cus / slices));
+        hipLaunchKernelGGL(kern, dim3((unsigned)(per_slice * slices)), dim3(SRG_WAVES * 64), lds_bytes, s, a_codes, a_scales, w_codes, w_scales,
+                           static_cast<const void*>(nullptr), 0, static_cast<void*>(nullptr), M, N, K, rows_a, rows_w, slices, slice_macs, partial);
+        return check_launch("mxfp_gemm_scaled");
+    };
+    static std::atomic<uint64_t> allowed2{0}, allowed4{0};
+    if (int rc = M <= 32 ? go(mxfp_gemm_scaled_rows_regs_kernel<F32, 2, SRG_WAVES>, 2, allowed2) : go(mxfp_gemm_scaled_rows_regs_kernel<F32, 4, SRG_WAVES>, 4, allowed4))
+        return rc;
+    const int64_t mn = (int64_t)M * N;
+    hipLaunchKernelGGL(split_k_reduce_kernel<DT_OUT>, dim3((unsigned)((mn / 4 + 255) / 256)), dim3(256), 0, s, static_cast<const float*>(partial), slices, mn, N, bias,
+                       bias_dtype, y);
+    return check_launch("mxfp_gemm_scaled");
+}
 
 template <int DT_OUT>
 int launch_gemm_scaled_rows(const uint8_t* a_codes, const uint32_t* a_scales, const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
@@ -434,7 +484,7 @@ int launch_gemm_scaled_rows(const uint8_t* a_codes, const uint32_t* a_scales, co
             const int lds_bytes = max(16 * SRR_ROW + SRG_WAVES * mt * 256 * (int)sizeof(float), 84 * 1024);
             if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, allowed)) return rc;
             hipLaunchKernelGGL(kern, dim3((unsigned)min((int)groups, cus)), dim3(SRG_WAVES * 64), lds_bytes, s, a_codes, a_scales, w_codes, w_scales, bias,
-                               bias_dtype, y, M, N, K, rows_a, rows_w);
+                               bias_dtype, y, M, N, K, rows_a, rows_w, 1, K / 128, static_cast<float*>(nullptr));
             return check_launch("mxfp_gemm_scaled");
         };
         static std::atomic<uint64_t> allowed2{0}, allowed4{0};

@@ -149,7 +149,7 @@ def minifloat_linear(
             raise NotImplementedError("fused_scaled: this product does not fit the block-scaled GEMM (bfloat16 x, formats E4M3 / "
                                       "E3M2 / E2M3 / E2M1 rounded to nearest, K a multiple of 256 and at least 512, N of 8)")
         rows = x.numel() // x.shape[-1] if x.numel() else 0
-        if ok and (backend == "fused_scaled" or takes_scaled_route(rows, _w_operand is not None, x.shape[-1])):
+        if ok and (backend == "fused_scaled" or takes_scaled_route(rows, _w_operand is not None)):
             if _w_operand is None:
                 _w_operand = scaled_weight_operand(w_element, w_tensor_meta, _narrowed)
             a_op = mxfp_kernels.scaled_operand_from_dense_minifloat(x.reshape(-1, x.shape[-1]), x_meta.exp_bits, x_meta.frac_bits)

@@ -127,7 +127,7 @@ class MinifloatLinearPTQ(nn.Module):
             return None
         rows = input.numel() // input.shape[-1] if input.numel() else 0
         bias = self.bias if not self.layer_type.endswith("Bq") else None
-        if not ((self.backend == "fused_scaled" or takes_scaled_route(rows, True, self.in_features))
+        if not ((self.backend == "fused_scaled" or takes_scaled_route(rows, True))
                 and L._scaled_eligible(input, self.x_minifloat_meta, self.w_tensor_meta, bias)):
             return None
         key = (w.data_ptr(), w._version, w.device)

@@ -36,31 +36,19 @@ from .cast import compose_mxfp_tensor, extract_mxfp_components, quantize_dequant
 _LAYER_TYPES = ("XWB", "XWBq", "XWqB", "XWqBq", "XqWB", "XqWBq", "XqWqB", "XqWqBq")
 _GEMM_DTYPES = (torch.bfloat16, torch.float32)
 _BACKENDS = ("separate", "fused", "fused_bf16", "fused_scaled")
-# rows of x from which "fused" takes the block-scaled route.  With the weight operand at hand (a layer keeps it) the
-# block-scaled kernel, K split over workgroups where its 256 x 256 tiles are few, is level with the weight-streaming bf16
-# kernels at 64 rows and ahead from there (N x K = 14336 x 4096: 30 / 33 / 44 / 45 us at 64 / 128 / 256 / 512 rows against
-# 30 / 37 / 49 / 73 us); when the operand has to be built inside the call (N * K bytes read and written, 25 us there) it
-# pays from about 512 rows (71 against 73 us; 72 against 104 at 768)
-SCALED_FROM_ROWS = 64
+# Which row counts of x backend="fused" sends to the block-scaled kernels.  With the weight operand at hand (a layer keeps
+# it): all of them.  Up to 64 rows the product is a read of W, which the block-scaled weight-streaming kernels do without
+# touching the codes (N x K = 14336 x 4096: 15 / 15.6 / 19.2 us at 16 / 32 / 64 rows against 21 / 23 / 31 us on the bf16
+# kernels; 4096 x 14336: 17.7 / 18.4 / 23.0 against 25.8 / 27.8 / 49.4); beyond, its 256 x 256 tiles, K split over workgroups where
+# they are few, stay ahead (14336 x 4096: 33 / 44 / 45 us at 128 / 256 / 512 rows against 37 / 49 / 73).  When the operand has to
+# be built inside the call (N * K bytes read and written, 25 us at that size) it pays from about 512 rows (71 against 73 us;
+# 72 against 104 at 768).
 SCALED_FROM_ROWS_UNPREPARED = 512
-# ... and, with the weight operand at hand, the rows of x up to which it takes it as well: decode-sized calls are a read of
-# W, which the block-scaled weight-streaming kernels do without touching the codes.  Up to 16 rows (one operand tile of x)
-# for any K: 15 against 21 us at N x K = 14336 x 4096, 17 against 25 at 4096 x 14336.  Up to 64 rows when K <= 4096 (a
-# wavefront's share of x stays in its registers: 15.6 / 19.2 us at 32 / 64 rows of 14336 x 4096 against 23 / 31 us on the
-# bf16 kernels), which closes the gap to SCALED_FROM_ROWS: with K <= 4096 every row count takes this route.  With a longer K,
-# 17 to 63 rows stay on the bf16 kernels.
-SCALED_UP_TO_ROWS = 16
-SCALED_UP_TO_ROWS_SHORT_K = 64
-SHORT_K = 4096
 
 
-def takes_scaled_route(rows: int, prepared: bool, in_features: int | None = None) -> bool:
-    """Does backend="fused" take the block-scaled kernels for this many rows of x (given that the operands qualify)?
-    ``in_features``: K of the product, where known."""
-    if prepared:
-        up_to = SCALED_UP_TO_ROWS_SHORT_K if in_features is not None and in_features <= SHORT_K else SCALED_UP_TO_ROWS
-        return rows >= SCALED_FROM_ROWS or 1 <= rows <= up_to
-    return rows >= SCALED_FROM_ROWS_UNPREPARED
+def takes_scaled_route(rows: int, prepared: bool) -> bool:
+    """Does backend="fused" take the block-scaled kernels for this many rows of x (given that the operands qualify)?"""
+    return rows >= (1 if prepared else SCALED_FROM_ROWS_UNPREPARED)
 
 
 def parse_mxfp_linear_type(x_meta: MXFPMeta | None, w_tensor_meta: MXFPTensorMeta | None,
@@ -152,7 +140,7 @@ def mxfp_linear(
     # ---- fused
     rows = x.numel() // x.shape[-1] if x.numel() else 0
     if quantised_x and quantised_w and backend != "fused_bf16" and _scaled_eligible(x, x_meta, w_tensor_meta, bias):
-        if backend == "fused_scaled" or takes_scaled_route(rows, w_operand is not None, x.shape[-1]):
+        if backend == "fused_scaled" or takes_scaled_route(rows, w_operand is not None):
             out_features, in_features = w_tensor_meta.shape
             assert x.shape[-1] == in_features
             a_op = kernels.scaled_operand_from_dense(x.reshape(-1, in_features), x_meta)

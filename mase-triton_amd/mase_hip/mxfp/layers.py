@@ -123,7 +123,7 @@ class MXFPLinearPTQ(nn.Module):
             return False
         rows = input.numel() // input.shape[-1] if input.numel() else 0
         bias = self.bias if not self.layer_type.endswith("Bq") else None
-        return ((self.backend == "fused_scaled" or L.takes_scaled_route(rows, True, self.in_features))
+        return ((self.backend == "fused_scaled" or L.takes_scaled_route(rows, True))
                 and L._scaled_eligible(input, self.x_mxfp_meta, self.w_tensor_meta, bias))
 
     def _weight_operand(self, input: Tensor):

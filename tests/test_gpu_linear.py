@@ -513,34 +513,28 @@ def test_config_c4_full_size(mh, backend):
 
 
 def test_fused_backend_picks_the_kernel_family_by_rows(mh):
-    """backend="fused": the bf16 kernels below the row thresholds (bit-identical to "fused_bf16"), the block-scaled
-    kernel from there on (bit-identical to "fused_scaled"); with a prepared weight operand the threshold is the lower
-    one, and decode-sized calls (up to SCALED_UP_TO_ROWS rows, SCALED_UP_TO_ROWS_SHORT_K when K <= SHORT_K) take the block-scaled
-    weight-streaming kernels as well.
-    Every result within the tolerance of the float64 checker."""
+    """backend="fused": without a prepared weight operand the bf16 kernels below SCALED_FROM_ROWS_UNPREPARED rows
+    (bit-identical to "fused_bf16") and the block-scaled kernels from there on (bit-identical to "fused_scaled"); with the
+    operand at hand the block-scaled kernels at every row count, for a K its weight-streaming kernels take in one piece and
+    for a longer one.  Every result within the tolerance of the float64 checker."""
     from mase_hip.mxfp.functional import linear as lin
 
     fmt = preset(mh, "MXFP8_E4M3_fn")
     g = torch.Generator().manual_seed(11)
-    for K in (512, lin.SHORT_K + 512):
+    for K in (512, 4608):
         w = torch.randn(256, K, generator=g).mul(0.02).to(torch.bfloat16)
         w_sc, w_el, w_tm = mh.F.extract_mxfp_components(w.to(DEV), block_dim=1, mxfp_meta=fmt)
         w_op = lin.scaled_weight_operand(w_sc, w_el, w_tm)
         w_dq = oracle.qdq_mxfp(w, 32, 4, 3)
-        # with the operand at hand: every row count when K is short (the weight-streaming kernels reach 64 rows there),
-        # else up to 16 and from 64
-        up_to = lin.SCALED_UP_TO_ROWS_SHORT_K if K <= lin.SHORT_K else lin.SCALED_UP_TO_ROWS
-        for rows in (1, lin.SCALED_UP_TO_ROWS, lin.SCALED_UP_TO_ROWS + 1, 33, lin.SCALED_FROM_ROWS - 8, lin.SCALED_FROM_ROWS,
-                     lin.SCALED_FROM_ROWS_UNPREPARED - 8, lin.SCALED_FROM_ROWS_UNPREPARED):
+        for rows in (1, 16, 17, 33, 56, 64, lin.SCALED_FROM_ROWS_UNPREPARED - 8, lin.SCALED_FROM_ROWS_UNPREPARED):
             x = torch.randn(rows, K, generator=g).to(torch.bfloat16)
             args = dict(x=x.to(DEV), x_meta=fmt, w=None, w_scales=w_sc, w_elements=w_el, w_tensor_meta=w_tm, b=None, b_scales=None,
                         b_elements=None, b_tensor_meta=None, layer_type="XqWqB")
             y_bf16 = mh.F.mxfp_linear(**args, backend="fused_bf16")
             y_scaled = mh.F.mxfp_linear(**args, backend="fused_scaled")
             assert torch.equal(mh.F.mxfp_linear(**args, backend="fused"), y_scaled if rows >= lin.SCALED_FROM_ROWS_UNPREPARED else y_bf16)
-            assert torch.equal(mh.F.mxfp_linear(**args, backend="fused", w_operand=w_op),
-                               y_scaled if rows >= lin.SCALED_FROM_ROWS or rows <= up_to else y_bf16), (K, rows)
-            assert lin.takes_scaled_route(rows, True, K) == (rows >= lin.SCALED_FROM_ROWS or rows <= up_to)
+            assert torch.equal(mh.F.mxfp_linear(**args, backend="fused", w_operand=w_op), y_scaled), (K, rows)
+            assert lin.takes_scaled_route(rows, True) and lin.takes_scaled_route(rows, False) == (rows >= lin.SCALED_FROM_ROWS_UNPREPARED)
             y_ref = oracle.matmul_nt(oracle.qdq_mxfp(x, 32, 4, 3), w_dq).to(torch.bfloat16)
             assert rel_fro(y_bf16, y_ref) <= REL_FRO_TOL
             assert rel_fro(y_scaled, y_ref) <= REL_FRO_TOL
@@ -564,12 +558,12 @@ def test_layer_keeps_and_refreshes_its_weight_operand(mh):
     sep = mh.MXFPLinearPTQ.from_linear(lin, fmt, wfmt, None, "XqWqB", "separate")
     small = torch.randn(40, 512, generator=g).to(torch.bfloat16).to(DEV)
     big = torch.randn(3, 200, 512, generator=g).to(torch.bfloat16).to(DEV)
-    long_k = mh.MXFPLinearPTQ.from_linear(torch.nn.Linear(4608, 264, bias=False, dtype=torch.bfloat16, device=DEV), fmt, wfmt, None, "XqWqB", "fused")
-    long_k(torch.randn(40, 4608, generator=g).to(torch.bfloat16).to(DEV))
-    assert long_k._scaled_w is None             # between 17 and 63 rows of a long K: the bf16 kernels, nothing cached
+    bf16_only = mh.MXFPLinearPTQ.from_linear(lin, fmt, wfmt, None, "XqWqB", "fused_bf16")
+    bf16_only(small)
+    assert bf16_only._scaled_w is None          # 40 rows on the bf16 kernels: no kernel there reads it, nothing cached
     assert layer._scaled_w is None
     layer(small)
-    assert layer._scaled_w is not None          # K <= 4096: the weight-streaming block-scaled kernel
+    assert layer._scaled_w is not None
     layer.invalidate_weight_operand()
     y = layer(big)
     first = layer._scaled_w

@@ -299,10 +299,9 @@ def test_minifloat_linear_scaled_vs_checker(mf, x_tag, w_tag, MNK):
 
 
 def test_minifloat_layer_routes(mf, monkeypatch):
-    """Which GEMM a layer's call takes: the block-scaled one for quantised bf16 activations in its formats at the row
-    counts of ``takes_scaled_route``, the bf16 one otherwise; the weight operand is built once and follows the codes."""
+    """Which GEMM a layer's call takes: the block-scaled one for quantised bf16 activations in its formats (every row
+    count: the layer keeps the weight operand), the bf16 one otherwise; the weight operand is built once and follows the codes."""
     from mase_hip.mxfp import kernels as K_
-    from mase_hip.mxfp.functional.linear import SCALED_FROM_ROWS, SCALED_UP_TO_ROWS
 
     calls = {"scaled": 0, "bf16": 0, "prepare": 0}
     real_scaled, real_bf16, real_prepare = K_.mxfp_gemm_scaled, K_.mxfp_gemm, K_.scaled_operand_from_mxfp
@@ -323,24 +322,24 @@ def test_minifloat_layer_routes(mf, monkeypatch):
     g = torch.Generator().manual_seed(21)
     layer = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")
     separate = mf.Layer.from_linear(lin, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "separate")
-    for rows in (SCALED_FROM_ROWS, SCALED_UP_TO_ROWS, SCALED_UP_TO_ROWS + 8, 4 * SCALED_FROM_ROWS):
+    for rows in (64, 16, 24, 256):
         before = dict(calls)
         x = torch.randn(rows, K, generator=g).to(torch.bfloat16).to(DEV)
         y = layer(x)
         assert (calls["scaled"] - before["scaled"], calls["bf16"] - before["bf16"]) == (1, 0), rows
         assert rel_fro(y, separate(x)) <= REL_FRO_TOL
     assert calls["prepare"] == 1
-    # a K beyond what the weight-streaming kernels keep in registers: 17 to 63 rows stay on the bf16 kernels
+    # ... also with a K beyond what the weight-streaming kernels take in one piece
     lin_long = torch.nn.Linear(4608, N, bias=False, dtype=torch.bfloat16, device=DEV)
     with torch.no_grad():
         lin_long.weight.mul_(16)
     long_k = mf.Layer.from_linear(lin_long, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "fused")
     long_sep = mf.Layer.from_linear(lin_long, mf.meta.FP8_E4M3_fn, mf.meta.FP6_E3M2_fn, None, "XqWqB", "separate")
-    for rows, scaled in ((SCALED_UP_TO_ROWS, True), (SCALED_UP_TO_ROWS + 8, False), (SCALED_FROM_ROWS, True)):
+    for rows in (16, 24, 64):
         before = dict(calls)
         x = torch.randn(rows, 4608, generator=g).to(torch.bfloat16).to(DEV)
         y = long_k(x)
-        assert (calls["scaled"] - before["scaled"], calls["bf16"] - before["bf16"]) == ((1, 0) if scaled else (0, 1)), rows
+        assert (calls["scaled"] - before["scaled"], calls["bf16"] - before["bf16"]) == (1, 0), rows
         assert rel_fro(y, long_sep(x)) <= REL_FRO_TOL
     calls["prepare"] = 1
     x = torch.randn(128, K, generator=g).to(torch.bfloat16).to(DEV)

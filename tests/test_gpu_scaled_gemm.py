@@ -275,12 +275,13 @@ def test_scaled_gemm_many_tiles(mh, MNK):
 
 @pytest.mark.parametrize("MNK", [(1, 4096, 4096), (7, 520, 1024), (16, 14336, 512), (17, 264, 2304), (32, 1032, 14336), (3, 8, 512),
                                  (17, 4104, 4096), (32, 14336, 4096), (33, 520, 768), (48, 4096, 3840), (49, 8, 512), (64, 4120, 4096),
-                                 (24, 40, 4352), (64, 6160, 2048)])
+                                 (24, 40, 4352), (64, 6160, 2048), (64, 4096, 14336), (40, 264, 8192), (17, 8, 4608)])
 @pytest.mark.parametrize("x_tag,w_tag", [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP4_E2M1")])
 def test_scaled_gemm_few_rows(mh, MNK, x_tag, w_tag):
     """Up to 64 rows of x: the weight-streaming kernels (a workgroup per 16 rows of W, its wavefronts taking the macro steps
-    of K in turn and adding their partial sums through LDS; x in LDS up to 16 rows, in registers from 17 to 64 when K <= 4096,
-    streamed beside W for a longer K up to 32 rows).  Row counts on both sides of the 16-row operand tiles, N that is not a
+    of K in turn and adding their partial sums through LDS; x in LDS up to 16 rows, in registers from 17 to 64, a K beyond
+    4096 cut into slices whose sums a second kernel adds (the Python wrapper brings the room for them), streamed beside W
+    up to 16 rows).  Row counts on both sides of the 16-row operand tiles, N that is not a
     multiple of 16, more and fewer row groups of W than the chip has CUs, K with fewer macro steps than a workgroup has
     wavefronts and with a count they do not divide; bias and every output type."""
     M, N, K = MNK
@@ -296,6 +297,8 @@ def test_scaled_gemm_few_rows(mh, MNK, x_tag, w_tag):
     y32 = mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.float32)
     assert y32.shape == (M, N)
     assert rel_fro(y32, y_ref) <= F32_TOL
+    # without room for partial sums (the C entry point without a workspace): the kernels that need none
+    assert rel_fro(mh.mxk.mxfp_gemm_scaled(a, wop, None, torch.float32, split_k=False), y_ref) <= F32_TOL
     err = (y32.cpu().double() - y_ref).abs().max()
     assert float(err) <= 1e-3 * float(y_ref.abs().max())
     y_b = y_ref + b.double()
