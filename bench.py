@@ -452,27 +452,29 @@ def bench_hbm(torch, with_cpu):
 
     x_cpu, w_cpu = workloads.make_c4()
     N, K = w_cpu.shape
-    x16 = x_cpu[:16].contiguous().to(dev)
+    x64 = x_cpu[:64].contiguous().to(dev)
     w_sc, w_el = kernels.extract_mxfp_components(w_cpu.to(dev).reshape(-1), MXFP8_E4M3_fn)
     del x_cpu, w_cpu
     comps = [(w_sc, w_el)] + [(w_sc.clone(), w_el.clone()) for _ in range(6)]
     wops = [kernels.scaled_operand_from_mxfp(sc, el, MXFP8_E4M3_fn, N, K) for sc, el in comps]
-    a_op = kernels.scaled_operand_from_dense(x16, MXFP8_E4M3_fn)
-    a_dq = kernels.quantize_dequantize(x16.view(-1), MXFP8_E4M3_fn, torch.bfloat16).view(16, K)
-    y16 = torch.empty(16, N, dtype=torch.bfloat16, device=dev)
-
-    def rows_gemm(i):
-        kernels.mxfp_gemm_scaled(a_op, wops[i], None, torch.bfloat16, out=y16)
-
-    def rows_gemm_bf16(i):
-        kernels.mxfp_gemm(a_dq, None, None, None, comps[i][0], comps[i][1], MXFP8_E4M3_fn, None, 16, N, K, torch.bfloat16, out=y16)
-
     w_bytes = N * K * (1 + 1 / 32)
-    for name, fn in (("mxfp_gemm_scaled_rows", rows_gemm), ("mxfp_gemm_skinny (bf16)", rows_gemm_bf16)):
-        avg, best = time_kernel(torch, fn, len(wops))
-        cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
-        roof(name, "C4 W x 16 rows", f"decode: 16 rows of C4's x against W [{N},{K}] MXFP8 E4M3, bf16 out (bytes = W's codes and scales)", w_bytes, avg, best, cavg,
-             ROWS_SOURCES if fn is rows_gemm else GEMM_SOURCES)
+    for rows in (16, 64):      # x in LDS up to 16 rows, in registers from 17 to 64
+        xr = x64[:rows].contiguous()
+        a_op = kernels.scaled_operand_from_dense(xr, MXFP8_E4M3_fn)
+        a_dq = kernels.quantize_dequantize(xr.view(-1), MXFP8_E4M3_fn, torch.bfloat16).view(rows, K)
+        y = torch.empty(rows, N, dtype=torch.bfloat16, device=dev)
+
+        def rows_gemm(i):
+            kernels.mxfp_gemm_scaled(a_op, wops[i], None, torch.bfloat16, out=y)
+
+        def rows_gemm_bf16(i):
+            kernels.mxfp_gemm(a_dq, None, None, None, comps[i][0], comps[i][1], MXFP8_E4M3_fn, None, rows, N, K, torch.bfloat16, out=y)
+
+        for name, fn in (("mxfp_gemm_scaled_rows", rows_gemm), ("mxfp_gemm_skinny (bf16)", rows_gemm_bf16)):
+            avg, best = time_kernel(torch, fn, len(wops))
+            cavg, _ = time_kernel(torch, lambda i: fn(0), 1)
+            roof(name, f"C4 W x {rows} rows", f"decode: {rows} rows of C4's x against W [{N},{K}] MXFP8 E4M3, bf16 out (bytes = W's codes and scales)", w_bytes,
+                 avg, best, cavg, ROWS_SOURCES if fn is rows_gemm else GEMM_SOURCES)
     return out
 
 
@@ -545,9 +547,9 @@ def shape_sweep(torch, MXFP_F, mxk, fmt, steps=30, warmup=15):
                         "fused_TFLOPs": round(2.0 * M * n_out * k_in / f_us / 1e6, 1)})
         return out
 
-    rows = linear_rows(N, K, (16, 64, 128, 256, 384, 512, 768, 1024, 2048, 4096, 8192))
-    rows_down = linear_rows(K, N, (16, 64, 256, 512, 1024, 2048, 4096))  # the transposed layer shape: few W rows, long K
-    rows_sq = linear_rows(K, K, (128, 256, 512, 1024, 2048, 4096))
+    rows = linear_rows(N, K, (16, 32, 64, 128, 256, 384, 512, 768, 1024, 2048, 4096, 8192))
+    rows_down = linear_rows(K, N, (16, 32, 64, 256, 512, 1024, 2048, 4096))  # the transposed layer shape: few W rows, long K
+    rows_sq = linear_rows(K, K, (32, 128, 256, 512, 1024, 2048, 4096))
     w = (0.02 * torch.randn(N, K, generator=gen, device=dev)).to(torch.bfloat16)
     n = w.numel()
     cast = {
@@ -647,10 +649,11 @@ def counter_probe(torch, MXFP_F, mxk, fmt8, fmt4):
         a_op = mxk.scaled_operand_from_dense(x, fmt8)
         w_op = L.scaled_weight_operand(w_sc, w_el, w_tm)
         mxk.mxfp_gemm_scaled(a_op, w_op, None, torch.bfloat16)
-    a16 = mxk.scaled_operand_from_dense(x[:16].contiguous(), fmt8)
+    a16, a64 = mxk.scaled_operand_from_dense(x[:16].contiguous(), fmt8), mxk.scaled_operand_from_dense(x[:64].contiguous(), fmt8)
     for _ in range(3):
-        mxk.mxfp_gemm_scaled(a16, w_op, None, torch.bfloat16)          # decode-sized: the weight-streaming kernel
-    del x, w, w_sc, w_el, a, a_op, w_op, a16
+        mxk.mxfp_gemm_scaled(a16, w_op, None, torch.bfloat16)          # decode-sized: the weight-streaming kernels
+        mxk.mxfp_gemm_scaled(a64, w_op, None, torch.bfloat16)
+    del x, w, w_sc, w_el, a, a_op, w_op, a16, a64
     # C5's kernels on the block-scaled route: gate + up GEMM, SwiGLU operand, down GEMM (after C4's launches of the same kernels)
     from mase_hip.mxfp.meta import MXFPMeta
 
@@ -701,8 +704,9 @@ COUNTER_ROWS = (
     ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", _M4 * _K4 * 2 + _N4 * _K4 * 33 // 32, _M4 * _N4 * 2, GEMM_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 gate+up", (_M5 + 2 * _I5) * _H5 * 33 // 32, _M5 * 2 * _I5 * 2, SCALED_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 down", (_M5 + _H5) * _I5 * 33 // 32, _M5 * _H5 * 2, SCALED_SOURCES),
-    ("scaled_from_dense_kernel|true>(", "scaled_operand_from_swiglu C5", _M5 * _I5 * 4, _M5 * _I5 * 33 // 32, CAST_SOURCES),
-    ("scaled_from_dense_kernel|false>(", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
+    ("mxfp_gemm_scaled_rows_regs_kernel", "mxfp_gemm_scaled_rows C4 W x 64 rows", _N4 * _K4 * 33 // 32 + 64 * _K4 * 33 // 32, 64 * _N4 * 2, ROWS_SOURCES),
+    ("scaled_from_dense_kernel|0>, 1>(", "scaled_operand_from_swiglu C5", _M5 * _I5 * 4, _M5 * _I5 * 33 // 32, CAST_SOURCES),
+    ("scaled_from_dense_kernel|0>, 0>(", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
     ("scaled_operand_kernel<mase::SFmt<4, 3", "scaled_operand_from_mxfp C4 W", _N4 * _K4 * 33 // 32, _N4 * _K4 * 33 // 32, CAST_SOURCES),
     ("mxfp_bf16_b32_kernel<mase::SFmt<4, 3|, 0>(", "extract_mxfp C1", _N1 * 2, _N1 + _N1 // 32, CAST_SOURCES),
     ("compose_mxfp_bf16_kernel<mase::SFmt<4, 3", "compose_mxfp C1", _N1 + _N1 // 32, _N1 * 2, CAST_SOURCES),

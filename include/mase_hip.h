@@ -282,8 +282,9 @@ int mase_hip_mxfp_gemm_static_ws(const void* a_dense, int a_dtype, const uint8_t
  *       y[M,N] = A[M,K] * W[N,K]^T (+ bias), A and W prepared as above with rows M and N.
  *
  * K % 256 == 0 and K >= 512; N a multiple of 8 (4 for fp32 output); codes and y 16-byte aligned.  Other shapes: -2,
- * use mase_hip_mxfp_gemm.  Up to 32 rows of A take a weight-streaming kernel (the product is a read of W), more rows
- * 256 x 256 tiles.
+ * use mase_hip_mxfp_gemm.  Up to 64 rows of A take weight-streaming kernels (the product is a read of W; 17 - 64 rows
+ * against a K beyond 4096 only through mase_hip_mxfp_gemm_scaled_ws, which brings the room for their K slices' sums),
+ * more rows 256 x 256 tiles.
  * Replaces, like mase_hip_mxfp_gemm, the unimplemented backend="fused" of mxfp_linear_XqWq
  *   src/mase_triton/mxfp/functional/linear.py:36-64
  * (extract of x :50-52, the two composes :53-54 and the linear :61 in one prepare call and one GEMM).
@@ -323,8 +324,8 @@ int mase_hip_mxfp_gemm_scaled(const uint8_t* a_codes, const uint32_t* a_scales, 
                               const uint32_t* w_scales, const void* bias, int bias_dtype, void* y,
                               int out_dtype, int64_t M, int64_t N, int64_t K, void* stream);
 /*
- * The same with room for partial sums, as mase_hip_mxfp_gemm_ws: a product with few 256 x 256 tiles and a long K is
- * split over K into fp32 partial sums in `workspace` (mase_hip_mxfp_gemm_scaled_workspace_bytes(M, N, K) bytes, 0 when
+ * The same with room for partial sums, as mase_hip_mxfp_gemm_ws: a product with few 256 x 256 tiles and a long K, or with
+ * 17 - 64 rows of A and a K beyond 4096, is split over K into fp32 partial sums in `workspace` (mase_hip_mxfp_gemm_scaled_workspace_bytes(M, N, K) bytes, 0 when
  * the shape is not split; 16-byte aligned; NULL or too small: no split), and a second kernel adds them, the bias, and
  * rounds.  Same reference counterpart as mase_hip_mxfp_gemm_scaled.
  */

@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kGemmThreads) __attribute__((amdgpu_waves_per_eu(1,
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-#include "gemm_scaled_rows.h"   // the weight-streaming kernel for up to 32 rows of A
+#include "gemm_scaled_rows.h"   // the weight-streaming kernels for up to 64 rows of A
 
 
 // K split for few tiles and a long K (a [1024, 4096] output has 64 tiles for 256 CUs): the number of walks per tile, chosen so

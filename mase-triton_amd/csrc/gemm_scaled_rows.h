@@ -1,4 +1,4 @@
-// Block-scaled MXFP GEMM for a few rows of A (decode-sized calls: M <= 32):  y[M,N] = A[M,K] * W[N,K]^T (+ bias) as a
+// Block-scaled MXFP GEMM for a few rows of A (decode-sized calls: M <= 64):  y[M,N] = A[M,K] * W[N,K]^T (+ bias) as a
 // read of W.  Operands in the prepared form of gemm_scaled.h (FP8 bytes [rows_pad, K], scales [K/128][rows_pad] dwords).
 //
 // The product is bound by HBM: W is N * K * 33/32 bytes, read once, against 2 M N K flop.  With the block-scaled
@@ -14,7 +14,9 @@
 //     back as operand fragments: lane 16 g + r reads pieces g and g + 4 of row r of a 128-k macro step; wave w multiplies
 //     the chunk's macro steps 2 w and 2 w + 1, its scale dwords straight from global memory (16 rows = 64 contiguous bytes);
 //   * the wavefronts' partial sums meet in LDS at the end.
-// A (16 MB rows, at most a few hundred KB, shared by every workgroup) takes the same route from L2.
+// A (at most a few hundred KB, shared by every workgroup) takes the same route from L2.  Three kernels: this one streams A
+// beside W (any K, M <= 32); the second keeps A in LDS (M <= 16, K <= 4096), the third in registers (17 <= M <= 64, K in
+// slices of at most 4096).
 // (included from gemm_impl.h's namespace, after gemm_scaled.h's typedefs)
 
 // the same instruction as mfma_scaled with the accumulator in ordinary registers (a kernel that asks for accumulation
@@ -420,8 +422,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
     }
 }
 
-// the shapes these kernels take: up to 32 rows of A (two 16-row operand tiles), up to 64 when a wavefront's share of A fits
-// its registers
+// the shapes these kernels take without room for partial sums: up to 32 rows of A (two 16-row operand tiles), up to 64 when
+// a wavefront's share of A fits its registers in one piece
 inline bool scaled_rows_shape_ok(int M, int K) { return K >= 128 && (M <= 32 || (M <= 64 && K <= 4096)); }
 
 // K beyond what a wavefront's registers hold of A in one piece, 17 - 64 rows: slices of at most 32 macro steps, their sums added
