@@ -278,6 +278,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 // four at 32 rows (sixteen: the same, and the registers of four tiles no longer fit).  N x K = 14336 x 4096: 15.6 / 19.2 us at
 // 32 / 64 rows against 23.2 / 30.8 on the bf16 weight-streaming kernels and 23.8 / 26.9 on the chunked and the tile kernel; 4096 x
 // 4096: 7.6 / 10.0 against 10.7 / 16.9.  (One tile, 16 rows: 15.2 us, level with the kernel above, which keeps them.)
+// W by DMA into two LDS units, the next but one asked for before the wait for the next (one to two units in flight per CU,
+// no registers on the way), measured 15.1 / 16.4 / 19.9 us at 16 / 32 / 64 rows: no faster, so the time is not in a pipe that runs
+// dry between units.  It is in what does not scale with the bytes: 896 units are 3.5 per CU, so half the CUs work a fourth
+// round while the others idle (12 %), and launch, the first unit's latency, the prologue of A and the last reduction are
+// about 4 of the 15 us.
 constexpr int SRG_WAVES = 8;
 
 template <int DT_OUT, int MT, int WAVES>
@@ -367,7 +372,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
             const int ms = min(SPW * wave + j, nmac - 1);
             const intx4 lo = *reinterpret_cast<const intx4*>(frag_w + ms * 128), hi = *reinterpret_cast<const intx4*>(frag_w + ms * 128 + 64);
             af[t][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            a_sc[t][j] = (a_sc[t][j] >> (8 * g)) & 0xFFu;
+            a_sc[t][j] = (a_sc[t][j] >> (8 * g)) & keep[j];     // (both sides' scale bytes 0 past the end of K: the product underflows to 0)
         }
     }
     for (int u = 0; u < units; ++u) {
