@@ -81,7 +81,7 @@ def _gemm_eligible(x: Tensor, x_meta: MinifloatMeta | None, w_tensor_meta: Minif
 
 
 def _scaled_format(meta: MinifloatMeta) -> bool:
-    return meta.is_finite and meta.round_mode == "rn" and (meta.exp_bits, meta.frac_bits) in mxfp_kernels._SCALED_FORMATS
+    return meta.is_finite and meta.round_mode == "rn" and mxfp_kernels.scaled_element_format_supported(meta.exp_bits, meta.frac_bits)
 
 
 def _scaled_eligible(x: Tensor, x_meta: MinifloatMeta | None, w_tensor_meta: MinifloatTensorMeta, b: Tensor | None) -> bool:

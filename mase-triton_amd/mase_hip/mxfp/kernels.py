@@ -238,9 +238,14 @@ class ScaledOperand:
         self.codes, self.scales, self.rows, self.K = codes, scales, rows, K
 
 
+def scaled_element_format_supported(exp_bits: int, frac_bits: int) -> bool:
+    """Is (exp_bits, frac_bits), finite, an element format the block-scaled GEMM's operands hold?"""
+    return (exp_bits, frac_bits) in _SCALED_FORMATS
+
+
 def scaled_format_supported(meta: MXFPMeta) -> bool:
     return (meta.block_size == 32 and meta.element_is_finite and meta.scale_exp_bits == 8
-            and (meta.element_exp_bits, meta.element_frac_bits) in _SCALED_FORMATS)
+            and scaled_element_format_supported(meta.element_exp_bits, meta.element_frac_bits))
 
 
 def scaled_shape_supported(N: int, K: int, output_dtype: torch.dtype) -> bool:
@@ -272,7 +277,7 @@ def scaled_operand_from_dense(x: Tensor, meta: MXFPMeta) -> ScaledOperand:
 def scaled_operand_from_dense_minifloat(x: Tensor, exp_bits: int, frac_bits: int) -> ScaledOperand:
     """Round every element of the bfloat16 matrix x [rows, K] to the finite minifloat format (exp_bits, frac_bits), to
     nearest, straight into a block-scaled GEMM operand whose blocks all carry the scale 2^0."""
-    assert x.ndim == 2 and x.dtype == torch.bfloat16 and (exp_bits, frac_bits) in _SCALED_FORMATS
+    assert x.ndim == 2 and x.dtype == torch.bfloat16 and scaled_element_format_supported(exp_bits, frac_bits)
     _lib.require_gpu(x, "activations")
     x = _lib.dense(x)
     rows, K = x.shape
