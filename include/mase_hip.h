@@ -336,6 +336,23 @@ int mase_hip_mxfp_gemm_scaled_ws(const uint8_t* a_codes, const uint32_t* a_scale
                                  int64_t workspace_bytes, void* stream);
 
 /*
+ * The whole XqWq linear in one call for a caller that keeps W in the prepared form: the operand of x
+ * (mase_hip_scaled_operand_from_dense, or ..._from_dense_minifloat when x_is_minifloat != 0) built in `scratch`, then
+ * mase_hip_mxfp_gemm_scaled_ws with the rest of `scratch` as its workspace.  `scratch`: 256-byte aligned,
+ * mase_hip_mxfp_linear_scaled_scratch_bytes(M, N, K) bytes (the operand of x plus whatever the product's K split asks
+ * for; with less than the operand: -1, with the operand alone: no split).  Nothing in it has to survive the call.
+ * A decode-sized product takes less time on the GPU than two calls through a binding take on the host; this is
+ * the one call.  Shapes, formats and results as of the two calls it makes.
+ * Replaces the body of mxfp_linear_XqWq / minifloat_linear_XqWq with backend="fused"
+ *   src/mase_triton/mxfp/functional/linear.py:36-64, src/mase_triton/minifloat/functional/linear.py:33-58.
+ */
+int64_t mase_hip_mxfp_linear_scaled_scratch_bytes(int64_t M, int64_t N, int64_t K);
+int mase_hip_mxfp_linear_scaled(const void* x, int x_dtype, int x_exp_bits, int x_frac_bits, int x_is_minifloat,
+                                const uint8_t* w_codes, const uint32_t* w_scales, const void* bias,
+                                int bias_dtype, void* y, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                void* scratch, int64_t scratch_bytes, void* stream);
+
+/*
  * y[M,N] = A[M,K] * W[N,K]^T (+ bias) with a DENSE bfloat16 A (used as is, like a_dense of mase_hip_mxfp_gemm) and W in
  * the prepared form above (mase_hip_scaled_operand_from_mxfp with rows = N), on the bf16 matrix instruction: the
  * 512 x 128 tile kernel of mase_hip_mxfp_gemm composing W to bfloat16 in registers, with what the prepared form saves it

@@ -44,6 +44,8 @@ SIGNATURES = {
     "mase_hip_mxfp_gemm_scaled": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _vp]),
     "mase_hip_mxfp_gemm_scaled_ws": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _vp, _i64, _vp]),
     "mase_hip_mxfp_gemm_scaled_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "mase_hip_mxfp_linear_scaled_scratch_bytes": (_i64, [_i64, _i64, _i64]),
+    "mase_hip_mxfp_linear_scaled": (_i32, [_vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _vp, _i64, _vp]),
     "mase_hip_mxfp_gemm_prepared_w": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _vp, _i32, _i64, _i64, _i64, _vp]),
 }
 

@@ -150,9 +150,13 @@ class MinifloatLinearPTQ(nn.Module):
                 from ..mxfp import kernels
 
                 xm = self.x_minifloat_meta
-                a_op = kernels.scaled_operand_from_dense_minifloat(input.reshape(-1, self.in_features), xm.exp_bits, xm.frac_bits)
+                x2 = input.reshape(-1, self.in_features)
                 bias = None if self.layer_type.endswith("Bq") else self.bias
-                return kernels.mxfp_gemm_scaled(a_op, self._scaled_w, bias, input.dtype).view(*input.shape[:-1], self.out_features)
+                if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and (bias is None or bias.is_contiguous()):
+                    y = kernels.linear_scaled(x2, xm.exp_bits, xm.frac_bits, True, self._scaled_w, bias)
+                else:
+                    y = kernels.mxfp_gemm_scaled(kernels.scaled_operand_from_dense_minifloat(x2, xm.exp_bits, xm.frac_bits), self._scaled_w, bias, input.dtype)
+                return y.view(*input.shape[:-1], self.out_features)
         w_operand = self._weight_operand(input)
         self._fast_sig = self._call_signature(input) if w_operand is not None else None
         return MinifloatF.minifloat_linear(

@@ -361,6 +361,33 @@ def mxfp_gemm_scaled(a: ScaledOperand, w: ScaledOperand, bias: Tensor | None, ou
     return y
 
 
+_LINEAR_SCRATCH_BYTES: dict[tuple, int] = {}
+
+
+def linear_scaled(x: Tensor, exp_bits: int, frac_bits: int, minifloat: bool, w: ScaledOperand, bias: Tensor | None) -> Tensor:
+    """x [M, K] (bfloat16, contiguous, 16-byte aligned) quantised to MXFP elements (exp_bits, frac_bits) with block scales,
+    or rounded element by element to that minifloat format, times W^T (+ bias) on the block-scaled matrix instruction:
+    ``mxfp_gemm_scaled(scaled_operand_from_dense*(x), w, bias, x.dtype)`` through ONE call into the library (a decode-sized
+    product is bound by the host otherwise).  The caller has checked formats and shape."""
+    M, K = x.shape
+    N = w.rows
+    dev = x.device
+    lib = _lib.load()
+    key = (dev.index, M, N, K)
+    nbytes = _LINEAR_SCRATCH_BYTES.get(key)
+    if nbytes is None:
+        with _lib.on_device(dev):
+            nbytes = _LINEAR_SCRATCH_BYTES[key] = lib.mase_hip_mxfp_linear_scaled_scratch_bytes(M, N, K)
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    y = torch.empty((M, N), dtype=x.dtype, device=dev)
+    b_ptr, b_dt = (None, 0) if bias is None else (bias.data_ptr(), _lib.dtype_code(bias.dtype))
+    with _lib.on_device(dev):
+        _lib.check(lib.mase_hip_mxfp_linear_scaled(
+            x.data_ptr(), _lib.dtype_code(x.dtype), exp_bits, frac_bits, int(minifloat), w.codes.data_ptr(), w.scales.data_ptr(), b_ptr, b_dt,
+            y.data_ptr(), _lib.dtype_code(x.dtype), M, N, K, scratch.data_ptr(), nbytes, _lib.stream_ptr(dev)))
+    return y
+
+
 def prepared_w_shape_supported(M: int, N: int, K: int) -> bool:
     return M >= 512 and N % 128 == 0 and K % 128 == 0 and K <= (1 << 23)
 

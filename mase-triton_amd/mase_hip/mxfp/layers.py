@@ -162,9 +162,14 @@ class MXFPLinearPTQ(nn.Module):
             if self._scaled_w_key == (w_elements.data_ptr(), w_elements._version, w_scales.data_ptr(), w_scales._version):
                 from . import kernels
 
-                a_op = kernels.scaled_operand_from_dense(input.reshape(-1, self.in_features), self.x_mxfp_meta)
+                x2 = input.reshape(-1, self.in_features)
                 bias = None if self.layer_type.endswith("Bq") else self.bias
-                return kernels.mxfp_gemm_scaled(a_op, self._scaled_w, bias, input.dtype).view(*input.shape[:-1], self.out_features)
+                meta = self.x_mxfp_meta
+                if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and (bias is None or bias.is_contiguous()):
+                    y = kernels.linear_scaled(x2, meta.element_exp_bits, meta.element_frac_bits, False, self._scaled_w, bias)
+                else:
+                    y = kernels.mxfp_gemm_scaled(kernels.scaled_operand_from_dense(x2, meta), self._scaled_w, bias, input.dtype)
+                return y.view(*input.shape[:-1], self.out_features)
         w_operand = self._weight_operand(input)
         self._fast_sig = self._call_signature(input) if w_operand is not None and self._takes_scaled_route(input) else None
         return MXFP_F.mxfp_linear(

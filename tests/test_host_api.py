@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol(lib):
     from mase_hip import _lib
 
     names = declared_symbols()
-    assert len(names) == 26
+    assert len(names) == 28
     for n in names:
         assert hasattr(lib, n), f"{n} declared in include/mase_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of step with the header"
@@ -66,6 +66,13 @@ def test_argument_errors_without_a_gpu(lib):
     assert lib.mase_hip_scaled_operand_from_dense_minifloat(p, 2, 5, 2, 8, 128, p, p, None) == -2    # E5M2
     assert lib.mase_hip_scaled_operand_from_dense_minifloat(p, 1, 4, 3, 8, 128, p, p, None) == -2    # fp16 input
     assert lib.mase_hip_scaled_operand_from_dense_minifloat(None, 2, 4, 3, 8, 128, p, p, None) == -1
+    assert lib.mase_hip_mxfp_linear_scaled_scratch_bytes(16, 4096, 4096) == 256 * 4096 + 32 * 256 * 4      # the operand of x alone
+    assert lib.mase_hip_mxfp_linear_scaled_scratch_bytes(40, 4096, 14336) == 256 * 14336 + 112 * 256 * 4 + 4 * 40 * 4096 * 4
+    assert lib.mase_hip_mxfp_linear_scaled_scratch_bytes(16, 4096, 384) == 0
+    assert lib.mase_hip_mxfp_linear_scaled(p, 2, 4, 3, 0, p, p, None, 0, p, 2, 8, 8, 512, None, 0, None) == -1          # no scratch
+    assert lib.mase_hip_mxfp_linear_scaled(p, 2, 4, 3, 0, p, p, None, 0, p, 2, 8, 8, 512, p, 1024, None) == -1         # scratch too small
+    assert lib.mase_hip_mxfp_linear_scaled(p, 2, 4, 3, 0, p, p, None, 0, p, 2, 8, 8, 384, p, 1 << 20, None) == -2      # K % 256
+    assert lib.mase_hip_mxfp_linear_scaled(None, 2, 4, 3, 0, None, None, None, 0, None, 2, 0, 8, 512, None, 0, None) == 0  # no rows
     assert lib.mase_hip_scaled_operand_from_swiglu(p, None, 2, 128, 4, 3, 8, 128, p, p, None) == -1   # no up
     assert lib.mase_hip_scaled_operand_from_swiglu(p, p, 2, 64, 4, 3, 8, 128, p, p, None) == -1     # row stride below K
     assert lib.mase_hip_scaled_operand_from_swiglu(p, p, 2, 132, 4, 3, 8, 128, p, p, None) == -1    # row stride not a multiple of 8
