@@ -458,7 +458,7 @@ def bench_hbm(torch, with_cpu):
     comps = [(w_sc, w_el)] + [(w_sc.clone(), w_el.clone()) for _ in range(6)]
     wops = [kernels.scaled_operand_from_mxfp(sc, el, MXFP8_E4M3_fn, N, K) for sc, el in comps]
     w_bytes = N * K * (1 + 1 / 32)
-    for rows in (16, 64):      # x in LDS up to 16 rows, in registers from 17 to 64
+    for rows in (16, 64):      # one and four operand tiles of x in the wavefronts' registers
         xr = x64[:rows].contiguous()
         a_op = kernels.scaled_operand_from_dense(xr, MXFP8_E4M3_fn)
         a_dq = kernels.quantize_dequantize(xr.view(-1), MXFP8_E4M3_fn, torch.bfloat16).view(rows, K)
@@ -700,11 +700,11 @@ _M5, _H5, _I5 = 8192, 4096, 14336
 COUNTER_ROWS = (
     ("stream_copy_kernel", "calibration copy (256 MiB read, 256 MiB written)", 256 << 20, 256 << 20, None),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C4", (_M4 + _N4) * _K4 * 33 // 32, _M4 * _N4 * 2, SCALED_SOURCES),
-    ("mxfp_gemm_scaled_rows_resident_kernel", "mxfp_gemm_scaled_rows C4 W x 16 rows", _N4 * _K4 * 33 // 32 + 16 * _K4 * 33 // 32, 16 * _N4 * 2, ROWS_SOURCES),
+    ("mxfp_gemm_scaled_rows_regs_kernel<2, 1, 8>", "mxfp_gemm_scaled_rows C4 W x 16 rows", _N4 * _K4 * 33 // 32 + 16 * _K4 * 33 // 32, 16 * _N4 * 2, ROWS_SOURCES),
     ("mxfp_gemm_tall_kernel", "mxfp_gemm_tall_kernel C4", _M4 * _K4 * 2 + _N4 * _K4 * 33 // 32, _M4 * _N4 * 2, GEMM_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 gate+up", (_M5 + 2 * _I5) * _H5 * 33 // 32, _M5 * 2 * _I5 * 2, SCALED_SOURCES),
     ("mxfp_gemm_scaled_kernel", "mxfp_gemm_scaled_kernel C5 down", (_M5 + _H5) * _I5 * 33 // 32, _M5 * _H5 * 2, SCALED_SOURCES),
-    ("mxfp_gemm_scaled_rows_regs_kernel", "mxfp_gemm_scaled_rows C4 W x 64 rows", _N4 * _K4 * 33 // 32 + 64 * _K4 * 33 // 32, 64 * _N4 * 2, ROWS_SOURCES),
+    ("mxfp_gemm_scaled_rows_regs_kernel<2, 4, 8>", "mxfp_gemm_scaled_rows C4 W x 64 rows", _N4 * _K4 * 33 // 32 + 64 * _K4 * 33 // 32, 64 * _N4 * 2, ROWS_SOURCES),
     ("scaled_from_dense_kernel|0>, 1>(", "scaled_operand_from_swiglu C5", _M5 * _I5 * 4, _M5 * _I5 * 33 // 32, CAST_SOURCES),
     ("scaled_from_dense_kernel|0>, 0>(", "scaled_operand_from_dense C4 x", _M4 * _K4 * 2, _M4 * _K4 * 33 // 32, CAST_SOURCES),
     ("scaled_operand_kernel<mase::SFmt<4, 3", "scaled_operand_from_mxfp C4 W", _N4 * _K4 * 33 // 32, _N4 * _K4 * 33 // 32, CAST_SOURCES),

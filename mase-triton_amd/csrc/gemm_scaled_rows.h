@@ -14,9 +14,8 @@
 //     back as operand fragments: lane 16 g + r reads pieces g and g + 4 of row r of a 128-k macro step; wave w multiplies
 //     the chunk's macro steps 2 w and 2 w + 1, its scale dwords straight from global memory (16 rows = 64 contiguous bytes);
 //   * the wavefronts' partial sums meet in LDS at the end.
-// A (at most a few hundred KB, shared by every workgroup) takes the same route from L2.  Three kernels: this one streams A
-// beside W (any K, M <= 32); the second keeps A in LDS (M <= 16, K <= 4096), the third in registers (17 <= M <= 64, K in
-// slices of at most 4096).
+// A (at most a few hundred KB, shared by every workgroup) takes the same route from L2.  Two kernels: this one streams A
+// beside W (any K, M <= 32); the other keeps A in registers (M <= 64, K <= 4096, or from 17 rows a longer K in slices).
 // (included from gemm_impl.h's namespace, after gemm_scaled.h's typedefs)
 
 // the same instruction as mfma_scaled with the accumulator in ordinary registers (a kernel that asks for accumulation
@@ -160,136 +159,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     }
 }
 
-// ---- The same product when all of A fits LDS beside 16 whole rows of W (K <= 4096, M <= 16).  A is loaded once per
-// workgroup and stays; workgroups are persistent (one per CU) and take 16 rows of W x all of K per unit, as whole rows
-// (the shape that reads fastest), one unit ahead in registers.  The L1 then fills W alone: 15.2 us against 17.4 us for the
-// chunked kernel above at N x K = 14336 x 4096, 16 rows.  (Two units ahead measured slower, 16.8 us.)
+// ---- The persistent kernels: K <= 4096 (or a slice of K that long), workgroups that stay (one per CU) and take 16 whole
+// rows of W x all of K per unit, as whole rows (the shape that reads fastest), one unit ahead in registers.
 constexpr int SRR_ROW = 4096 + 16;        // LDS row pitch: K <= 4096 bytes and 16 of padding (conflict-free 128-bit accesses)
 
-template <int DT_OUT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mxfp_gemm_scaled_rows_resident_kernel(
-    const uint8_t* __restrict__ a_codes, const uint32_t* __restrict__ a_scales, const uint8_t* __restrict__ w_codes,
-    const uint32_t* __restrict__ w_scales, const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int rows_a,
-    int rows_w) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];            // A [16][SRR_ROW], W [16][SRR_ROW], partial sums [3][256]
-    uint8_t* const tile_a = lds;
-    uint8_t* const tile_w = lds + 16 * SRR_ROW;
-    float (*const red)[256] = reinterpret_cast<float (*)[256]>(lds + 32 * SRR_ROW);
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int g = lane >> 4, r = lane & 15;
-    const int nmac = K / 128;
-    const int groups = (N + 15) / 16;
-    const int units = ((int)blockIdx.x < groups) ? (groups - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
-    // lane l reads bytes 1024 q + 16 l of a row, q = 0..3, clamped to the row's last 16 bytes (K < 4096)
-    uint32_t off[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) off[q] = min(1024u * q + 16u * lane, (uint32_t)K - 16u);
-
-    // ---- A and its scales, once
-    {
-        intx4 areg[4][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) areg[i][q] = *reinterpret_cast<const intx4*>(a_codes + (size_t)(4 * wave + i) * K + off[q]);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) *reinterpret_cast<intx4*>(tile_a + (4 * wave + i) * SRR_ROW + 1024 * q + 16 * lane) = areg[i][q];
-    }
-    uint32_t a_sc[8], keep[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int ms = 8 * wave + j;
-        keep[j] = ms < nmac ? 0xFFu : 0u;                        // a macro step past the end of K is multiplied with scale bytes 0
-        a_sc[j] = (a_scales[(size_t)min(ms, nmac - 1) * rows_a + r] >> (8 * g)) & keep[j];
-    }
-
-    intx4 wreg[4][4];
-    uint32_t w_sc_next[8];
-    auto issue = [&](int u) __attribute__((always_inline)) {
-        // (plain arithmetic: a unit past the end has pitch 0 and offset 0, every lane of a wavefront reads the same line)
-        const uint32_t live = u < units ? 1u : 0u;
-        const int group = (int)blockIdx.x + u * (int)gridDim.x;
-        const uint8_t* row0 = w_codes + (size_t)live * (size_t)(group * 16 + 4 * wave) * K;
-        const size_t pitch = (size_t)live * (size_t)K;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) wreg[i][q] = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(row0 + i * pitch + live * off[q]));
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            w_sc_next[j] = __builtin_nontemporal_load(w_scales + (size_t)live * ((size_t)min(8 * wave + j, nmac - 1) * rows_w + group * 16 + r));
-    };
-    issue(0);
-    const uint8_t* const frag_a = tile_a + r * SRR_ROW + 16 * g;
-    const uint8_t* const frag_w = tile_w + r * SRR_ROW + 16 * g;
-    for (int u = 0; u < units; ++u) {
-        const int group = (int)blockIdx.x + u * (int)gridDim.x;
-        __syncthreads();                                         // the reads of the unit before (fragments, partial sums) are done
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) *reinterpret_cast<intx4*>(tile_w + (4 * wave + i) * SRR_ROW + 1024 * q + 16 * lane) = wreg[i][q];
-        uint32_t w_sc[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) w_sc[j] = (w_sc_next[j] >> (8 * g)) & keep[j];
-        __builtin_amdgcn_sched_barrier(0);
-        issue(u + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-        floatx4 acc = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int ms = 8 * wave + j;
-            const intx4 w_lo = *reinterpret_cast<const intx4*>(frag_w + ms * 128), w_hi = *reinterpret_cast<const intx4*>(frag_w + ms * 128 + 64);
-            const intx4 a_lo = *reinterpret_cast<const intx4*>(frag_a + ms * 128), a_hi = *reinterpret_cast<const intx4*>(frag_a + ms * 128 + 64);
-            mfma_scaled_after_valu(acc, __builtin_shufflevector(w_lo, w_hi, 0, 1, 2, 3, 4, 5, 6, 7), __builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7),
-                                   w_sc[j], a_sc[j]);
-        }
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");     // the matrix unit's last results have left its pipeline
-        if (wave > 0) *reinterpret_cast<floatx4*>(&red[wave - 1][lane * 4]) = acc;
-        __syncthreads();
-        if (wave == 0) {
-            floatx4 s = acc;
-#pragma unroll
-            for (int w = 0; w < 3; ++w) s += *reinterpret_cast<const floatx4*>(&red[w][lane * 4]);
-            const int n = group * 16 + 4 * g, m = r;
-            if (m < M && n < N) {
-                float out[4] = {s[0], s[1], s[2], s[3]};
-                const int valid = min(4, N - n);
-                if (bias)
-                    for (int t = 0; t < valid; ++t) out[t] += load_bias(bias, bias_dtype, n + t);
-                store_out4<DT_OUT>(y, (int64_t)m * N + n, out, true, valid);
-            }
-        }
-    }
+// How the persistent kernels below deal the row groups of W (16 rows each) to their workgroups.  Whole rounds first: group
+// b + u * grid is unit u of workgroup b.  What is left after the whole rounds, when it is at most half a round, is dealt in
+// HALF units: eight rows of a group each (the matrix instruction still multiplies sixteen; the other eight are whatever
+// the buffer holds and their results are not stored), two workgroups to a group, so that a tail of L groups keeps 2 L CUs
+// busy for half a unit's time instead of L CUs for a whole one (N = 14336 on 256 CUs: 3.5 rounds instead of 4).
+struct RowsDeal {
+    int grid, full_rounds, tail_halves;   // workgroups; units every workgroup takes; workgroups that take a half unit after them
+};
+inline RowsDeal deal_row_groups(int groups, int cus) {
+    const int full = groups / cus, left = groups - full * cus;
+    if (left > 0 && 2 * left <= cus) return RowsDeal{full > 0 ? cus : 2 * left, full, 2 * left};
+    return RowsDeal{min(groups, cus), 0, 0};      // whole units only: unit u of workgroup b is group b + u * grid while there are groups
+}
+// unit u of workgroup b: its group, and which half of it (-1: all sixteen rows)
+struct RowsUnit { int group, half; };
+__device__ inline int rows_unit_count(int b, int grid, int groups, int full_rounds, int tail_halves) {
+    if (tail_halves > 0) return full_rounds + (b < tail_halves ? 1 : 0);
+    return b < groups ? (groups - b + grid - 1) / grid : 0;
+}
+__device__ inline RowsUnit rows_unit(int b, int u, int grid, int full_rounds, int tail_halves) {
+    if (tail_halves > 0 && u >= full_rounds) return RowsUnit{full_rounds * grid + (b >> 1), b & 1};
+    return RowsUnit{b + u * grid, -1};
 }
 
-// ---- The same with A in registers (K <= 4096, M <= 16 MT, MT = 2 or 4 operand tiles of 16 rows: 17 - 64 rows of A).  A
-// wavefront multiplies the same macro steps of every unit (wave w: SPW w .. SPW w + SPW - 1, SPW = 32 / WAVES), so the
-// fragments of A it needs are the same for the whole launch: MT x SPW x 8 registers (128 for four tiles on eight
-// wavefronts), filled once.  LDS then holds W alone and no byte of A is read a second time.  W takes the route of the
-// kernel above: 1 KB of one row per load instruction, one unit ahead in registers, through LDS; so does A on its way to
-// the registers, tile by tile through W's place in LDS (read straight from global memory in the operand layout, 64 bytes
-// of a row at a time, every cache line is fetched twice, and with every CU of an XCD asking its L2 for the same A that is
-// what the prologue costs: 22 against 19 us at 64 rows, N x K = 14336 x 4096).  Eight wavefronts: 15.6 against 18.4 us with
-// four at 32 rows (sixteen: the same, and the registers of four tiles no longer fit).  N x K = 14336 x 4096: 15.6 / 19.2 us at
-// 32 / 64 rows against 23.2 / 30.8 on the bf16 weight-streaming kernels and 23.8 / 26.9 on the chunked and the tile kernel; 4096 x
-// 4096: 7.6 / 10.0 against 10.7 / 16.9.  (One tile, 16 rows: 15.2 us, level with the kernel above, which keeps them.)
+// ---- A in registers (K <= 4096, M <= 16 MT, MT = 1, 2 or 4 operand tiles of 16 rows: up to 64 rows of A).  A wavefront
+// multiplies the same macro steps of every unit (wave w: SPW w .. SPW w + SPW - 1, SPW = 32 / WAVES), so the fragments of
+// A it needs are the same for the whole launch: MT x SPW x 8 registers (128 for four tiles on eight wavefronts), filled
+// once.  LDS holds W alone (rows 4112 bytes apart: conflict-free 128-bit writes and fragment reads) and no byte of A is
+// read a second time.  W: 1 KB of one row per load instruction, one unit ahead in registers, through LDS; so does A on its
+// way to the registers, tile by tile through W's place in LDS (read straight from global memory in the operand layout, 64
+// bytes of a row at a time, every cache line is fetched twice, and with every CU of an XCD asking its L2 for the same A
+// that is what the prologue costs: 22 against 19 us at 64 rows, N x K = 14336 x 4096).  The wavefronts' partial sums meet
+// in LDS; wavefront t adds and stores tile t.  Eight wavefronts: 15.6 against 18.4 us with four at 32 rows (sixteen: the
+// same, and the registers of four tiles no longer fit).  N x K = 14336 x 4096: 14.0 / 15.6 / 19.2 us at 16 / 32 / 64 rows against
+// 20.9 / 23.2 / 30.8 on the bf16 weight-streaming kernels (23.8 / 26.9 at 32 / 64 rows on the chunked and the tile kernel); 4096 x
+// 4096: 6.8 / 7.6 / 10.0 against 9.7 / 10.7 / 16.9.  (A build that kept 16 rows of A in LDS instead, four wavefronts: 14.8 us at
+// 16 rows where this one takes 14.0, same box.)
 // W by DMA into two LDS units, the next but one asked for before the wait for the next (one to two units in flight per CU,
 // no registers on the way), measured 15.1 / 16.4 / 19.9 us at 16 / 32 / 64 rows: no faster, so the time is not in a pipe that runs
-// dry between units.  It is in what does not scale with the bytes: 896 units are 3.5 per CU, so half the CUs work a fourth
-// round while the others idle (12 %), and launch, the first unit's latency, the prologue of A and the last reduction are
-// about 4 of the 15 us.
+// dry between units; nor is it in the last round (half units, above: 0.1 - 0.4 us).  Launch, the first unit's latency,
+// the prologue of A and the last reduction are about 4 of the 14 us.
 constexpr int SRG_WAVES = 8;
 
 template <int DT_OUT, int MT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4))) void mxfp_gemm_scaled_rows_regs_kernel(
     const uint8_t* __restrict__ a_codes, const uint32_t* __restrict__ a_scales, const uint8_t* __restrict__ w_codes,
     const uint32_t* __restrict__ w_scales, const void* __restrict__ bias, int bias_dtype, void* __restrict__ y, int M, int N, int K, int rows_a,
-    int rows_w, int slices, int slice_macs, float* __restrict__ partial) {
+    int rows_w, int slices, int slice_macs, float* __restrict__ partial, int full_rounds, int tail_halves) {
     constexpr int SPW = 32 / WAVES;          // macro steps of a unit per wavefront
     constexpr int RPW = 16 / WAVES;          // rows of W a wavefront carries from global memory to LDS
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];            // W [16][SRR_ROW], partial sums [WAVES][MT][256]
@@ -307,7 +228,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
     const int nmac = min(slice_macs, K / 128 - mac0);            // this slice's macro steps: at most 32
     const size_t k0 = (size_t)mac0 * 128;
     const int groups = (N + 15) / 16;
-    const int units = first_group < groups ? (groups - first_group + group_step - 1) / group_step : 0;
+    const int units = rows_unit_count(first_group, group_step, groups, full_rounds, tail_halves);      // (half units: one slice only)
     uint32_t off[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) off[q] = min(1024u * q + 16u * lane, (uint32_t)nmac * 128u - 16u);
@@ -319,9 +240,11 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
     intx4 wreg[RPW][4];
     uint32_t w_sc_next[SPW];
     auto issue = [&](int u) __attribute__((always_inline)) {
-        // (plain arithmetic: a unit past the end has pitch 0 and offset 0, every lane of a wavefront reads the same line)
-        const uint32_t live = u < units ? 1u : 0u;
-        const int group = first_group + u * group_step;
+        // (plain arithmetic: a unit past the end, or the rows of the half that a half unit leaves out, have pitch 0 and
+        // offset 0: every lane of a wavefront reads the same line)
+        const RowsUnit ru = rows_unit(first_group, u, group_step, full_rounds, tail_halves);
+        const uint32_t live = u < units && (ru.half < 0 || (RPW * wave >> 3) == ru.half) ? 1u : 0u;      // this wavefront's rows: RPW wave .. + RPW - 1
+        const int group = u < units ? ru.group : 0;
         const uint8_t* row0 = w_codes + (size_t)live * (size_t)(group * 16 + RPW * wave) * K;
         const size_t pitch = (size_t)live * (size_t)K;
 #pragma unroll
@@ -330,7 +253,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
             for (int q = 0; q < 4; ++q) wreg[i][q] = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(row0 + i * pitch + live * off[q]));
 #pragma unroll
         for (int j = 0; j < SPW; ++j)
-            w_sc_next[j] = __builtin_nontemporal_load(w_scales + (size_t)live * ((size_t)min(SPW * wave + j, nmac - 1) * rows_w + group * 16 + r));
+            w_sc_next[j] = __builtin_nontemporal_load(w_scales + (size_t)min(SPW * wave + j, nmac - 1) * rows_w + group * 16 + r);
     };
     // ---- this wavefront's fragments of A and their scale bytes, once.  A tile takes W's route (whole 1 KB pieces of a row per
     // load instruction, through LDS): read in the operand layout straight from global memory, 64 bytes of a row at a time,
@@ -376,7 +299,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
         }
     }
     for (int u = 0; u < units; ++u) {
-        const int group = first_group + u * group_step;
+        const RowsUnit ru = rows_unit(first_group, u, group_step, full_rounds, tail_halves);
+        const int group = ru.group;
         __syncthreads();                                         // the reads of the unit before (fragments, partial sums) are done
 #pragma unroll
         for (int i = 0; i < RPW; ++i)
@@ -411,7 +335,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(WAVE
 #pragma unroll
             for (int w = 1; w < WAVES; ++w) s += *reinterpret_cast<const floatx4*>(&red[w][t][lane * 4]);
             const int n = group * 16 + 4 * g, m = 16 * t + r;
-            if (m < M && n < N) {
+            if (m < M && n < N && (ru.half < 0 || (g >> 1) == ru.half)) {
                 float out[4] = {s[0], s[1], s[2], s[3]};
                 const int valid = min(4, N - n);
                 if (partial) {
@@ -453,7 +377,7 @@ int launch_gemm_scaled_rows_sliced(const uint8_t* a_codes, const uint32_t* a_sca
         // as many workgroups per slice as fill the CUs between them (every slice the same count)
         const int per_slice = max(1, min(groups, cus / slices));
         hipLaunchKernelGGL(kern, dim3((unsigned)(per_slice * slices)), dim3(SRG_WAVES * 64), lds_bytes, s, a_codes, a_scales, w_codes, w_scales,
-                           static_cast<const void*>(nullptr), 0, static_cast<void*>(nullptr), M, N, K, rows_a, rows_w, slices, slice_macs, partial);
+                           static_cast<const void*>(nullptr), 0, static_cast<void*>(nullptr), M, N, K, rows_a, rows_w, slices, slice_macs, partial, 0, 0);
         return check_launch("mxfp_gemm_scaled");
     };
     static std::atomic<uint64_t> allowed2{0}, allowed4{0};
@@ -470,19 +394,7 @@ int launch_gemm_scaled_rows(const uint8_t* a_codes, const uint32_t* a_scales, co
                             int bias_dtype, void* y, int M, int N, int K, hipStream_t s) {
     const int rows_a = (M + 255) / 256 * 256, rows_w = (N + 255) / 256 * 256;
     const unsigned groups = (unsigned)((N + 15) / 16);
-    if (M <= 16 && K <= 4096) {
-        // all of A stays in LDS: persistent workgroups, one per CU
-        const int cus = device_cu_count();
-        if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
-        auto kern = mxfp_gemm_scaled_rows_resident_kernel<DT_OUT>;
-        const int lds_bytes = 32 * SRR_ROW + 3 * 256 * (int)sizeof(float);
-        static std::atomic<uint64_t> lds_allowed{0};
-        if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_allowed)) return rc;
-        hipLaunchKernelGGL(kern, dim3((unsigned)min((int)groups, cus)), dim3(256), lds_bytes, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N, K,
-                           rows_a, rows_w);
-        return check_launch("mxfp_gemm_scaled");
-    }
-    if (K <= 4096 && M > 16) {
+    if (K <= 4096) {
         // a wavefront's share of A stays in its registers: persistent workgroups of eight wavefronts, one per CU
         const int cus = device_cu_count();
         if (cus <= 0) return fail(ERR_RUNTIME, "cannot read the compute-unit count of the current device");
@@ -490,11 +402,13 @@ int launch_gemm_scaled_rows(const uint8_t* a_codes, const uint32_t* a_scales, co
             // (more than half a CU's LDS, so that no CU is given two of these workgroups while another has none)
             const int lds_bytes = max(16 * SRR_ROW + SRG_WAVES * mt * 256 * (int)sizeof(float), 84 * 1024);
             if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, allowed)) return rc;
-            hipLaunchKernelGGL(kern, dim3((unsigned)min((int)groups, cus)), dim3(SRG_WAVES * 64), lds_bytes, s, a_codes, a_scales, w_codes, w_scales, bias,
-                               bias_dtype, y, M, N, K, rows_a, rows_w, 1, K / 128, static_cast<float*>(nullptr));
+            const RowsDeal d = deal_row_groups((int)groups, cus);
+            hipLaunchKernelGGL(kern, dim3((unsigned)d.grid), dim3(SRG_WAVES * 64), lds_bytes, s, a_codes, a_scales, w_codes, w_scales, bias, bias_dtype, y, M, N,
+                               K, rows_a, rows_w, 1, K / 128, static_cast<float*>(nullptr), d.full_rounds, d.tail_halves);
             return check_launch("mxfp_gemm_scaled");
         };
-        static std::atomic<uint64_t> allowed2{0}, allowed4{0};
+        static std::atomic<uint64_t> allowed1{0}, allowed2{0}, allowed4{0};
+        if (M <= 16) return go(mxfp_gemm_scaled_rows_regs_kernel<DT_OUT, 1, SRG_WAVES>, 1, allowed1);
         if (M <= 32) return go(mxfp_gemm_scaled_rows_regs_kernel<DT_OUT, 2, SRG_WAVES>, 2, allowed2);
         return go(mxfp_gemm_scaled_rows_regs_kernel<DT_OUT, 4, SRG_WAVES>, 4, allowed4);
     }

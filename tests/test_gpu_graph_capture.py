@@ -11,7 +11,7 @@ DEV = "cuda:0"
 
 @pytest.mark.parametrize("M,K,N", [(8, 512, 12288), (200, 512, 12288), (1024, 512, 12288),
                                    (200, 4096, 512),    # K split over workgroups, workspace from torch's allocator
-                                   (16, 4096, 1024), (40, 4096, 1024),   # the weight-streaming kernels: x in LDS, x in registers
+                                   (16, 4096, 1024), (40, 4096, 1024),   # the weight-streaming kernel: one and three operand tiles of x
                                    (48, 8192, 520)])    # ... on K slices: workspace and the reduce kernel inside the capture
 def test_fused_layer_replays_from_a_graph(M, K, N):
     from mase_hip import _lib

@@ -279,9 +279,9 @@ def test_scaled_gemm_many_tiles(mh, MNK):
 @pytest.mark.parametrize("x_tag,w_tag", [("MXFP8_E4M3_fn", "MXFP8_E4M3_fn"), ("MXFP8_E4M3_fn", "OCP_MXFP4_E2M1")])
 def test_scaled_gemm_few_rows(mh, MNK, x_tag, w_tag):
     """Up to 64 rows of x: the weight-streaming kernels (a workgroup per 16 rows of W, its wavefronts taking the macro steps
-    of K in turn and adding their partial sums through LDS; x in LDS up to 16 rows, in registers from 17 to 64, a K beyond
-    4096 cut into slices whose sums a second kernel adds (the Python wrapper brings the room for them), streamed beside W
-    up to 16 rows).  Row counts on both sides of the 16-row operand tiles, N that is not a
+    of K in turn and adding their partial sums through LDS; x in the wavefronts' registers, a K beyond 4096 cut into slices
+    whose sums a second kernel adds (from 17 rows; the Python wrapper brings the room for them) or x streamed beside W (up to 16
+    rows, and whenever there is no such room); the last row groups dealt in halves.  Row counts on both sides of the 16-row operand tiles, N that is not a
     multiple of 16, more and fewer row groups of W than the chip has CUs, K with fewer macro steps than a workgroup has
     wavefronts and with a count they do not divide; bias and every output type."""
     M, N, K = MNK
