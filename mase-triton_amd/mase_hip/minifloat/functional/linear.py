@@ -152,8 +152,12 @@ def minifloat_linear(
         if ok and (backend == "fused_scaled" or takes_scaled_route(rows, _w_operand is not None)):
             if _w_operand is None:
                 _w_operand = scaled_weight_operand(w_element, w_tensor_meta, _narrowed)
-            a_op = mxfp_kernels.scaled_operand_from_dense_minifloat(x.reshape(-1, x.shape[-1]), x_meta.exp_bits, x_meta.frac_bits)
-            y = mxfp_kernels.mxfp_gemm_scaled(a_op, _w_operand, b, x.dtype)
+            x2 = x.reshape(-1, x.shape[-1])
+            if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and x2.shape[0] > 0 and (b is None or b.is_contiguous()):
+                y = mxfp_kernels.linear_scaled(x2, x_meta.exp_bits, x_meta.frac_bits, True, _w_operand, b)
+            else:
+                a_op = mxfp_kernels.scaled_operand_from_dense_minifloat(x2, x_meta.exp_bits, x_meta.frac_bits)
+                y = mxfp_kernels.mxfp_gemm_scaled(a_op, _w_operand, b, x.dtype)
             return y.view(*x.shape[:-1], w_tensor_meta.shape[0])
     elif backend == "fused_scaled":
         raise NotImplementedError("fused_scaled needs quantised activations and weights (XqWq layer types)")

@@ -152,7 +152,7 @@ class MinifloatLinearPTQ(nn.Module):
                 xm = self.x_minifloat_meta
                 x2 = input.reshape(-1, self.in_features)
                 bias = None if self.layer_type.endswith("Bq") else self.bias
-                if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and (bias is None or bias.is_contiguous()):
+                if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and x2.shape[0] > 0 and (bias is None or bias.is_contiguous()):
                     y = kernels.linear_scaled(x2, xm.exp_bits, xm.frac_bits, True, self._scaled_w, bias)
                 else:
                     y = kernels.mxfp_gemm_scaled(kernels.scaled_operand_from_dense_minifloat(x2, xm.exp_bits, xm.frac_bits), self._scaled_w, bias, input.dtype)

@@ -143,11 +143,15 @@ def mxfp_linear(
         if backend == "fused_scaled" or takes_scaled_route(rows, w_operand is not None):
             out_features, in_features = w_tensor_meta.shape
             assert x.shape[-1] == in_features
-            a_op = kernels.scaled_operand_from_dense(x.reshape(-1, in_features), x_meta)
             if w_operand is None:
                 w_operand = scaled_weight_operand(w_scales, w_elements, w_tensor_meta)
             assert w_operand.rows == out_features and w_operand.K == in_features
-            y = kernels.mxfp_gemm_scaled(a_op, w_operand, bias, x.dtype)
+            x2 = x.reshape(-1, in_features)
+            if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and x2.shape[0] > 0 and (bias is None or bias.is_contiguous()):
+                # operand of x and product behind one call into the library (a decode-sized product is bound by the host)
+                y = kernels.linear_scaled(x2, x_meta.element_exp_bits, x_meta.element_frac_bits, False, w_operand, bias)
+            else:
+                y = kernels.mxfp_gemm_scaled(kernels.scaled_operand_from_dense(x2, x_meta), w_operand, bias, x.dtype)
             return y.view(*x.shape[:-1], out_features)
     elif backend == "fused_scaled":
         raise NotImplementedError("backend 'fused_scaled' needs quantised bfloat16 x and W in E4M3 / E3M2 / E2M3 / E2M1 with in_features a "

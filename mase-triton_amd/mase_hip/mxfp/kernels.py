@@ -380,6 +380,7 @@ def linear_scaled(x: Tensor, exp_bits: int, frac_bits: int, minifloat: bool, w: 
             nbytes = _LINEAR_SCRATCH_BYTES[key] = lib.mase_hip_mxfp_linear_scaled_scratch_bytes(M, N, K)
     scratch = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     y = torch.empty((M, N), dtype=x.dtype, device=dev)
+    assert w.K == K and (bias is None or (bias.numel() == N and bias.device == dev))
     b_ptr, b_dt = (None, 0) if bias is None else (bias.data_ptr(), _lib.dtype_code(bias.dtype))
     with _lib.on_device(dev):
         _lib.check(lib.mase_hip_mxfp_linear_scaled(

@@ -165,7 +165,7 @@ class MXFPLinearPTQ(nn.Module):
                 x2 = input.reshape(-1, self.in_features)
                 bias = None if self.layer_type.endswith("Bq") else self.bias
                 meta = self.x_mxfp_meta
-                if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and (bias is None or bias.is_contiguous()):
+                if x2.is_contiguous() and x2.data_ptr() % 16 == 0 and x2.shape[0] > 0 and (bias is None or bias.is_contiguous()):
                     y = kernels.linear_scaled(x2, meta.element_exp_bits, meta.element_frac_bits, False, self._scaled_w, bias)
                 else:
                     y = kernels.mxfp_gemm_scaled(kernels.scaled_operand_from_dense(x2, meta), self._scaled_w, bias, input.dtype)

@@ -313,6 +313,7 @@ def test_minifloat_layer_routes(mf, monkeypatch):
         return wrapped
 
     monkeypatch.setattr(K_, "mxfp_gemm_scaled", count("scaled", real_scaled))
+    monkeypatch.setattr(K_, "linear_scaled", count("scaled", K_.linear_scaled))     # (operand of x and the same GEMM behind one call)
     monkeypatch.setattr(K_, "mxfp_gemm", count("bf16", real_bf16))
     monkeypatch.setattr(K_, "scaled_operand_from_mxfp", count("prepare", real_prepare))
     N, K = 256, 512
